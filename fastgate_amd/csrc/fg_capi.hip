@@ -1,0 +1,272 @@
+// C ABI of libfastgate: argument validation, launch planning, dispatch.  Host code only;
+// the kernels live in fg_kernels_*.hip.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstring>
+
+#include "fg_internal.h"
+
+namespace fg {
+namespace {
+
+constexpr int kCUs = 256;              // MI355X compute units
+constexpr int kTargetWaves = 8 * kCUs; // wavefronts wanted in flight for a weight stream
+
+int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+int pick_waves(int items) { return items >= 4 ? 4 : (items >= 2 ? 2 : 1); }
+
+// Work items = groups of `unroll` K units handed round-robin to waves*S slots.  Returns the
+// fraction of slot-steps that carry real work (1.0 = perfectly even).
+double balance(int items, int slots) {
+  const int per = ceil_div(items, slots);
+  return (double)items / ((double)per * slots);
+}
+
+// Cross-workgroup split-K factor.  A split costs a second launch and S*M*N*8 bytes of
+// fp32 partial traffic, so it is only taken when the un-split grid leaves CUs idle.
+int pick_splitk(int tiles, int waves, int items, int M, int N, int K, int wbytes) {
+  static const int cand[] = {1, 2, 3, 4, 6, 8, 12, 16};
+  int best = 1;
+  double best_score = -1.0;
+  for (int S : cand) {
+    if (S > 1 && items / (waves * S) < 2) continue;  // keep >= 2 steps per wave
+    const double fill = std::min(1.0, (double)tiles * S * waves / kTargetWaves);
+    const double cu_fill = std::min(1.0, (double)tiles * S / kCUs);
+    const double extra =
+        S > 1 ? (8.0 * S * M * N) / ((double)wbytes * K * N) : 0.0;  // partials vs weights
+    double score = balance(items, waves * S) * (0.5 * fill + 0.5 * cu_fill) / (1.0 + extra);
+    if (S > 1) score *= 0.92;  // second launch
+    if (score > best_score + 1e-9) {
+      best_score = score;
+      best = S;
+    }
+  }
+  return best;
+}
+
+int validate_shape(int M, int N, int K, int w_layout) {
+  if (M <= 0 || N <= 0 || K <= 0) return FG_ERR_INVALID_ARG;
+  if (w_layout != FG_W_KN && w_layout != FG_W_NK) return FG_ERR_INVALID_ARG;
+  if (N % 128 != 0 || K % 128 != 0) return FG_ERR_ALIGN128;
+  return FG_OK;
+}
+
+// Fills grid/block/workspace from the tile fields; rejects tiles that were not built.
+int finish_plan(int M, int N, int K, fg_plan_t* p) {
+  if (p->splitk < 1 || p->waves < 1 || p->waves > 4 || (p->waves & (p->waves - 1))) {
+    return FG_ERR_INVALID_ARG;
+  }
+  switch (p->kernel) {
+    case FG_KERNEL_NK_DOT2:
+      if (!nk_dot2_supported(p->m_block, p->tile_n, p->unroll)) return FG_ERR_UNSUPPORTED;
+      break;
+    case FG_KERNEL_NK_MFMA:
+      p->m_block = 16;
+      if (!nk_mfma_supported(p->tile_n, p->unroll)) return FG_ERR_UNSUPPORTED;
+      break;
+    case FG_KERNEL_KN_DOT2:
+      p->tile_n = 128;
+      if (!kn_dot2_supported(p->m_block, p->unroll)) return FG_ERR_UNSUPPORTED;
+      break;
+    case FG_KERNEL_KN_MFMA:
+      p->tile_n = 128;
+      p->m_block = 16;
+      if (!kn_mfma_supported(p->unroll)) return FG_ERR_UNSUPPORTED;
+      break;
+    default:
+      return FG_ERR_UNSUPPORTED;
+  }
+  if (N % p->tile_n != 0) return FG_ERR_UNSUPPORTED;
+  if (p->splitk > 65535) return FG_ERR_INVALID_ARG;
+  p->grid_x = N / p->tile_n;
+  p->grid_y = ceil_div(M, p->m_block);
+  p->grid_z = p->splitk;
+  p->block = 64 * p->waves;
+  p->workspace_bytes = p->splitk > 1 ? (size_t)p->splitk * M * N * sizeof(float) : 0;
+  (void)K;
+  return FG_OK;
+}
+
+int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
+  std::memset(p, 0, sizeof(*p));
+  p->stream_w = 1;
+  int items;
+  if (w_layout == FG_W_NK) {
+    if (M <= 7) {
+      p->kernel = FG_KERNEL_NK_DOT2;
+      p->m_block = M <= 1 ? 1 : (M <= 2 ? 2 : (M <= 4 ? 4 : 8));
+      const int rn_max = std::min(16, 64 / p->m_block);
+      p->tile_n = 4;
+      for (int rn = rn_max; rn >= 4; rn >>= 1) {
+        if (N / rn >= 2 * kCUs) {
+          p->tile_n = rn;
+          break;
+        }
+      }
+      const int nq = K / 8;
+      p->unroll = std::max(1, std::min(std::min(4, 16 / p->tile_n), nq / 64));
+      items = ceil_div(nq, 64 * p->unroll);
+    } else {
+      p->kernel = FG_KERNEL_NK_MFMA;
+      p->m_block = 16;
+      p->tile_n = (N / 32 >= 2 * kCUs) ? 32 : 16;
+      p->unroll = p->tile_n == 32 ? 4 : 8;
+      if (K / 32 < 4 * p->unroll) p->unroll = 4;
+      items = ceil_div(K / 32, p->unroll);
+    }
+  } else {
+    if (M <= 7) {
+      p->kernel = FG_KERNEL_KN_DOT2;
+      p->m_block = M <= 1 ? 1 : (M <= 2 ? 2 : (M <= 4 ? 4 : 8));
+    } else {
+      p->kernel = FG_KERNEL_KN_MFMA;
+      p->m_block = 16;
+    }
+    p->tile_n = 128;
+    p->unroll = (K / 32 >= 64) ? 2 : 1;
+    items = ceil_div(K / 32, p->unroll);
+  }
+  p->waves = pick_waves(items);
+  const int tiles = (N / p->tile_n) * ceil_div(M, p->m_block);
+  p->splitk = splitk > 0 ? splitk : pick_splitk(tiles, p->waves, items, M, N, K, 2);
+  return finish_plan(M, N, K, p);
+}
+
+int check_launch() {
+  return hipGetLastError() == hipSuccess ? FG_OK : FG_ERR_LAUNCH;
+}
+
+int run_gemm(const void* A, const void* W, void* C, int M, int N, int K, int accumulate,
+             const fg_plan_t& p, void* ws, size_t ws_bytes, hipStream_t s) {
+  if (p.splitk > 1 && (ws == nullptr || ws_bytes < p.workspace_bytes)) return FG_ERR_WORKSPACE;
+  if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(W) |
+       reinterpret_cast<uintptr_t>(C) | reinterpret_cast<uintptr_t>(ws)) & 15) {
+    return FG_ERR_INVALID_ARG;  // 16-byte loads and stores
+  }
+  GemmArgs a{A, W, C, static_cast<float*>(ws), M, N, K, accumulate ? 1 : 0};
+  (void)hipGetLastError();
+  bool ok = false;
+  switch (p.kernel) {
+    case FG_KERNEL_NK_DOT2: ok = launch_nk_dot2(p, a, s); break;
+    case FG_KERNEL_NK_MFMA: ok = launch_nk_mfma(p, a, s); break;
+    case FG_KERNEL_KN_DOT2: ok = launch_kn_dot2(p, a, s); break;
+    case FG_KERNEL_KN_MFMA: ok = launch_kn_mfma(p, a, s); break;
+    default: break;
+  }
+  if (!ok) return FG_ERR_UNSUPPORTED;
+  if (check_launch() != FG_OK) return FG_ERR_LAUNCH;
+  if (p.splitk > 1) {
+    launch_splitk_reduce(a.ws, C, p.splitk, M, N, a.accumulate, s);
+    if (check_launch() != FG_OK) return FG_ERR_LAUNCH;
+  }
+  return FG_OK;
+}
+
+}  // namespace
+}  // namespace fg
+
+extern "C" {
+
+int fg_version(void) { return FG_VERSION; }
+
+const char* fg_strerror(int status) {
+  switch (status) {
+    case FG_OK: return "ok";
+    case FG_ERR_INVALID_ARG: return "invalid argument (null or misaligned pointer, bad size or enum)";
+    case FG_ERR_ALIGN128: return "K and N must be multiples of 128";
+    case FG_ERR_WORKSPACE: return "split-K workspace missing or too small";
+    case FG_ERR_LAUNCH: return "HIP kernel launch failed";
+    case FG_ERR_UNSUPPORTED: return "plan names a kernel/tile combination that is not built";
+    default: return "unknown fastgate status";
+  }
+}
+
+int fg_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* out) {
+  if (out == nullptr || splitk < 0) return FG_ERR_INVALID_ARG;
+  const int st = fg::validate_shape(M, N, K, w_layout);
+  if (st != FG_OK) return st;
+  return fg::make_plan(M, N, K, w_layout, splitk, out);
+}
+
+size_t fg_workspace_bytes(int M, int N, int K, int w_layout, int splitk) {
+  fg_plan_t p;
+  if (fg_plan(M, N, K, w_layout, splitk, &p) != FG_OK) return 0;
+  return p.workspace_bytes;
+}
+
+int fg_gemm_f16(const void* A, const void* W, void* C, int M, int N, int K, int w_layout,
+                int accumulate, int splitk, void* ws, size_t ws_bytes, void* stream) {
+  if (A == nullptr || W == nullptr || C == nullptr) return FG_ERR_INVALID_ARG;
+  fg_plan_t p;
+  const int st = fg_plan(M, N, K, w_layout, splitk, &p);
+  if (st != FG_OK) return st;
+  return fg::run_gemm(A, W, C, M, N, K, accumulate, p, ws, ws_bytes,
+                      static_cast<hipStream_t>(stream));
+}
+
+int fg_gemm_f16_planned(const void* A, const void* W, void* C, int M, int N, int K, int w_layout,
+                        int accumulate, fg_plan_t* plan, void* ws, size_t ws_bytes, void* stream) {
+  if (A == nullptr || W == nullptr || C == nullptr || plan == nullptr) return FG_ERR_INVALID_ARG;
+  int st = fg::validate_shape(M, N, K, w_layout);
+  if (st != FG_OK) return st;
+  const bool nk = plan->kernel == FG_KERNEL_NK_DOT2 || plan->kernel == FG_KERNEL_NK_MFMA;
+  const bool kn = plan->kernel == FG_KERNEL_KN_DOT2 || plan->kernel == FG_KERNEL_KN_MFMA;
+  if ((w_layout == FG_W_NK && !nk) || (w_layout == FG_W_KN && !kn)) return FG_ERR_UNSUPPORTED;
+  st = fg::finish_plan(M, N, K, plan);
+  if (st != FG_OK) return st;
+  return fg::run_gemm(A, W, C, M, N, K, accumulate, *plan, ws, ws_bytes,
+                      static_cast<hipStream_t>(stream));
+}
+
+int fg_gemv_w8a16(const void* Wq, const void* x, const void* scale, float scalar_scale,
+                  float zero_point, void* y, int M, int N, int K, void* stream) {
+  if (Wq == nullptr || x == nullptr || y == nullptr) return FG_ERR_INVALID_ARG;
+  if (M <= 0 || M > 8 || N <= 0 || K <= 0) return FG_ERR_INVALID_ARG;
+  if (N % 128 != 0 || K % 128 != 0) return FG_ERR_ALIGN128;
+  if ((reinterpret_cast<uintptr_t>(Wq) | reinterpret_cast<uintptr_t>(x)) & 15) {
+    return FG_ERR_INVALID_ARG;
+  }
+  fg::W8A16Args a{Wq, x, scale, scalar_scale, zero_point, y, M, N, K};
+  (void)hipGetLastError();
+  if (!fg::launch_w8a16(a, static_cast<hipStream_t>(stream))) return FG_ERR_UNSUPPORTED;
+  return fg::check_launch();
+}
+
+int fg_gemv_i8i8_i32(const void* Wq, const void* xq, int32_t* acc, int M, int N, int K,
+                     void* stream) {
+  if (Wq == nullptr || xq == nullptr || acc == nullptr) return FG_ERR_INVALID_ARG;
+  if (M <= 0 || M > 8 || N <= 0 || K <= 0) return FG_ERR_INVALID_ARG;
+  if (N % 128 != 0 || K % 128 != 0) return FG_ERR_ALIGN128;
+  if ((reinterpret_cast<uintptr_t>(Wq) | reinterpret_cast<uintptr_t>(xq)) & 15) {
+    return FG_ERR_INVALID_ARG;
+  }
+  (void)hipGetLastError();
+  if (!fg::launch_i8i8_i32(Wq, xq, acc, M, N, K, static_cast<hipStream_t>(stream))) {
+    return FG_ERR_UNSUPPORTED;
+  }
+  return fg::check_launch();
+}
+
+int fg_dequant_i32_f16(const int32_t* acc, const void* scale, float x_scale, void* y, int M, int N,
+                       void* stream) {
+  if (acc == nullptr || y == nullptr || M <= 0 || N <= 0) return FG_ERR_INVALID_ARG;
+  (void)hipGetLastError();
+  fg::launch_dequant_i32_f16(acc, scale, x_scale, y, M, N, static_cast<hipStream_t>(stream));
+  return fg::check_launch();
+}
+
+size_t fg_stream_read_sink_bytes(void) { return (size_t)fg::kStreamReadBlocks * sizeof(uint32_t); }
+
+int fg_stream_read(const void* src, size_t bytes, void* sink, void* stream) {
+  if (src == nullptr || sink == nullptr || bytes == 0 || (bytes & 15) ||
+      (reinterpret_cast<uintptr_t>(src) & 15)) {
+    return FG_ERR_INVALID_ARG;
+  }
+  (void)hipGetLastError();
+  fg::launch_stream_read(src, bytes, sink, static_cast<hipStream_t>(stream));
+  return fg::check_launch();
+}
+
+}  // extern "C"

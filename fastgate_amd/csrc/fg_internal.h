@@ -1,0 +1,55 @@
+// Host-side contract between the C ABI (fg_capi.hip) and the kernel translation units.
+// Each kernel file exports one launcher that maps a validated plan onto a template
+// instantiation; the launchers return false when the plan names a combination that was not
+// instantiated.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "../../include/fastgate.h"
+
+namespace fg {
+
+struct GemmArgs {
+  const void* A;  // fp16 [M,K]
+  const void* W;  // fp16 [N,K] or [K,N]
+  void* C;        // fp16 [M,N]
+  float* ws;      // fp32 [S,M,N] partials when plan.splitk > 1
+  int M, N, K;
+  int accumulate;
+};
+
+// Tile sets that exist as instantiations (the planner and the validators share these).
+bool nk_dot2_supported(int m_block, int tile_n, int unroll);
+bool nk_mfma_supported(int tile_n, int unroll);
+bool kn_dot2_supported(int m_block, int unroll);
+bool kn_mfma_supported(int unroll);
+
+bool launch_nk_dot2(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
+bool launch_nk_mfma(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
+bool launch_kn_dot2(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
+bool launch_kn_mfma(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
+
+// Second pass of split-K: C[m,n] = fp16( Σ_s ws[s,m,n] (+ C[m,n]) ), fixed summation order.
+void launch_splitk_reduce(const float* ws, void* C, int S, int M, int N, int accumulate,
+                          hipStream_t s);
+
+struct W8A16Args {
+  const void* Wq;     // int8 [N,K]
+  const void* x;      // fp16 [M,K]
+  const void* scale;  // fp16 [N] or null
+  float scalar_scale, zero_point;
+  void* y;  // fp16 [M,N]
+  int M, N, K;
+};
+bool launch_w8a16(const W8A16Args& a, hipStream_t s);
+bool launch_i8i8_i32(const void* Wq, const void* xq, int32_t* acc, int M, int N, int K,
+                     hipStream_t s);
+void launch_dequant_i32_f16(const int32_t* acc, const void* scale, float x_scale, void* y, int M,
+                            int N, hipStream_t s);
+
+constexpr int kStreamReadBlocks = 2048;
+void launch_stream_read(const void* src, size_t bytes, void* sink, hipStream_t s);
+
+}  // namespace fg

@@ -1,0 +1,273 @@
+// fp16 kernels for weights stored [K,N] (row k holds the weights of every output column).
+//
+// A 16-byte load of a [K,N] matrix yields 8 neighbouring columns at one k, while both
+// v_dot2_f32_f16 and the MFMA B operand want neighbouring k for one column.  Each lane
+// therefore owns an 8(k) x 8(n) block per step: 8 loads from 8 consecutive rows, then 32
+// v_perm_b32 transpose it in registers into 8 columns x 4 registers of k-pairs.  No LDS is
+// used for the weights.  Lane l = (j = l%16, g = l/16): columns n0+8j..+7 (16 lanes cover
+// 256 contiguous bytes of a row), rows 32*unit+8g..+7.  Workgroup tile = 128 columns;
+// waves (and gridDim.z workgroups) interleave over K and meet in LDS / the workspace.
+//
+// Replaces the device side of eed_hgemm_m8n128k64x4_v7 / _v8 (backend/cuda/hk/edgemm.cuh:
+// 1669-1868, 1873-2049), eed_hgemm_m8n256k32x8 (:2241-2414) and the flat_gemm kernels
+// (backend/cuda/hk/flatgemm.cuh:18-915) of the reference.
+#include "fg_device.h"
+#include "fg_internal.h"
+
+namespace fg {
+
+constexpr uint32_t kSelLo = 0x05040100u;  // (lo16 of S1, lo16 of S0)
+constexpr uint32_t kSelHi = 0x07060302u;  // (hi16 of S1, hi16 of S0)
+
+// rows[i] = 8 columns of row k0+i  ->  bt[c] = 8 consecutive k of column c (4 k-pairs).
+__device__ __forceinline__ void transpose8x8(const u32x4 (&rows)[8], u32x4 (&bt)[8]) {
+#pragma unroll
+  for (int p = 0; p < 4; ++p) {
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const uint32_t even = rows[2 * p][c], odd = rows[2 * p + 1][c];
+      bt[2 * c][p] = __builtin_amdgcn_perm(odd, even, kSelLo);
+      bt[2 * c + 1][p] = __builtin_amdgcn_perm(odd, even, kSelHi);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// MFMA variant: 8 MFMAs per step, MFMA i owns the columns n0 + 8*jj + i (jj = B-operand
+// column index), so acc[i][r] = D[m = 4g + r][n = n0 + 8j + i]: a lane ends up with 8
+// consecutive columns per row, which makes the epilogue 16-byte stores.
+// ---------------------------------------------------------------------------------------
+template <int U, bool STREAM>
+__global__ __launch_bounds__(256) void kn_mfma_kernel(const half_t* __restrict__ A,
+                                                      const half_t* __restrict__ W,
+                                                      half_t* __restrict__ C,
+                                                      float* __restrict__ ws, int M, int N, int K,
+                                                      int accumulate) {
+  __shared__ float red[4][16][128];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int nw = blockDim.x >> 6;
+  const int j = lane & 15, g = lane >> 4;
+  const int n0 = blockIdx.x * 128;
+  const int m0 = blockIdx.y * 16;
+  const int slots = nw * gridDim.z;
+  const int slot = blockIdx.z * nw + wave;
+  const int nunits = K >> 5;
+
+  float4_t acc[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) acc[i] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+  const bool arow = (m0 + j) < M;
+  const half_t* Ap = A + (size_t)(m0 + (arow ? j : 0)) * K + g * 8;
+  const half_t* Wp = W + (size_t)(g * 8) * N + n0 + j * 8;
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+
+  for (int u0 = slot * U; u0 < nunits; u0 += slots * U) {
+    u32x4 rows[U][8];
+    u32x4 a[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int unit = u0 + u;
+      const bool ok = unit < nunits;
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        rows[u][i] = ok ? load16<STREAM>(Wp + (size_t)(unit * 32 + i) * N) : zero;
+      a[u] = (ok && arow) ? load16<false>(Ap + (size_t)unit * 32) : zero;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      u32x4 bt[8];
+      transpose8x8(rows[u], bt);
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(a[u]), as_half8(bt[i]), acc[i], 0,
+                                                        0, 0);
+    }
+  }
+
+#pragma unroll
+  for (int r = 0; r < 4; ++r)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) red[wave][4 * g + r][8 * j + i] = acc[i][r];
+  __syncthreads();
+  // 16 x 128 outputs, 8 consecutive columns per thread.
+  for (int e = threadIdx.x; e < 256; e += blockDim.x) {
+    const int m = e >> 4, c0 = (e & 15) * 8;
+    const int mg = m0 + m;
+    if (mg < M) {
+      float sum[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) sum[i] = 0.f;
+      for (int w = 0; w < nw; ++w)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) sum[i] += red[w][m][c0 + i];
+      if (gridDim.z == 1) {
+        half_t* c = C + (size_t)mg * N + n0 + c0;
+        half8_t out;
+        if (accumulate) {
+          const half8_t old = *reinterpret_cast<const half8_t*>(c);
+#pragma unroll
+          for (int i = 0; i < 8; ++i) sum[i] += static_cast<float>(old[i]);
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) out[i] = static_cast<half_t>(sum[i]);
+        *reinterpret_cast<half8_t*>(c) = out;
+      } else {
+        float* o = ws + ((size_t)blockIdx.z * M + mg) * N + n0 + c0;
+        *reinterpret_cast<float4_t*>(o) = float4_t{sum[0], sum[1], sum[2], sum[3]};
+        *reinterpret_cast<float4_t*>(o + 4) = float4_t{sum[4], sum[5], sum[6], sum[7]};
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// v_dot2 variant for few rows of A: acc[i][m] per lane, the activations of the lane's 8 k
+// positions are one 16-byte load per row m (identical for the 16 lanes of a DPP row).
+// The four k-groups g of a wave are summed in LDS together with the waves.
+// ---------------------------------------------------------------------------------------
+template <int MB, int U, bool STREAM>
+__global__ __launch_bounds__(256) void kn_dot2_kernel(const half_t* __restrict__ A,
+                                                      const half_t* __restrict__ W,
+                                                      half_t* __restrict__ C,
+                                                      float* __restrict__ ws, int M, int N, int K,
+                                                      int accumulate) {
+  __shared__ float red[16][MB][128];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int nw = blockDim.x >> 6;
+  const int j = lane & 15, g = lane >> 4;
+  const int n0 = blockIdx.x * 128;
+  const int m0 = blockIdx.y * MB;
+  const int slots = nw * gridDim.z;
+  const int slot = blockIdx.z * nw + wave;
+  const int nunits = K >> 5;
+
+  float acc[8][MB];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int m = 0; m < MB; ++m) acc[i][m] = 0.f;
+
+  const half_t* Ap = A + (size_t)m0 * K + g * 8;
+  const half_t* Wp = W + (size_t)(g * 8) * N + n0 + j * 8;
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+
+  for (int u0 = slot * U; u0 < nunits; u0 += slots * U) {
+    u32x4 rows[U][8];
+    u32x4 xr[U][MB];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int unit = u0 + u;
+      const bool ok = unit < nunits;
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        rows[u][i] = ok ? load16<STREAM>(Wp + (size_t)(unit * 32 + i) * N) : zero;
+#pragma unroll
+      for (int m = 0; m < MB; ++m)
+        xr[u][m] =
+            (ok && (m0 + m) < M) ? load16<false>(Ap + (size_t)m * K + (size_t)unit * 32) : zero;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      u32x4 bt[8];
+      transpose8x8(rows[u], bt);
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int m = 0; m < MB; ++m) acc[i][m] = dot8(bt[i], xr[u][m], acc[i][m]);
+    }
+  }
+
+#pragma unroll
+  for (int m = 0; m < MB; ++m)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) red[wave * 4 + g][m][8 * j + i] = acc[i][m];
+  __syncthreads();
+  for (int e = threadIdx.x; e < MB * 128; e += blockDim.x) {
+    const int m = e >> 7, nn = e & 127;
+    float sum = 0.f;
+    for (int p = 0; p < nw * 4; ++p) sum += red[p][m][nn];
+    const int mg = m0 + m, n = n0 + nn;
+    if (mg < M) {
+      if (gridDim.z == 1) {
+        half_t* c = C + (size_t)mg * N + n;
+        if (accumulate) sum += static_cast<float>(*c);
+        *c = static_cast<half_t>(sum);
+      } else {
+        ws[((size_t)blockIdx.z * M + mg) * N + n] = sum;
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Host launchers
+// ---------------------------------------------------------------------------------------
+bool kn_dot2_supported(int mb, int u) {
+  return (mb == 1 || mb == 2 || mb == 4 || mb == 8) && (u == 1 || u == 2 || u == 4) &&
+         !(mb == 8 && u == 4);
+}
+bool kn_mfma_supported(int u) { return u == 1 || u == 2 || u == 4; }
+
+template <int MB, int U>
+static void kn_dot2_go(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
+  const dim3 grid(p.grid_x, p.grid_y, p.grid_z), block(p.block);
+  auto* A = static_cast<const half_t*>(a.A);
+  auto* W = static_cast<const half_t*>(a.W);
+  auto* C = static_cast<half_t*>(a.C);
+  if (p.stream_w)
+    hipLaunchKernelGGL((kn_dot2_kernel<MB, U, true>), grid, block, 0, s, A, W, C, a.ws, a.M, a.N,
+                       a.K, a.accumulate);
+  else
+    hipLaunchKernelGGL((kn_dot2_kernel<MB, U, false>), grid, block, 0, s, A, W, C, a.ws, a.M, a.N,
+                       a.K, a.accumulate);
+}
+
+template <int MB>
+static bool kn_dot2_u(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
+  switch (p.unroll) {
+    case 1: kn_dot2_go<MB, 1>(p, a, s); return true;
+    case 2: kn_dot2_go<MB, 2>(p, a, s); return true;
+    case 4:
+      if constexpr (MB < 8) { kn_dot2_go<MB, 4>(p, a, s); return true; }
+      return false;
+    default: return false;
+  }
+}
+
+bool launch_kn_dot2(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
+  switch (p.m_block) {
+    case 1: return kn_dot2_u<1>(p, a, s);
+    case 2: return kn_dot2_u<2>(p, a, s);
+    case 4: return kn_dot2_u<4>(p, a, s);
+    case 8: return kn_dot2_u<8>(p, a, s);
+    default: return false;
+  }
+}
+
+template <int U>
+static void kn_mfma_go(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
+  const dim3 grid(p.grid_x, p.grid_y, p.grid_z), block(p.block);
+  auto* A = static_cast<const half_t*>(a.A);
+  auto* W = static_cast<const half_t*>(a.W);
+  auto* C = static_cast<half_t*>(a.C);
+  if (p.stream_w)
+    hipLaunchKernelGGL((kn_mfma_kernel<U, true>), grid, block, 0, s, A, W, C, a.ws, a.M, a.N, a.K,
+                       a.accumulate);
+  else
+    hipLaunchKernelGGL((kn_mfma_kernel<U, false>), grid, block, 0, s, A, W, C, a.ws, a.M, a.N, a.K,
+                       a.accumulate);
+}
+
+bool launch_kn_mfma(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
+  switch (p.unroll) {
+    case 1: kn_mfma_go<1>(p, a, s); return true;
+    case 2: kn_mfma_go<2>(p, a, s); return true;
+    case 4: kn_mfma_go<4>(p, a, s); return true;
+    default: return false;
+  }
+}
+
+}  // namespace fg

@@ -1,0 +1,270 @@
+// fp16 kernels for weights stored [N,K] (each output column's weights contiguous along K).
+//
+// Both kernels stream W exactly once with 16-byte loads and keep the M x K activation
+// panel out of the way: every wave re-reads only the slice of A that matches the K
+// positions it owns (an L2 hit, 1/tile_n of the weight traffic) straight into registers,
+// so the main loop has no LDS traffic and no barrier.  The wavefronts of a workgroup (and,
+// with split-K, of gridDim.z workgroups) interleave over K; their partial sums meet in LDS.
+//
+// Replaces the device side of gemv_fp16 / gemm_fp16 (backend/cuda/hk/fastgemv.cuh:503-561,
+// 244-311), eed_hgemm_m8n128k64x4_v7_bt (hk/edgemm.cuh:1467-1667) and
+// gemm_m8n128k64x4_v8_tr (hk/edgemm_tr.cuh:371-549) of the reference.
+#include "fg_device.h"
+#include "fg_internal.h"
+
+namespace fg {
+
+// ---------------------------------------------------------------------------------------
+// v_dot2 kernel.  Workgroup = blockDim.x/64 waves, tile = RN columns of C x MB rows of A.
+// Lane l of wave slot s owns the 16-byte chunks q = (step*slots + s)*64*U + u*64 + l of
+// every row of its tile: 1 KB contiguous per row and load instruction.
+// ---------------------------------------------------------------------------------------
+template <int MB, int RN, int U, bool STREAM>
+__global__ __launch_bounds__(256) void nk_dot2_kernel(const half_t* __restrict__ A,
+                                                      const half_t* __restrict__ W,
+                                                      half_t* __restrict__ C,
+                                                      float* __restrict__ ws, int M, int N, int K,
+                                                      int accumulate) {
+  __shared__ float red[16][RN * MB];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int nw = blockDim.x >> 6;
+  const int n0 = blockIdx.x * RN;
+  const int m0 = blockIdx.y * MB;
+  const int slots = nw * gridDim.z;
+  const int slot = blockIdx.z * nw + wave;
+  const int nq = K >> 3;
+
+  float acc[RN][MB];
+#pragma unroll
+  for (int r = 0; r < RN; ++r)
+#pragma unroll
+    for (int m = 0; m < MB; ++m) acc[r][m] = 0.f;
+
+  const half_t* Wt = W + (size_t)n0 * K;
+  const half_t* At = A + (size_t)m0 * K;
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+
+  for (int q0 = slot * (64 * U); q0 < nq; q0 += slots * (64 * U)) {
+    u32x4 wr[U][RN];
+    u32x4 xr[U][MB];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int q = q0 + u * 64 + lane;
+      const bool ok = q < nq;
+#pragma unroll
+      for (int r = 0; r < RN; ++r)
+        wr[u][r] = ok ? load16<STREAM>(Wt + (size_t)r * K + (size_t)q * 8) : zero;
+#pragma unroll
+      for (int m = 0; m < MB; ++m)
+        xr[u][m] = (ok && (m0 + m) < M) ? load16<false>(At + (size_t)m * K + (size_t)q * 8) : zero;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int r = 0; r < RN; ++r)
+#pragma unroll
+        for (int m = 0; m < MB; ++m) acc[r][m] = dot8(wr[u][r], xr[u][m], acc[r][m]);
+  }
+
+  // 64 lanes -> 4 row sums per wave (DPP), then waves x 4 partials through LDS.
+#pragma unroll
+  for (int r = 0; r < RN; ++r)
+#pragma unroll
+    for (int m = 0; m < MB; ++m) {
+      const float v = row16_allreduce(acc[r][m]);
+      if ((lane & 15) == 0) red[wave * 4 + (lane >> 4)][r * MB + m] = v;
+    }
+  __syncthreads();
+  for (int t = threadIdx.x; t < RN * MB; t += blockDim.x) {
+    const int m = t / RN, r = t % RN;
+    float sum = 0.f;
+    for (int p = 0; p < nw * 4; ++p) sum += red[p][r * MB + m];
+    const int mg = m0 + m, n = n0 + r;
+    if (mg < M) {
+      if (gridDim.z == 1) {
+        half_t* c = C + (size_t)mg * N + n;
+        if (accumulate) sum += static_cast<float>(*c);
+        *c = static_cast<half_t>(sum);
+      } else {
+        ws[((size_t)blockIdx.z * M + mg) * N + n] = sum;
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// MFMA kernel.  Workgroup tile = 16*TNW columns of C x 16 rows of A.  A 16-byte weight load
+// of lane l (j = l%16, g = l/16) lands directly in the B-operand layout of
+// v_mfma_f32_16x16x32_f16: column n0+16t+j, k = 32*unit + 8g .. +7; the matching A operand is
+// row m0+j at the same k.  One MFMA consumes one load instruction of the wave.
+// ---------------------------------------------------------------------------------------
+template <int TNW, int U, bool STREAM>
+__global__ __launch_bounds__(256) void nk_mfma_kernel(const half_t* __restrict__ A,
+                                                      const half_t* __restrict__ W,
+                                                      half_t* __restrict__ C,
+                                                      float* __restrict__ ws, int M, int N, int K,
+                                                      int accumulate) {
+  __shared__ float red[4][TNW][256];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int nw = blockDim.x >> 6;
+  const int j = lane & 15, g = lane >> 4;
+  const int n0 = blockIdx.x * (16 * TNW);
+  const int m0 = blockIdx.y * 16;
+  const int slots = nw * gridDim.z;
+  const int slot = blockIdx.z * nw + wave;
+  const int nunits = K >> 5;
+
+  float4_t acc[TNW];
+#pragma unroll
+  for (int t = 0; t < TNW; ++t) acc[t] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+  const bool arow = (m0 + j) < M;
+  const half_t* Ap = A + (size_t)(m0 + (arow ? j : 0)) * K + g * 8;
+  const half_t* Wp = W + (size_t)(n0 + j) * K + g * 8;
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+
+  for (int u0 = slot * U; u0 < nunits; u0 += slots * U) {
+    u32x4 b[U][TNW];
+    u32x4 a[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int unit = u0 + u;
+      const bool ok = unit < nunits;
+#pragma unroll
+      for (int t = 0; t < TNW; ++t)
+        b[u][t] = ok ? load16<STREAM>(Wp + (size_t)t * 16 * K + (size_t)unit * 32) : zero;
+      a[u] = (ok && arow) ? load16<false>(Ap + (size_t)unit * 32) : zero;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int t = 0; t < TNW; ++t)
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(a[u]), as_half8(b[u][t]), acc[t],
+                                                        0, 0, 0);
+  }
+
+  // acc[t][r] = D[m = 4g + r][n = j]
+#pragma unroll
+  for (int t = 0; t < TNW; ++t)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) red[wave][t][(4 * g + r) * 16 + j] = acc[t][r];
+  __syncthreads();
+  for (int e = threadIdx.x; e < TNW * 256; e += blockDim.x) {
+    const int t = e >> 8, m = (e >> 4) & 15, nn = e & 15;
+    float sum = 0.f;
+    for (int w = 0; w < nw; ++w) sum += red[w][t][m * 16 + nn];
+    const int mg = m0 + m, n = n0 + t * 16 + nn;
+    if (mg < M) {
+      if (gridDim.z == 1) {
+        half_t* c = C + (size_t)mg * N + n;
+        if (accumulate) sum += static_cast<float>(*c);
+        *c = static_cast<half_t>(sum);
+      } else {
+        ws[((size_t)blockIdx.z * M + mg) * N + n] = sum;
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Host launchers
+// ---------------------------------------------------------------------------------------
+bool nk_dot2_supported(int mb, int rn, int u) {
+  const bool mb_ok = mb == 1 || mb == 2 || mb == 4 || mb == 8;
+  const bool rn_ok = rn == 4 || rn == 8 || rn == 16;
+  const bool u_ok = u == 1 || u == 2 || u == 4;
+  return mb_ok && rn_ok && u_ok && mb * rn <= 64 && rn * u <= 32;
+}
+
+bool nk_mfma_supported(int tile_n, int u) {
+  return (tile_n == 16 || tile_n == 32) && (u == 1 || u == 2 || u == 4 || u == 8);
+}
+
+template <int MB, int RN, int U>
+static void nk_dot2_go(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
+  const dim3 grid(p.grid_x, p.grid_y, p.grid_z), block(p.block);
+  auto* A = static_cast<const half_t*>(a.A);
+  auto* W = static_cast<const half_t*>(a.W);
+  auto* C = static_cast<half_t*>(a.C);
+  if (p.stream_w)
+    hipLaunchKernelGGL((nk_dot2_kernel<MB, RN, U, true>), grid, block, 0, s, A, W, C, a.ws, a.M,
+                       a.N, a.K, a.accumulate);
+  else
+    hipLaunchKernelGGL((nk_dot2_kernel<MB, RN, U, false>), grid, block, 0, s, A, W, C, a.ws, a.M,
+                       a.N, a.K, a.accumulate);
+}
+
+template <int MB, int RN>
+static bool nk_dot2_u(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
+  if constexpr (MB * RN <= 64) {
+    switch (p.unroll) {
+      case 1: nk_dot2_go<MB, RN, 1>(p, a, s); return true;
+      case 2:
+        if constexpr (RN * 2 <= 32) { nk_dot2_go<MB, RN, 2>(p, a, s); return true; }
+        return false;
+      case 4:
+        if constexpr (RN * 4 <= 32) { nk_dot2_go<MB, RN, 4>(p, a, s); return true; }
+        return false;
+      default: return false;
+    }
+  } else {
+    return false;
+  }
+}
+
+template <int MB>
+static bool nk_dot2_rn(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
+  switch (p.tile_n) {
+    case 4: return nk_dot2_u<MB, 4>(p, a, s);
+    case 8: return nk_dot2_u<MB, 8>(p, a, s);
+    case 16: return nk_dot2_u<MB, 16>(p, a, s);
+    default: return false;
+  }
+}
+
+bool launch_nk_dot2(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
+  switch (p.m_block) {
+    case 1: return nk_dot2_rn<1>(p, a, s);
+    case 2: return nk_dot2_rn<2>(p, a, s);
+    case 4: return nk_dot2_rn<4>(p, a, s);
+    case 8: return nk_dot2_rn<8>(p, a, s);
+    default: return false;
+  }
+}
+
+template <int TNW, int U>
+static void nk_mfma_go(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
+  const dim3 grid(p.grid_x, p.grid_y, p.grid_z), block(p.block);
+  auto* A = static_cast<const half_t*>(a.A);
+  auto* W = static_cast<const half_t*>(a.W);
+  auto* C = static_cast<half_t*>(a.C);
+  if (p.stream_w)
+    hipLaunchKernelGGL((nk_mfma_kernel<TNW, U, true>), grid, block, 0, s, A, W, C, a.ws, a.M, a.N,
+                       a.K, a.accumulate);
+  else
+    hipLaunchKernelGGL((nk_mfma_kernel<TNW, U, false>), grid, block, 0, s, A, W, C, a.ws, a.M, a.N,
+                       a.K, a.accumulate);
+}
+
+template <int TNW>
+static bool nk_mfma_u(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
+  switch (p.unroll) {
+    case 1: nk_mfma_go<TNW, 1>(p, a, s); return true;
+    case 2: nk_mfma_go<TNW, 2>(p, a, s); return true;
+    case 4: nk_mfma_go<TNW, 4>(p, a, s); return true;
+    case 8: nk_mfma_go<TNW, 8>(p, a, s); return true;
+    default: return false;
+  }
+}
+
+bool launch_nk_mfma(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
+  switch (p.tile_n) {
+    case 16: return nk_mfma_u<1>(p, a, s);
+    case 32: return nk_mfma_u<2>(p, a, s);
+    default: return false;
+  }
+}
+
+}  // namespace fg

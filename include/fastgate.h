@@ -1,0 +1,152 @@
+/*
+ * libfastgate — C ABI of the MI355X (gfx950) small-batch GEMM / GEMV library.
+ *
+ * Every entry point takes plain device pointers and sizes, enqueues its kernels on the
+ * HIP stream it is given (a hipStream_t passed as void*; NULL = the null stream), returns
+ * 0 or a negative fg_status, never throws and never allocates device memory.  The library
+ * keeps no state.  There is no CPU path: without a HIP device every compute call fails
+ * with FG_ERR_LAUNCH.
+ *
+ * The reference (chanzhennan/Fastgate, paths relative to its root) exposes this path as
+ * C++ host functions `void f(at::Tensor A, at::Tensor B, at::Tensor C[, int bz])`; each
+ * declaration below cites the host functions it services.  The pybind11 module `speedgate`
+ * keeps those names and argument conventions and forwards to these entry points.
+ *
+ * Common conventions
+ *   A      fp16 [M,K] row-major activations (contiguous)
+ *   W      fp16 weights, w_layout FG_W_KN = [K,N] row-major, FG_W_NK = [N,K] row-major
+ *   C      fp16 [M,N] row-major, caller allocated
+ *   K, N   multiples of 128 (the reference's only documented constraint, README.md:6-12)
+ *   M      any positive value; the kernels are meant for M = 1..16
+ *   arithmetic: fp16 products, fp32 accumulation, one rounding to fp16 at the end
+ */
+#ifndef FASTGATE_H_
+#define FASTGATE_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FG_VERSION 100
+
+typedef enum fg_status {
+  FG_OK = 0,
+  FG_ERR_INVALID_ARG = -1, /* null pointer, non-positive size, bad enum value        */
+  FG_ERR_ALIGN128 = -2,    /* K or N not a multiple of 128 (reference: invalid_argument) */
+  FG_ERR_WORKSPACE = -3,   /* split-K requested/needed and workspace missing or small */
+  FG_ERR_LAUNCH = -4,      /* HIP reported an error at launch (no device, bad stream) */
+  FG_ERR_UNSUPPORTED = -5  /* plan names a kernel/tile combination that does not exist */
+} fg_status;
+
+enum { FG_W_KN = 0, FG_W_NK = 1 };
+
+/* Kernel families (fg_plan_t.kernel). */
+enum {
+  FG_KERNEL_AUTO = 0,
+  FG_KERNEL_NK_DOT2 = 1, /* [N,K] weights, lanes along K, v_dot2_f32_f16                */
+  FG_KERNEL_NK_MFMA = 2, /* [N,K] weights, v_mfma_f32_16x16x32_f16, 16 rows of A a block */
+  FG_KERNEL_KN_DOT2 = 3, /* [K,N] weights, 8x8 register transpose + v_dot2_f32_f16       */
+  FG_KERNEL_KN_MFMA = 4  /* [K,N] weights, 8x8 register transpose + MFMA                 */
+};
+
+/*
+ * Launch plan for one fg_gemm_f16 call.  fg_plan() fills it with the library's choice;
+ * fg_gemm_f16_planned() accepts a caller-edited copy (the shape sweep uses this to
+ * compare kernels and split-K factors).  Fields a kernel family does not use are ignored.
+ */
+typedef struct fg_plan_t {
+  int kernel;   /* FG_KERNEL_*                                                        */
+  int splitk;   /* S >= 1: K is interleaved over S workgroups per output tile; S > 1
+                   writes fp32 partials [S,M,N] to the workspace and runs the second-pass
+                   reduction kernel (no data atomics)                                */
+  int tile_n;   /* output columns per workgroup                                       */
+  int m_block;  /* rows of A per workgroup (grid.y = ceil(M / m_block))               */
+  int waves;    /* wavefronts per workgroup; they interleave over K, reduced in LDS   */
+  int unroll;   /* independent 16-byte load groups in flight per lane and step        */
+  int stream_w; /* 1 = weight loads carry the non-temporal hint                       */
+  int grid_x, grid_y, grid_z, block; /* filled by fg_plan / fg_gemm_f16_planned       */
+  size_t workspace_bytes;            /* 0 when splitk == 1                            */
+} fg_plan_t;
+
+/*
+ * C = A·W (accumulate = 0) or C += A·W (accumulate = 1; C holds fp16 on entry and the sum
+ * is formed in fp32 before the single rounding).
+ *   splitk  0 = library heuristic, S >= 1 = forced (the reference's trailing `int bz`).
+ *   ws      device scratch of at least fg_workspace_bytes() bytes when the plan's
+ *           splitk > 1, else may be NULL.  Contents need no initialisation.
+ * Services, with w_layout = FG_W_KN: edgemm_m8n128k64x4 (backend/cuda/hk/edgemm.cu:102-156),
+ * edgemm_m8n128k64x4_amd (:159-213), edgemm_m8n256k32x8 (:363-385, accumulate),
+ * flat_gemm_m8n128k64x4_bz1, flat_gemm_m8n256k32x8_bz1, flat_gemm_m8n256k64x8,
+ * flat_gemm_m8n256k32x16, flat_gemm_m8n512k32x16, flat_gemm_m8n64k128x8,
+ * flat_gemm_m8n32k256x8 (backend/cuda/hk/flatgemm.cu:13-169), hgemm (hk/hgemm.cu:29-74);
+ * with w_layout = FG_W_NK: edgemm_m8n128k64x4_bt (hk/edgemm.cu:274-324),
+ * edgemm_m8n128k64x4_tr_amd (:216-270), gemm_m8n128k64x4_bt, gemm_m8n32k128x8_bt,
+ * gemm_m8n64k128x8_bt_exp, gemm_m8n32k256x8_bt, gemm_m8n32k256x8_bt_bz2
+ * (backend/cuda/hk/edgemm_tr.cu:19-139), fastgemv, fastgemv_tuned, fastgemv_extend
+ * (backend/cuda/hk/fastgemv.cu:12-33,63-111), fastgemm (backend/cuda/czn/fastgemm.cu:13-55).
+ */
+int fg_gemm_f16(const void* A, const void* W, void* C, int M, int N, int K, int w_layout,
+                int accumulate, int splitk, void* ws, size_t ws_bytes, void* stream);
+
+/* Same computation with an explicit plan (kernel family, tile, split-K, unroll).  Grid and
+ * workspace fields of *plan are recomputed and written back. */
+int fg_gemm_f16_planned(const void* A, const void* W, void* C, int M, int N, int K,
+                        int w_layout, int accumulate, fg_plan_t* plan, void* ws,
+                        size_t ws_bytes, void* stream);
+
+/* The plan fg_gemm_f16 would use for this shape (splitk as above).  Host only. */
+int fg_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* out);
+
+/* Workspace bytes fg_gemm_f16 needs for this shape and splitk argument (0 when the plan
+ * does not split across workgroups).  Host only. */
+size_t fg_workspace_bytes(int M, int N, int K, int w_layout, int splitk);
+
+/*
+ * W8A16 GEMV: y[m,n] = s_n · ( Σ_k x[m,k]·float(Wq[n,k]) − zero_point·Σ_k x[m,k] ),
+ * s_n = scalar_scale · (scale ? float(scale[n]) : 1).  Wq int8 [N,K] row-major, x fp16
+ * [M,K], scale fp16 [N] or NULL, y fp16 [M,N].  fp32 accumulation, int8→fp16 conversion
+ * is exact.  1 <= M <= 8.
+ * Services fastgemv_int8 (backend/cuda/hk/fastgemv.cu:35-61; kernel formula
+ * hk/fastgemv.cuh:316-389, whose host passes scale = 1, zero_point = 0); the per-channel
+ * scale vector is an extension the reference does not have.
+ */
+int fg_gemv_w8a16(const void* Wq, const void* x, const void* scale, float scalar_scale,
+                  float zero_point, void* y, int M, int N, int K, void* stream);
+
+/*
+ * Integer dot stage: acc[m,n] = Σ_k int32(xq[m,k])·int32(Wq[n,k]) with v_dot4_i32_i8.
+ * Wq int8 [N,K], xq int8 [M,K], acc int32 [M,N].  Exact for K <= 2^17.  1 <= M <= 8.
+ * No counterpart in the reference (its int8 GEMV multiplies fp16 activations); this is the
+ * stage whose result is compared bit for bit.
+ */
+int fg_gemv_i8i8_i32(const void* Wq, const void* xq, int32_t* acc, int M, int N, int K,
+                     void* stream);
+
+/*
+ * Dequantising epilogue of the integer stage: y[m,n] = fp16( float(acc[m,n]) · x_scale ·
+ * (scale ? float(scale[n]) : 1) ).  Together with fg_gemv_i8i8_i32 this is the W8A8 GEMV.
+ */
+int fg_dequant_i32_f16(const int32_t* acc, const void* scale, float x_scale, void* y, int M,
+                       int N, void* stream);
+
+/*
+ * Roofline calibration: read `bytes` (multiple of 16) from src with 16-byte loads and
+ * fold them into one 32-bit word per workgroup at sink (at least fg_stream_read_sink_bytes()
+ * bytes).  Reports the read-only streaming ceiling the GEMV kernels are compared with.
+ */
+int fg_stream_read(const void* src, size_t bytes, void* sink, void* stream);
+size_t fg_stream_read_sink_bytes(void);
+
+/* Human-readable text for a status code; never NULL. */
+const char* fg_strerror(int status);
+
+/* FG_VERSION of the built library. */
+int fg_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FASTGATE_H_ */

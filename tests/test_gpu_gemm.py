@@ -1,0 +1,160 @@
+"""GPU parity of the fp16 GEMM/GEMV kernels against the CPU oracle, through the C ABI
+(ctypes) and through the pybind11 operator surface."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from fastgate_amd import capi
+from helpers import assert_close_f16, capi_gemm, gen, make_plan, normal, uniform_pm1
+
+pytestmark = pytest.mark.gpu
+
+KN, NK = capi.FG_W_KN, capi.FG_W_NK
+
+
+def _case(M, N, K, layout, seed, wstd=0.02):
+    g = gen(seed)
+    A = normal((M, K), g)
+    W = normal((K, N) if layout == KN else (N, K), g, wstd)
+    return A, W
+
+
+def _run(A, W, layout, device, accumulate=False, C0=None, plan=None, splitk=0):
+    M = A.shape[0]
+    N = W.shape[1] if layout == KN else W.shape[0]
+    Ad, Wd = A.to(device), W.to(device)
+    if C0 is None:
+        Cd = torch.full((M, N), float("nan"), dtype=torch.half, device=device)
+    else:
+        Cd = C0.to(device).clone()
+    p = capi_gemm(Ad, Wd, Cd, layout, accumulate=accumulate, splitk=splitk, plan=plan)
+    torch.cuda.synchronize()
+    return Cd.cpu().numpy(), p
+
+
+# Every kernel family x tile x unroll x waves x split-K on one small ragged-ish shape
+# (K = 640 = 5*128 leaves partial steps in every unroll setting).
+def _all_plans():
+    plans = []
+    for mb in (1, 2, 4, 8):
+        for rn in (4, 8, 16):
+            for u in (1, 2, 4):
+                if mb * rn <= 64 and rn * u <= 32:
+                    plans.append(("nk_dot2", NK, dict(kernel=capi.FG_KERNEL_NK_DOT2, tile_n=rn, m_block=mb, unroll=u)))
+    for tn in (16, 32):
+        for u in (1, 2, 4, 8):
+            plans.append(("nk_mfma", NK, dict(kernel=capi.FG_KERNEL_NK_MFMA, tile_n=tn, unroll=u)))
+    for mb in (1, 2, 4, 8):
+        for u in (1, 2, 4):
+            if not (mb == 8 and u == 4):
+                plans.append(("kn_dot2", KN, dict(kernel=capi.FG_KERNEL_KN_DOT2, m_block=mb, unroll=u)))
+    for u in (1, 2, 4):
+        plans.append(("kn_mfma", KN, dict(kernel=capi.FG_KERNEL_KN_MFMA, unroll=u)))
+    return plans
+
+
+@pytest.mark.parametrize("name,layout,kw", _all_plans(), ids=lambda v: str(v) if not isinstance(v, dict) else "-".join("%s%s" % (k[0], v[k]) for k in v if k != "kernel"))
+def test_every_instantiation(device, name, layout, kw):
+    K, N = 640, 384
+    for M in sorted({1, 3, kw.get("m_block", 16), 11}):
+        A, W = _case(M, N, K, layout, 7 + M)
+        ref, _ = oracle.gemm_f16(A.numpy(), W.numpy(), layout)
+        for waves, splitk in ((4, 1), (2, 1), (1, 1), (4, 3), (2, 2)):
+            got, _ = _run(A, W, layout, device, plan=make_plan(waves=waves, splitk=splitk, **kw))
+            assert_close_f16(got, ref, "%s M=%d waves=%d S=%d" % (name, M, waves, splitk))
+
+
+@pytest.mark.parametrize("layout", [KN, NK])
+@pytest.mark.parametrize("M", [1, 2, 3, 4, 5, 7, 8, 9, 15, 16, 17, 33])
+def test_auto_plan_small(device, layout, M):
+    for (N, K) in ((128, 128), (256, 1024), (1024, 384), (1152, 2176)):
+        A, W = _case(M, N, K, layout, 100 * M + N)
+        ref, _ = oracle.gemm_f16(A.numpy(), W.numpy(), layout)
+        got, p = _run(A, W, layout, device)
+        assert_close_f16(got, ref, "auto M=%d N=%d K=%d %s" % (M, N, K, p.as_dict()))
+
+
+@pytest.mark.parametrize("layout", [KN, NK])
+@pytest.mark.parametrize("splitk", [0, 1, 2, 5])
+def test_accumulate_protocol(device, layout, splitk):
+    M, N, K = 8, 512, 1024
+    A, W = _case(M, N, K, layout, 31)
+    C0 = normal((M, N), gen(32), 4.0)
+    ref, _ = oracle.gemm_f16(A.numpy(), W.numpy(), layout, C=C0.numpy(), accumulate=True)
+    got, _ = _run(A, W, layout, device, accumulate=True, C0=C0, splitk=splitk)
+    assert_close_f16(got, ref, "accumulate S=%d" % splitk)
+    # overwrite must ignore what C held (NaN-filled by _run)
+    ref0, _ = oracle.gemm_f16(A.numpy(), W.numpy(), layout)
+    got0, _ = _run(A, W, layout, device, splitk=splitk)
+    assert_close_f16(got0, ref0, "overwrite S=%d" % splitk)
+
+
+def test_closed_forms(device):
+    # ones x ones = K exactly (script/ncu-gemv-test.py:29-30 of the reference)
+    for layout in (KN, NK):
+        for K in (128, 1024, 2048):
+            A = torch.ones((3, K), dtype=torch.half)
+            W = torch.ones((K, 256) if layout == KN else (256, K), dtype=torch.half)
+            got, _ = _run(A, W, layout, device)
+            assert (got == K).all()
+    # unit vector e_k selects row k of W[K,N] bit for bit
+    K, N = 512, 384
+    W = normal((K, N), gen(5), 1.0)
+    for k in (0, 1, 255, 511):
+        A = torch.zeros((2, K), dtype=torch.half)
+        A[0, k] = 1.0
+        A[1, k] = -2.0
+        got, _ = _run(A, W, KN, device)
+        assert (got[0].view(np.uint16) == W[k].numpy().view(np.uint16)).all()
+        assert (got[1] == (-2.0 * W[k].float()).half().numpy()).all()
+        got, _ = _run(A, W.t().contiguous(), NK, device)
+        assert (got[0].view(np.uint16) == W[k].numpy().view(np.uint16)).all()
+
+
+def test_small_integers_exact(device):
+    # |a|,|w| <= 8 and K <= 256: every partial sum is an integer below 2^24, and |y| <= 2048
+    # keeps the fp16 result exact, so any summation order must give the same bits.
+    g = gen(77)
+    for layout in (KN, NK):
+        for M in (1, 4, 8, 16):
+            K, N = 256, 256
+            A = torch.randint(-2, 3, (M, K), generator=g).half()
+            W = torch.randint(-3, 4, (K, N) if layout == KN else (N, K), generator=g).half()
+            ref, raw = oracle.gemm_f16(A.numpy(), W.numpy(), layout)
+            assert np.abs(raw).max() <= 2048
+            got, _ = _run(A, W, layout, device)
+            assert (got == ref).all()
+
+
+def test_row_of_batch_equals_single(device):
+    # row m of an M-row call equals the M = 1 call on that row (script/cublas-gemv.py:30-35)
+    M, N, K = 4, 512, 1024
+    for layout in (KN, NK):
+        A, W = _case(M, N, K, layout, 55)
+        got, _ = _run(A, W, layout, device)
+        for m in range(M):
+            one, _ = _run(A[m:m + 1].contiguous(), W, layout, device)
+            assert_close_f16(one[0], got[m], "row %d" % m)
+
+
+def test_bitwise_reproducible(device):
+    M, N, K = 16, 1024, 4096
+    for layout in (KN, NK):
+        A, W = _case(M, N, K, layout, 91)
+        first, _ = _run(A, W, layout, device)
+        for _ in range(3):
+            again, _ = _run(A, W, layout, device)
+            assert (first.view(np.uint16) == again.view(np.uint16)).all()
+
+
+def test_error_codes_on_device(device):
+    L = capi.lib()
+    A = torch.zeros((8, 256), dtype=torch.half, device=device)
+    W = torch.zeros((256, 256), dtype=torch.half, device=device)
+    C = torch.zeros((8, 256), dtype=torch.half, device=device)
+    from helpers import ptr, stream_ptr
+    assert L.fg_gemm_f16(ptr(A), ptr(W), ptr(C), 8, 200, 256, NK, 0, 0, None, 0, stream_ptr()) == capi.FG_ERR_ALIGN128
+    assert L.fg_gemm_f16(None, ptr(W), ptr(C), 8, 256, 256, NK, 0, 0, None, 0, stream_ptr()) == capi.FG_ERR_INVALID_ARG
+    assert L.fg_gemm_f16(ptr(A), ptr(W), ptr(C), 8, 256, 256, NK, 0, 4, None, 0, stream_ptr()) == capi.FG_ERR_WORKSPACE
+    assert L.fg_gemm_f16(ptr(A), ptr(W), ptr(C), 8, 256, 256, 7, 0, 0, None, 0, stream_ptr()) == capi.FG_ERR_INVALID_ARG
