@@ -1,0 +1,239 @@
+#!/usr/bin/env python3
+"""Benchmark of the small-batch GEMM/GEMV hot path on one MI355X.
+
+Workload (the configuration the headline metric is quoted on): fp16, K = N = 8192,
+M in {1, 8, 16}.  One step = one call of each of the six (M, weight layout) combinations:
+
+    fastgemv(W[N,K], x[1,K], y)                 M = 1,  weights [N,K]
+    edgemm_m8n128k64x4_bt(A, W_t[N,K], C)       M = 8, 16
+    edgemm_m8n128k64x4(A, W[K,N], C)            M = 1, 8, 16, weights [K,N]
+
+through the pybind11 operator surface, on torch's current HIP stream, with all inputs
+resident in HBM.  Every call streams a different one of R weight buffers per layout (10
+buffers, 1.3 GB in total) so that no weight is served from the 256 MB Infinity Cache.
+
+value = algorithmic bytes of a step / time of a step (GB/s).  Algorithmic bytes of one call:
+2*K*N (weights) + 2*M*K (activations) + 2*M*N (result); split-K partials are not counted.
+
+Prints ONE JSON line.  `roofline` describes the kernel that takes the most time in the step,
+timed with HIP events inside the timed region; `cpu_baseline` is the CPU oracle
+(oracle/fg_oracle.c, one thread) on the same step, timed on this host.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+if str(ROOT) not in sys.path:
+    sys.path.insert(0, str(ROOT))
+
+K = N = 8192
+MS = (1, 8, 16)
+R = 5  # weight buffers per layout
+HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E peak
+
+# HBM bytes per launch of the roofline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE,
+# keyed by kernel family and M; see profiles/ for the runs.  None = not measured.
+TRAFFIC_BYTES = {}
+
+
+def algorithmic_bytes(M: int) -> int:
+    return 2 * K * N + 2 * M * K + 2 * M * N
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--cpu-repeats", type=int, default=3, help="repetitions of the step on the CPU oracle (0 = skip)")
+    ap.add_argument("--no-inner-events", action="store_true", help="do not record per-call events inside the timed region")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on exactly one GPU; --gpus %d is not supported "
+              "(the path shards by output columns without any collective, see DESIGN.md)" % args.gpus,
+              file=sys.stderr)
+        return 2
+
+    import numpy as np
+    import torch
+
+    import fastgate_amd
+    from fastgate_amd import capi
+
+    if not torch.cuda.is_available():
+        print("bench.py: no HIP device", file=sys.stderr)
+        return 2
+    sg = fastgate_amd.speedgate  # ImportError if the extension was not built
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    # ---- synthetic inputs, seeded on the CPU so the CPU baseline sees the same bits ----------
+    g = torch.Generator().manual_seed(8192)
+    acts = {M: torch.randn((M, K), generator=g).half() for M in MS}
+    w_nk_host = (torch.randn((N, K), generator=g) * 0.02).half()
+    w_nk = [w_nk_host.to(dev)]
+    w_kn = [w_nk_host.t().contiguous().to(dev)]
+    for r in range(1, R):  # further buffers only have to be distinct memory with the same statistics
+        w_nk.append((torch.randn((N, K), device=dev) * 0.02).half())
+        w_kn.append((torch.randn((K, N), device=dev) * 0.02).half())
+    acts_d = {M: a.to(dev) for M, a in acts.items()}
+    outs = {M: torch.empty((M, N), dtype=torch.half, device=dev) for M in MS}
+    y1 = torch.empty(N, dtype=torch.half, device=dev)
+
+    calls = []  # (label, M, layout, callable(i))
+    calls.append(("fastgemv", 1, capi.FG_W_NK, lambda i: sg.fastgemv(w_nk[i % R], acts_d[1], y1)))
+    for M in (8, 16):
+        calls.append(("edgemm_m8n128k64x4_bt", M, capi.FG_W_NK,
+                      lambda i, M=M: sg.edgemm_m8n128k64x4_bt(acts_d[M], w_nk[i % R], outs[M])))
+    for M in MS:
+        calls.append(("edgemm_m8n128k64x4", M, capi.FG_W_KN,
+                      lambda i, M=M: sg.edgemm_m8n128k64x4(acts_d[M], w_kn[i % R], outs[M])))
+    step_bytes = sum(algorithmic_bytes(M) for _, M, _, _ in calls)
+
+    def barrier():
+        torch.cuda.synchronize()
+
+    # ---- on-box read ceiling (1 GiB, 16-byte loads) ---------------------------------------------
+    L = capi.lib()
+    import ctypes
+    probe = [torch.empty(1 << 30, dtype=torch.uint8, device=dev).random_(0, 256) for _ in range(2)]
+    sink = torch.empty(L.fg_stream_read_sink_bytes(), dtype=torch.uint8, device=dev)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for i in range(3):
+        L.fg_stream_read(ctypes.c_void_p(probe[i % 2].data_ptr()), 1 << 30, ctypes.c_void_p(sink.data_ptr()), stream)
+    barrier()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for i in range(10):
+        L.fg_stream_read(ctypes.c_void_p(probe[i % 2].data_ptr()), 1 << 30, ctypes.c_void_p(sink.data_ptr()), stream)
+    e1.record()
+    barrier()
+    ceiling_gbps = (1 << 30) * 10 / (e0.elapsed_time(e1) * 1e-3) / 1e9
+    del probe
+
+    # ---- warm-up, then exactly `steps` timed steps ------------------------------------------------
+    it = 0
+    for _ in range(args.warmup):
+        for _, _, _, fn in calls:
+            fn(it)
+        it += 1
+    inner = not args.no_inner_events
+    marks = [[torch.cuda.Event(enable_timing=True) for _ in range(len(calls) + 1)] for _ in range(args.steps)] if inner else None
+    ev_a, ev_b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    barrier()
+    t0 = time.perf_counter()
+    ev_a.record()
+    for s in range(args.steps):
+        if inner:
+            marks[s][0].record()
+        for c, (_, _, _, fn) in enumerate(calls):
+            fn(it)
+            if inner:
+                marks[s][c + 1].record()
+        it += 1
+    ev_b.record()
+    barrier()
+    t1 = time.perf_counter()
+    wall_ms = (t1 - t0) * 1e3
+    gpu_ms = ev_a.elapsed_time(ev_b)
+    ms_per_step = wall_ms / args.steps
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+
+    per_call = []
+    for c, (label, M, layout, _) in enumerate(calls):
+        p = capi.plan(M, N, K, layout).as_dict()
+        if inner:
+            us = sum(marks[s][c].elapsed_time(marks[s][c + 1]) for s in range(args.steps)) * 1e3 / args.steps
+        else:
+            us = None
+        entry = {
+            "op": label, "M": M, "w_layout": "[N,K]" if layout == capi.FG_W_NK else "[K,N]",
+            "kernel": p["kernel_name"], "splitk": p["splitk"], "tile_n": p["tile_n"], "waves": p["waves"],
+            "unroll": p["unroll"], "launches": 1 + (p["splitk"] > 1),
+            "bytes": algorithmic_bytes(M),
+        }
+        if us is not None:
+            gbps = algorithmic_bytes(M) / (us * 1e-6) / 1e9
+            entry.update({"us_per_call": round(us, 2), "GBps": round(gbps, 1),
+                          "TFLOPs": round(2.0 * M * N * K / (us * 1e-6) / 1e12, 2),
+                          "frac_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4),
+                          "frac_read_ceiling": round(gbps / ceiling_gbps, 4)})
+        per_call.append(entry)
+
+    roofline = None
+    if inner:
+        dom = max(per_call, key=lambda e: e["us_per_call"])
+        key = "%s_M%d" % (dom["kernel"], dom["M"])
+        roofline = {
+            "bound": "hbm", "achieved": dom["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": round(dom["GBps"] / HBM_PEAK_GBPS, 4), "traffic": TRAFFIC_BYTES.get(key),
+            "kernel": "%s (%s M=%d %s)" % (dom["kernel"], dom["op"], dom["M"], dom["w_layout"]),
+            "launches_in_call": dom["launches"], "us": dom["us_per_call"],
+            "algorithmic_bytes": dom["bytes"], "measured_read_ceiling_GBps": round(ceiling_gbps, 1),
+            "frac_of_read_ceiling": dom["frac_read_ceiling"],
+        }
+
+    # ---- CPU baseline: the oracle on the same step -------------------------------------------------
+    cpu = None
+    if args.cpu_repeats > 0:
+        import oracle
+
+        w_nk_np = w_nk_host.numpy()
+        w_kn_np = np.ascontiguousarray(w_nk_np.T)
+        oracle.gemm_f16(acts[1].numpy()[:, :256], w_nk_np[:128, :256], oracle.W_NK)  # loads the library
+        c0 = time.perf_counter()
+        for _ in range(args.cpu_repeats):
+            for M in MS:
+                oracle.gemm_f16(acts[M].numpy(), w_nk_np, oracle.W_NK)
+                oracle.gemm_f16(acts[M].numpy(), w_kn_np, oracle.W_KN)
+        cpu_s = (time.perf_counter() - c0) / args.cpu_repeats
+        torch.set_num_threads(os.cpu_count() or 1)
+        a32 = {M: acts[M].float() for M in MS}
+        w32 = w_nk_host.float()
+        w32t = w32.t().contiguous()
+        for M in MS:
+            torch.matmul(a32[M], w32.t()), torch.matmul(a32[M], w32t)
+        tt = []
+        for _ in range(5):
+            q0 = time.perf_counter()
+            for M in MS:
+                torch.matmul(a32[M], w32.t())
+                torch.matmul(a32[M], w32t)
+            tt.append(time.perf_counter() - q0)
+        tm = sorted(tt)[len(tt) // 2]
+        cpu = {
+            "value": round(step_bytes / cpu_s / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": "the full step (six calls, K=N=8192, M=1/8/16, both weight layouts) on oracle/fg_oracle.c, "
+                      "%d repetitions, %.1f s per step" % (args.cpu_repeats, cpu_s),
+            "torch_matmul_fp32": {"value": round(step_bytes / tm / 1e9, 2), "unit": "GB/s",
+                                  "cores": torch.get_num_threads(), "s_per_step": round(tm, 4),
+                                  "note": "the reference's own check (torch.matmul, fp32 copies made outside the timed region)"},
+        }
+
+    out = {
+        "metric": "achieved HBM GB/s (% of roofline) and us/call, M=1/8/16, K=N=8192 fp16",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "fp16 K=N=8192, M in {1,8,16}, weights [N,K] (fastgemv, edgemm_m8n128k64x4_bt) and "
+                               "[K,N] (edgemm_m8n128k64x4): six calls per step, %d rotating weight buffers per layout" % R,
+                   "K": K, "N": N, "M": list(MS), "calls_per_step": len(calls), "seed": 8192,
+                   "device": torch.cuda.get_device_name(0)},
+        "roofline": roofline, "cpu_baseline": cpu,
+        "gpu_ms_per_step": round(gpu_ms / args.steps, 4),
+        "frac_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
+        "read_ceiling_GBps": round(ceiling_gbps, 1), "frac_read_ceiling": round(value / ceiling_gbps, 4),
+        "per_call": per_call,
+    }
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

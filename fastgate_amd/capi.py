@@ -28,7 +28,8 @@ FG_KERNEL_NK_DOT2 = 1
 FG_KERNEL_NK_MFMA = 2
 FG_KERNEL_KN_DOT2 = 3
 FG_KERNEL_KN_MFMA = 4
-KERNEL_NAMES = {1: "nk_dot2", 2: "nk_mfma", 3: "kn_dot2", 4: "kn_mfma"}
+FG_KERNEL_NK_MFMA4 = 5
+KERNEL_NAMES = {1: "nk_dot2", 2: "nk_mfma", 3: "kn_dot2", 4: "kn_mfma", 5: "nk_mfma4"}
 
 # Every symbol include/fastgate.h declares.
 EXPORTS = (

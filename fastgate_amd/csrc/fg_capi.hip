@@ -66,6 +66,9 @@ int finish_plan(int M, int N, int K, fg_plan_t* p) {
       p->m_block = 16;
       if (!nk_mfma_supported(p->tile_n, p->unroll)) return FG_ERR_UNSUPPORTED;
       break;
+    case FG_KERNEL_NK_MFMA4:
+      if (!nk_mfma4_supported(p->m_block, p->tile_n, p->unroll)) return FG_ERR_UNSUPPORTED;
+      break;
     case FG_KERNEL_KN_DOT2:
       p->tile_n = 128;
       if (!kn_dot2_supported(p->m_block, p->unroll)) return FG_ERR_UNSUPPORTED;
@@ -151,6 +154,7 @@ int run_gemm(const void* A, const void* W, void* C, int M, int N, int K, int acc
   switch (p.kernel) {
     case FG_KERNEL_NK_DOT2: ok = launch_nk_dot2(p, a, s); break;
     case FG_KERNEL_NK_MFMA: ok = launch_nk_mfma(p, a, s); break;
+    case FG_KERNEL_NK_MFMA4: ok = launch_nk_mfma4(p, a, s); break;
     case FG_KERNEL_KN_DOT2: ok = launch_kn_dot2(p, a, s); break;
     case FG_KERNEL_KN_MFMA: ok = launch_kn_mfma(p, a, s); break;
     default: break;
@@ -211,7 +215,8 @@ int fg_gemm_f16_planned(const void* A, const void* W, void* C, int M, int N, int
   if (A == nullptr || W == nullptr || C == nullptr || plan == nullptr) return FG_ERR_INVALID_ARG;
   int st = fg::validate_shape(M, N, K, w_layout);
   if (st != FG_OK) return st;
-  const bool nk = plan->kernel == FG_KERNEL_NK_DOT2 || plan->kernel == FG_KERNEL_NK_MFMA;
+  const bool nk = plan->kernel == FG_KERNEL_NK_DOT2 || plan->kernel == FG_KERNEL_NK_MFMA ||
+                  plan->kernel == FG_KERNEL_NK_MFMA4;
   const bool kn = plan->kernel == FG_KERNEL_KN_DOT2 || plan->kernel == FG_KERNEL_KN_MFMA;
   if ((w_layout == FG_W_NK && !nk) || (w_layout == FG_W_KN && !kn)) return FG_ERR_UNSUPPORTED;
   st = fg::finish_plan(M, N, K, plan);

@@ -23,11 +23,13 @@ struct GemmArgs {
 // Tile sets that exist as instantiations (the planner and the validators share these).
 bool nk_dot2_supported(int m_block, int tile_n, int unroll);
 bool nk_mfma_supported(int tile_n, int unroll);
+bool nk_mfma4_supported(int m_block, int tile_n, int unroll);
 bool kn_dot2_supported(int m_block, int unroll);
 bool kn_mfma_supported(int unroll);
 
 bool launch_nk_dot2(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
 bool launch_nk_mfma(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
+bool launch_nk_mfma4(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
 bool launch_kn_dot2(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
 bool launch_kn_mfma(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
 

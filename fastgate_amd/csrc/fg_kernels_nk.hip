@@ -45,7 +45,13 @@ __global__ __launch_bounds__(256) void nk_dot2_kernel(const half_t* __restrict__
   const half_t* At = A + (size_t)m0 * K;
   const u32x4 zero = {0u, 0u, 0u, 0u};
 
-  for (int q0 = slot * (64 * U); q0 < nq; q0 += slots * (64 * U)) {
+  // Rows are K*2 bytes apart, a power of two for the usual K, so workgroups that walk K in
+  // lockstep would all sit on the same HBM channels; each workgroup starts at its own step.
+  const int nsteps = (nq + slots * (64 * U) - 1) / (slots * (64 * U));
+  int step = (blockIdx.x + blockIdx.y) % nsteps;
+  for (int it = 0; it < nsteps; ++it) {
+    const int q0 = (step * slots + slot) * (64 * U);
+    step = step + 1 == nsteps ? 0 : step + 1;
     u32x4 wr[U][RN];
     u32x4 xr[U][MB];
 #pragma unroll
@@ -125,7 +131,11 @@ __global__ __launch_bounds__(256) void nk_mfma_kernel(const half_t* __restrict__
   const half_t* Wp = W + (size_t)(n0 + j) * K + g * 8;
   const u32x4 zero = {0u, 0u, 0u, 0u};
 
-  for (int u0 = slot * U; u0 < nunits; u0 += slots * U) {
+  const int nsteps = (nunits + slots * U - 1) / (slots * U);
+  int step = (blockIdx.x + blockIdx.y) % nsteps;  // staggered start, see nk_dot2_kernel
+  for (int it = 0; it < nsteps; ++it) {
+    const int u0 = (step * slots + slot) * U;
+    step = step + 1 == nsteps ? 0 : step + 1;
     u32x4 b[U][TNW];
     u32x4 a[U];
 #pragma unroll
@@ -156,6 +166,110 @@ __global__ __launch_bounds__(256) void nk_mfma_kernel(const half_t* __restrict__
     float sum = 0.f;
     for (int w = 0; w < nw; ++w) sum += red[w][t][m * 16 + nn];
     const int mg = m0 + m, n = n0 + t * 16 + nn;
+    if (mg < M) {
+      if (gridDim.z == 1) {
+        half_t* c = C + (size_t)mg * N + n;
+        if (accumulate) sum += static_cast<float>(*c);
+        *c = static_cast<half_t>(sum);
+      } else {
+        ws[((size_t)blockIdx.z * M + mg) * N + n] = sum;
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// MFMA 4x4x4 kernel.  v_mfma_f32_4x4x4_16B_f16 multiplies 16 independent 4x4x4 blocks; here
+// block b = lane/4 owns the 8 k positions 128*chunk + 8b..8b+7 (two MFMAs of 4 k each) and its
+// four lanes j = lane%4 own four neighbouring weight rows.  One 16-byte load instruction of a
+// wave therefore reads 4 weight rows x 256 contiguous bytes -- the same row-friendly pattern as
+// the v_dot2 kernel with a 4-row tile, instead of the 16 rows x 64 bytes the 16x16x32 operand
+// layout forces -- and one instruction per 4 rows of A replaces 4*4 v_dot2.
+// Workgroup tile = 4*R4 columns of C x 4*MG rows of A; acc[r][g][i] at lane (b,j) is the
+// partial C[m0+4g+i][n0+4r+j] over the k positions of block b, summed over b at the end.
+// ---------------------------------------------------------------------------------------
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ half4_t lo4(u32x4 v) { return __builtin_bit_cast(half4_t, u32x2{v.x, v.y}); }
+__device__ __forceinline__ half4_t hi4(u32x4 v) { return __builtin_bit_cast(half4_t, u32x2{v.z, v.w}); }
+
+template <int MG, int R4, int U, bool STREAM>
+__global__ __launch_bounds__(256) void nk_mfma4_kernel(const half_t* __restrict__ A,
+                                                       const half_t* __restrict__ W,
+                                                       half_t* __restrict__ C,
+                                                       float* __restrict__ ws, int M, int N, int K,
+                                                       int accumulate) {
+  __shared__ float red[16][R4 * MG * 16];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int nw = blockDim.x >> 6;
+  const int j = lane & 3, b = lane >> 2;
+  const int n0 = blockIdx.x * (4 * R4);
+  const int m0 = blockIdx.y * (4 * MG);
+  const int slots = nw * gridDim.z;
+  const int slot = blockIdx.z * nw + wave;
+  const int nchunks = K >> 7;
+
+  float4_t acc[R4][MG];
+#pragma unroll
+  for (int r = 0; r < R4; ++r)
+#pragma unroll
+    for (int g = 0; g < MG; ++g) acc[r][g] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+  const half_t* Wp = W + (size_t)(n0 + j) * K + b * 8;
+  const half_t* Ap = A + (size_t)(m0 + j) * K + b * 8;
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+
+  const int nsteps = (nchunks + slots * U - 1) / (slots * U);
+  int step = (blockIdx.x + blockIdx.y) % nsteps;  // staggered start, see nk_dot2_kernel
+  for (int it = 0; it < nsteps; ++it) {
+    const int c0 = (step * slots + slot) * U;
+    step = step + 1 == nsteps ? 0 : step + 1;
+    u32x4 w[U][R4];
+    u32x4 a[U][MG];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int c = c0 + u;
+      const bool ok = c < nchunks;
+#pragma unroll
+      for (int r = 0; r < R4; ++r)
+        w[u][r] = ok ? load16<STREAM>(Wp + (size_t)(4 * r) * K + (size_t)c * 128) : zero;
+#pragma unroll
+      for (int g = 0; g < MG; ++g)
+        a[u][g] = (ok && (m0 + 4 * g + j) < M)
+                      ? load16<false>(Ap + (size_t)(4 * g) * K + (size_t)c * 128)
+                      : zero;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int r = 0; r < R4; ++r)
+#pragma unroll
+        for (int g = 0; g < MG; ++g) {
+          acc[r][g] = __builtin_amdgcn_mfma_f32_4x4x4f16(lo4(a[u][g]), lo4(w[u][r]), acc[r][g], 0, 0, 0);
+          acc[r][g] = __builtin_amdgcn_mfma_f32_4x4x4f16(hi4(a[u][g]), hi4(w[u][r]), acc[r][g], 0, 0, 0);
+        }
+  }
+
+  // Sum the 16 blocks: 4 per DPP row with row_ror:4 / row_ror:8, the 4 rows and the waves in LDS.
+#pragma unroll
+  for (int r = 0; r < R4; ++r)
+#pragma unroll
+    for (int g = 0; g < MG; ++g)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float v = acc[r][g][i];
+        v += dpp_f32<0x124>(v);
+        v += dpp_f32<0x128>(v);
+        if ((lane & 12) == 0) red[wave * 4 + (lane >> 4)][((r * MG + g) * 4 + i) * 4 + j] = v;
+      }
+  __syncthreads();
+  for (int e = threadIdx.x; e < R4 * MG * 16; e += blockDim.x) {
+    // e = ((g*4 + i) * R4 + r) * 4 + jj : consecutive threads write consecutive columns
+    const int jj = e & 3, r = (e >> 2) % R4, gi = (e >> 2) / R4, g = gi >> 2, i = gi & 3;
+    float sum = 0.f;
+    for (int p = 0; p < nw * 4; ++p) sum += red[p][((r * MG + g) * 4 + i) * 4 + jj];
+    const int mg = m0 + 4 * g + i, n = n0 + 4 * r + jj;
     if (mg < M) {
       if (gridDim.z == 1) {
         half_t* c = C + (size_t)mg * N + n;
@@ -255,6 +369,68 @@ static bool nk_mfma_u(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
     case 2: nk_mfma_go<TNW, 2>(p, a, s); return true;
     case 4: nk_mfma_go<TNW, 4>(p, a, s); return true;
     case 8: nk_mfma_go<TNW, 8>(p, a, s); return true;
+    default: return false;
+  }
+}
+
+bool nk_mfma4_supported(int m_block, int tile_n, int u) {
+  const int mg = m_block / 4, r4 = tile_n / 4;
+  if (m_block % 4 || tile_n % 4) return false;
+  const bool mg_ok = mg >= 1 && mg <= 4;
+  const bool r4_ok = r4 == 1 || r4 == 2 || r4 == 4 || r4 == 8;
+  const bool u_ok = u == 1 || u == 2 || u == 4;
+  return mg_ok && r4_ok && u_ok && mg * r4 <= 16 && (mg + r4) * u <= 24;
+}
+
+template <int MG, int R4, int U>
+static void nk_mfma4_go(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
+  const dim3 grid(p.grid_x, p.grid_y, p.grid_z), block(p.block);
+  auto* A = static_cast<const half_t*>(a.A);
+  auto* W = static_cast<const half_t*>(a.W);
+  auto* C = static_cast<half_t*>(a.C);
+  if (p.stream_w)
+    hipLaunchKernelGGL((nk_mfma4_kernel<MG, R4, U, true>), grid, block, 0, s, A, W, C, a.ws, a.M,
+                       a.N, a.K, a.accumulate);
+  else
+    hipLaunchKernelGGL((nk_mfma4_kernel<MG, R4, U, false>), grid, block, 0, s, A, W, C, a.ws, a.M,
+                       a.N, a.K, a.accumulate);
+}
+
+template <int MG, int R4>
+static bool nk_mfma4_u(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
+  if constexpr (MG * R4 <= 16) {
+    switch (p.unroll) {
+      case 1: nk_mfma4_go<MG, R4, 1>(p, a, s); return true;
+      case 2:
+        if constexpr ((MG + R4) * 2 <= 24) { nk_mfma4_go<MG, R4, 2>(p, a, s); return true; }
+        return false;
+      case 4:
+        if constexpr ((MG + R4) * 4 <= 24) { nk_mfma4_go<MG, R4, 4>(p, a, s); return true; }
+        return false;
+      default: return false;
+    }
+  } else {
+    return false;
+  }
+}
+
+template <int MG>
+static bool nk_mfma4_r(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
+  switch (p.tile_n) {
+    case 4: return nk_mfma4_u<MG, 1>(p, a, s);
+    case 8: return nk_mfma4_u<MG, 2>(p, a, s);
+    case 16: return nk_mfma4_u<MG, 4>(p, a, s);
+    case 32: return nk_mfma4_u<MG, 8>(p, a, s);
+    default: return false;
+  }
+}
+
+bool launch_nk_mfma4(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
+  switch (p.m_block) {
+    case 4: return nk_mfma4_r<1>(p, a, s);
+    case 8: return nk_mfma4_r<2>(p, a, s);
+    case 12: return nk_mfma4_r<3>(p, a, s);
+    case 16: return nk_mfma4_r<4>(p, a, s);
     default: return false;
   }
 }

@@ -49,7 +49,8 @@ enum {
   FG_KERNEL_NK_DOT2 = 1, /* [N,K] weights, lanes along K, v_dot2_f32_f16                */
   FG_KERNEL_NK_MFMA = 2, /* [N,K] weights, v_mfma_f32_16x16x32_f16, 16 rows of A a block */
   FG_KERNEL_KN_DOT2 = 3, /* [K,N] weights, 8x8 register transpose + v_dot2_f32_f16       */
-  FG_KERNEL_KN_MFMA = 4  /* [K,N] weights, 8x8 register transpose + MFMA                 */
+  FG_KERNEL_KN_MFMA = 4, /* [K,N] weights, 8x8 register transpose + MFMA                 */
+  FG_KERNEL_NK_MFMA4 = 5 /* [N,K] weights, v_mfma_f32_4x4x4_16B_f16: 4 rows x 256 B a load */
 };
 
 /*

@@ -45,6 +45,12 @@ def _all_plans():
     for tn in (16, 32):
         for u in (1, 2, 4, 8):
             plans.append(("nk_mfma", NK, dict(kernel=capi.FG_KERNEL_NK_MFMA, tile_n=tn, unroll=u)))
+    for mb in (4, 8, 12, 16):
+        for tn in (4, 8, 16, 32):
+            for u in (1, 2, 4):
+                mg, r4 = mb // 4, tn // 4
+                if mg * r4 <= 16 and (mg + r4) * u <= 24:
+                    plans.append(("nk_mfma4", NK, dict(kernel=capi.FG_KERNEL_NK_MFMA4, tile_n=tn, m_block=mb, unroll=u)))
     for mb in (1, 2, 4, 8):
         for u in (1, 2, 4):
             if not (mb == 8 and u == 4):

@@ -1,0 +1,129 @@
+"""GPU parity of the int8-weight GEMV kernels: the W8A16 path against the fp32 oracle within
+tolerance, the integer stage bit for bit."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from fastgate_amd import capi
+from helpers import assert_close_f16, gen, normal, ptr, stream_ptr
+
+pytestmark = pytest.mark.gpu
+
+
+def _w8a16(Wq, x, scale, scalar_scale, zp, device):
+    L = capi.lib()
+    N, K = Wq.shape
+    M = x.shape[0]
+    y = torch.full((M, N), float("nan"), dtype=torch.half, device=device)
+    Wd, xd = Wq.to(device), x.to(device)
+    sd = None if scale is None else scale.to(device)
+    capi.check(L.fg_gemv_w8a16(ptr(Wd), ptr(xd), ptr(sd), scalar_scale, zp, ptr(y), M, N, K,
+                               stream_ptr()), "fg_gemv_w8a16")
+    torch.cuda.synchronize()
+    return y.cpu().numpy()
+
+
+@pytest.mark.parametrize("M", [1, 2, 3, 4, 5, 8])
+@pytest.mark.parametrize("N,K", [(128, 128), (256, 1152), (1024, 4096), (4096, 1024)])
+def test_w8a16_matches_oracle(device, M, N, K):
+    g = gen(4000 + M + N)
+    x = normal((M, K), g)
+    Wq = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8)
+    scale = (torch.rand(N, generator=g) * 0.009 + 0.001).half()
+    ref, _ = oracle.gemv_w8a16(Wq.numpy(), x.numpy(), scale.numpy(), 1.0, 0.0)
+    assert_close_f16(_w8a16(Wq, x, scale, 1.0, 0.0, device), ref, "per-channel scale")
+    # the reference's effective configuration: scalar scale 1, zero point 0, no vector
+    ref, _ = oracle.gemv_w8a16(Wq.numpy(), (x * 0.01).half().numpy(), None, 1.0, 0.0)
+    assert_close_f16(_w8a16(Wq, (x * 0.01).half(), None, 1.0, 0.0, device), ref, "reference default")
+    # scalar scale and zero point (kernel formula hk/fastgemv.cuh:344-363)
+    ref, _ = oracle.gemv_w8a16(Wq.numpy(), x.numpy(), scale.numpy(), 0.5, 3.0)
+    assert_close_f16(_w8a16(Wq, x, scale, 0.5, 3.0, device), ref, "scale 0.5 zp 3")
+
+
+def test_w8a16_every_int8_value_is_exact(device):
+    # x = e_k picks single weights: the result must be the int8 value itself, all 256 of them.
+    N, K = 256, 128
+    Wq = torch.arange(-128, 128, dtype=torch.int16).to(torch.int8).reshape(N, 1).repeat(1, K).contiguous()
+    for k in (0, 1, 2, 3, 17, 127):
+        x = torch.zeros((1, K), dtype=torch.half)
+        x[0, k] = 1.0
+        got = _w8a16(Wq, x, None, 1.0, 0.0, device)
+        assert (got[0] == np.arange(-128, 128, dtype=np.float16)).all()
+
+
+def test_w8a16_byte_order_within_chunk(device):
+    # weights 1..16 along k against x = e_k: catches a swapped byte / pair mapping
+    N, K = 128, 256
+    Wq = (torch.arange(K) % 16 + 1).to(torch.int8).repeat(N, 1).contiguous()
+    for k in range(0, 48):
+        x = torch.zeros((1, K), dtype=torch.half)
+        x[0, k] = 2.0
+        got = _w8a16(Wq, x, None, 1.0, 0.0, device)
+        assert (got == 2.0 * (k % 16 + 1)).all(), k
+
+
+def _i8i8(Wq, xq, device):
+    L = capi.lib()
+    N, K = Wq.shape
+    M = xq.shape[0]
+    acc = torch.full((M, N), -7, dtype=torch.int32, device=device)
+    Wd, xd = Wq.to(device), xq.to(device)
+    capi.check(L.fg_gemv_i8i8_i32(ptr(Wd), ptr(xd), ptr(acc), M, N, K, stream_ptr()),
+               "fg_gemv_i8i8_i32")
+    torch.cuda.synchronize()
+    return acc.cpu().numpy()
+
+
+@pytest.mark.parametrize("M", [1, 2, 4, 7, 8])
+@pytest.mark.parametrize("N,K", [(128, 128), (384, 2176), (2048, 8192)])
+def test_integer_stage_bit_exact(device, M, N, K):
+    g = gen(5000 + M + K)
+    Wq = torch.randint(-128, 128, (N, K), generator=g, dtype=torch.int8)
+    xq = torch.randint(-128, 128, (M, K), generator=g, dtype=torch.int8)
+    ref = oracle.gemv_i8i8_i32(Wq.numpy(), xq.numpy())
+    assert (ref == (xq.numpy().astype(np.int64) @ Wq.numpy().astype(np.int64).T)).all()
+    got = _i8i8(Wq, xq, device)
+    assert (got == ref).all()
+
+
+def test_integer_stage_extremes(device):
+    # all -128 x -128 at K = 8192: 2^14 * 2^13 = 2^27, the largest magnitude reachable
+    N, K = 128, 8192
+    Wq = torch.full((N, K), -128, dtype=torch.int8)
+    xq = torch.full((1, K), -128, dtype=torch.int8)
+    assert (_i8i8(Wq, xq, device) == 128 * 128 * K).all()
+    xq = torch.full((1, K), 127, dtype=torch.int8)
+    assert (_i8i8(Wq, xq, device) == -128 * 127 * K).all()
+
+
+def test_w8a8_dequant_epilogue(device):
+    L = capi.lib()
+    g = gen(6001)
+    M, N, K = 2, 1024, 2048
+    x = normal((M, K), g)
+    Wq = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8)
+    scale = (torch.rand(N, generator=g) * 0.009 + 0.001).half()
+    s_x = float(x.abs().max()) / 127.0
+    xq = torch.clamp(torch.round(x.float() / s_x), -127, 127).to(torch.int8)
+    acc_ref = oracle.gemv_i8i8_i32(Wq.numpy(), xq.numpy())
+    y_ref = oracle.dequant_i32_f16(acc_ref, scale.numpy(), s_x)
+    acc = torch.from_numpy(_i8i8(Wq, xq, device)).to(device)
+    y = torch.empty((M, N), dtype=torch.half, device=device)
+    sd = scale.to(device)
+    capi.check(L.fg_dequant_i32_f16(ptr(acc), ptr(sd), s_x, ptr(y), M, N, stream_ptr()), "dequant")
+    torch.cuda.synchronize()
+    # same integer input, same two fp32 multiplications: identical bits
+    assert (y.cpu().numpy().view(np.uint16) == y_ref.view(np.uint16)).all()
+
+
+def test_int8_error_codes(device):
+    L = capi.lib()
+    W = torch.zeros((128, 128), dtype=torch.int8, device=device)
+    x = torch.zeros((1, 128), dtype=torch.half, device=device)
+    y = torch.zeros((1, 128), dtype=torch.half, device=device)
+    assert L.fg_gemv_w8a16(ptr(W), ptr(x), None, 1.0, 0.0, ptr(y), 9, 128, 128, stream_ptr()) == capi.FG_ERR_INVALID_ARG
+    assert L.fg_gemv_w8a16(ptr(W), ptr(x), None, 1.0, 0.0, ptr(y), 1, 100, 128, stream_ptr()) == capi.FG_ERR_ALIGN128
+    assert L.fg_gemv_w8a16(None, ptr(x), None, 1.0, 0.0, ptr(y), 1, 128, 128, stream_ptr()) == capi.FG_ERR_INVALID_ARG

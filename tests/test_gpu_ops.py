@@ -1,0 +1,157 @@
+"""The pybind11 operator surface on the GPU: every reference name, with the reference's
+argument order and C protocol, against the oracle's restatement of that operator."""
+import zlib
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from helpers import assert_close_f16, gen, normal, uniform_pm1
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def sg():
+    import fastgate_amd
+
+    return fastgate_amd.speedgate
+
+
+@pytest.mark.parametrize("name", sorted(oracle.GEMM_OPS))
+def test_gemm_operator_semantics(device, sg, name):
+    layout, protocol, has_bz = oracle.GEMM_OPS[name]
+    g = gen(zlib.crc32(name.encode()) % 10000)
+    for M in (1, 8, 16):
+        K, N = 1024, 768
+        A = normal((M, K), g)
+        B = normal((K, N) if layout == oracle.W_KN else (N, K), g, 0.02)
+        C0 = normal((M, N), g, 2.0)  # what the caller left in C
+        for bz in ((2, 8, 0) if has_bz else (None,)):
+            Cd = C0.to(device).clone()
+            args = (A.to(device), B.to(device), Cd) + ((bz,) if has_bz else ())
+            assert getattr(sg, name)(*args) is None
+            torch.cuda.synchronize()
+            ref = oracle.gemm_op(name, A.numpy(), B.numpy(), C0.numpy(), bz=bz)
+            assert_close_f16(Cd.cpu().numpy(), ref, "%s M=%d bz=%s (%s)" % (name, M, bz, protocol))
+
+
+def test_legacy_edgemm_names(device, sg):
+    g = gen(12)
+    A, B = normal((8, 512), g), normal((512, 256), g, 0.02)
+    ref, _ = oracle.gemm_f16(A.numpy(), B.numpy(), oracle.W_KN)
+    for name in ("edgemm", "edgemm_m8n256k64", "edgemm_m8n128k64", "edgemm_m8n128k128"):
+        C = torch.full((8, 256), float("nan"), dtype=torch.half, device=device)
+        getattr(sg, name)(A.to(device), B.to(device), C)
+        assert_close_f16(C.cpu().numpy(), ref, name)
+    C0 = normal((1, 256), g)
+    refa, _ = oracle.gemm_f16(A[:1].numpy(), B.numpy(), oracle.W_KN, C=C0.numpy(), accumulate=True)
+    for name in ("edgemv_m1n128k64x4", "edgemv_m1n256k64x4"):
+        C = C0.to(device).clone()
+        getattr(sg, name)(A[:1].contiguous().to(device), B.to(device), C)
+        assert_close_f16(C.cpu().numpy(), refa, name)
+
+
+def test_fastgemv_weight_first_and_shapes(device, sg):
+    g = gen(1001)
+    N, K = 1024, 2048
+    W = uniform_pm1((N, K), g)
+    x = uniform_pm1((1, K), g)
+    ref = oracle.fastgemv(W.numpy(), x.numpy())
+    Wd = W.to(device)
+    for xs, ys in (((1, K), (N,)), ((K, 1), (N, 1)), ((K,), (1, N))):
+        y = torch.full(ys, float("nan"), dtype=torch.half, device=device)
+        sg.fastgemv(Wd, x.reshape(xs).contiguous().to(device), y)
+        assert_close_f16(y.cpu().numpy().reshape(-1), ref, "fastgemv %s" % (xs,))
+        y.fill_(float("nan"))
+        sg.fastgemv_tuned(Wd, x.reshape(xs).contiguous().to(device), y)
+        assert_close_f16(y.cpu().numpy().reshape(-1), ref, "fastgemv_tuned %s" % (xs,))
+    # ones x ones = K (script/ncu-gemv-test.py:29-30)
+    y = torch.zeros(N, dtype=torch.half, device=device)
+    sg.fastgemv(torch.ones((N, K), dtype=torch.half, device=device),
+                torch.ones((1, K), dtype=torch.half, device=device), y)
+    assert (y.cpu() == K).all()
+
+
+@pytest.mark.parametrize("M", [1, 2, 5, 8])
+def test_fastgemv_extend_and_fastgemm(device, sg, M):
+    g = gen(1100 + M)
+    N, K = 512, 1024
+    W, X = normal((N, K), g, 0.05), normal((M, K), g)
+    ref = oracle.fastgemv_extend(W.numpy(), X.numpy())
+    for fn in (sg.fastgemv_extend, sg.fastgemm):
+        C = torch.full((M, N), float("nan"), dtype=torch.half, device=device)
+        fn(W.to(device), X.to(device), C)
+        assert_close_f16(C.cpu().numpy(), ref, fn.__name__)
+
+
+def test_fastgemv_int8_defaults_and_extension(device, sg):
+    g = gen(1004)
+    N, K = 1024, 2048
+    x = (normal((1, K), g) * 0.05).half()
+    Wq = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8)
+    y = torch.empty(N, dtype=torch.half, device=device)
+    sg.fastgemv_int8(Wq.to(device), x.to(device), y)
+    assert_close_f16(y.cpu().numpy(), oracle.fastgemv_int8(Wq.numpy(), x.numpy()), "defaults")
+    scale = (torch.rand(N, generator=g) * 0.009 + 0.001).half()
+    x1 = normal((1, K), g)
+    sg.fastgemv_int8(Wq.to(device), x1.to(device), y, scale=scale.to(device))
+    ref, _ = oracle.gemv_w8a16(Wq.numpy(), x1.numpy(), scale.numpy())
+    assert_close_f16(y.cpu().numpy(), ref.reshape(-1), "per-channel scale")
+
+
+def test_integer_ops(device, sg):
+    g = gen(1005)
+    N, K = 512, 1024
+    Wq = torch.randint(-128, 128, (N, K), generator=g, dtype=torch.int8)
+    xq = torch.randint(-128, 128, (1, K), generator=g, dtype=torch.int8)
+    acc = torch.empty((1, N), dtype=torch.int32, device=device)
+    sg.gemv_i8i8_i32(Wq.to(device), xq.to(device), acc)
+    assert (acc.cpu().numpy() == oracle.gemv_i8i8_i32(Wq.numpy(), xq.numpy())).all()
+
+
+def test_vendor_comparators(device, sg):
+    g = gen(9)
+    A, B = normal((16, 512), g), normal((512, 256), g, 0.02)
+    ref, _ = oracle.gemm_f16(A.numpy(), B.numpy(), oracle.W_KN)
+    C = torch.empty((16, 256), dtype=torch.half, device=device)
+    sg.hgemm(A.to(device), B.to(device), C)
+    assert_close_f16(C.cpu().numpy(), ref, "hgemm")
+    for fn in (sg.hgemm_tr, sg.mma):
+        C.zero_()
+        fn(A.to(device), B.t().contiguous().to(device), C)
+        assert_close_f16(C.cpu().numpy(), ref, fn.__name__)
+
+
+def test_errors_on_device(device, sg):
+    h = dict(dtype=torch.half, device=device)
+    A, B, C = torch.zeros((8, 256), **h), torch.zeros((256, 384), **h), torch.zeros((8, 384), **h)
+    with pytest.raises(ValueError, match="multiple of 128"):
+        sg.edgemm_m8n128k64x4(torch.zeros((8, 200), **h), torch.zeros((200, 384), **h), C)
+    with pytest.raises(ValueError, match="multiple of 128"):
+        sg.edgemm_m8n128k64x4_bt(A, torch.zeros((100, 256), **h), C)
+    with pytest.raises(RuntimeError, match="inner dimensions"):
+        sg.edgemm_m8n128k64x4(A, torch.zeros((384, 384), **h), C)
+    with pytest.raises(RuntimeError, match="Half"):
+        sg.edgemm_m8n128k64x4(A.float(), B, C)
+    with pytest.raises(RuntimeError, match="contiguous"):
+        sg.edgemm_m8n128k64x4(A, torch.zeros((384, 256), **h).t(), C)
+    with pytest.raises(RuntimeError, match="M\\*N"):
+        sg.edgemm_m8n128k64x4(A, B, torch.zeros((8, 128), **h))
+    with pytest.raises(RuntimeError, match="HIP device"):
+        sg.edgemm_m8n128k64x4(A.cpu(), B, C)
+
+
+def test_runs_on_the_current_stream(device, sg):
+    g = gen(3)
+    A, B = normal((8, 1024), g).to(device), normal((1024, 1024), g, 0.02).to(device)
+    ref, _ = oracle.gemm_f16(A.cpu().numpy(), B.cpu().numpy(), oracle.W_KN)
+    s = torch.cuda.Stream()
+    C = torch.zeros((8, 1024), dtype=torch.half, device=device)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(s):
+        for _ in range(3):
+            sg.edgemm_m8n128k64x4(A, B, C)
+    s.synchronize()
+    assert_close_f16(C.cpu().numpy(), ref, "side stream")

@@ -1,0 +1,192 @@
+"""Host-side checks that need no GPU: the C ABI library loads and exports every symbol the
+header declares, the launch planner is self-consistent, the pybind11 surface carries every
+reference name with the reference's error behaviour, and the product never reaches the oracle."""
+import ctypes
+import re
+import subprocess
+from pathlib import Path
+
+import pytest
+
+from fastgate_amd import capi
+
+ROOT = Path(__file__).resolve().parent.parent
+HEADER = ROOT / "include" / "fastgate.h"
+
+KN, NK = capi.FG_W_KN, capi.FG_W_NK
+SWEEP = [(M, n, n) for M in (1, 2, 4, 8, 16) for n in (1024, 4096, 8192, 16384)]
+CONFIGS = [(1, 4096, 4096), (8, 11008, 4096), (16, 12288, 3072), (16, 3072, 12288), (1, 8192, 8192)]
+
+
+def _declared():
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    return sorted(set(re.findall(r"\b(fg_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported():
+    names = _declared()
+    assert names == sorted(capi.EXPORTS)
+    L = ctypes.CDLL(str(capi.LIB_PATH))
+    for n in names:
+        assert getattr(L, n) is not None
+    assert capi.lib().fg_version() == 100
+
+
+def test_header_is_plain_c():
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-fsyntax-only", "-x", "c", str(HEADER)], check=True)
+
+
+def test_strerror_covers_every_status():
+    texts = {capi.strerror(s) for s in (0, -1, -2, -3, -4, -5)}
+    assert len(texts) == 6 and all(texts)
+    assert "unknown" in capi.strerror(-99)
+    assert "128" in capi.strerror(capi.FG_ERR_ALIGN128)
+
+
+@pytest.mark.parametrize("layout", [KN, NK])
+@pytest.mark.parametrize("M,N,K", SWEEP + CONFIGS + [(3, 128, 128), (33, 256, 384), (7, 1152, 2176)])
+def test_plan_is_consistent(layout, M, N, K):
+    p = capi.plan(M, N, K, layout)
+    d = p.as_dict()
+    assert p.kernel in ((capi.FG_KERNEL_KN_DOT2, capi.FG_KERNEL_KN_MFMA) if layout == KN
+                        else (capi.FG_KERNEL_NK_DOT2, capi.FG_KERNEL_NK_MFMA)), d
+    assert N % p.tile_n == 0 and p.grid_x == N // p.tile_n, d
+    assert p.grid_y == -(-M // p.m_block) and p.grid_z == p.splitk >= 1, d
+    assert p.block == 64 * p.waves and p.waves in (1, 2, 4), d
+    assert p.workspace_bytes == (p.splitk * M * N * 4 if p.splitk > 1 else 0), d
+    assert capi.workspace_bytes(M, N, K, layout) == p.workspace_bytes
+    # the MFMA kernels are reserved for M >= 8
+    if M < 8:
+        assert p.kernel in (capi.FG_KERNEL_KN_DOT2, capi.FG_KERNEL_NK_DOT2), d
+    # a forced split is honoured
+    for s in (1, 2, 7):
+        q = capi.plan(M, N, K, layout, s)
+        assert q.splitk == s and q.workspace_bytes == (s * M * N * 4 if s > 1 else 0)
+
+
+def test_plan_fills_the_chip_on_the_metric_shapes():
+    for layout in (KN, NK):
+        for M in (1, 8, 16):
+            p = capi.plan(M, 8192, 8192, layout)
+            assert p.grid_x * p.grid_y * p.grid_z >= 256, p.as_dict()
+
+
+def test_plan_rejects_bad_arguments():
+    L = capi.lib()
+    p = capi.Plan()
+    assert L.fg_plan(8, 200, 256, KN, 0, ctypes.byref(p)) == capi.FG_ERR_ALIGN128
+    assert L.fg_plan(8, 256, 200, NK, 0, ctypes.byref(p)) == capi.FG_ERR_ALIGN128
+    assert L.fg_plan(0, 256, 256, KN, 0, ctypes.byref(p)) == capi.FG_ERR_INVALID_ARG
+    assert L.fg_plan(8, 256, 256, 2, 0, ctypes.byref(p)) == capi.FG_ERR_INVALID_ARG
+    assert L.fg_plan(8, 256, 256, KN, -1, ctypes.byref(p)) == capi.FG_ERR_INVALID_ARG
+    assert L.fg_plan(8, 256, 256, KN, 0, None) == capi.FG_ERR_INVALID_ARG
+    assert L.fg_workspace_bytes(8, 200, 256, KN, 0) == 0
+    with pytest.raises(capi.FastgateError, match="128"):
+        capi.plan(8, 200, 256, KN)
+
+
+def test_compute_entry_points_validate_before_touching_the_device():
+    # argument errors are reported without a device; nothing here launches a kernel
+    L = capi.lib()
+    one = ctypes.c_void_p(16)
+    assert L.fg_gemm_f16(None, one, one, 8, 256, 256, KN, 0, 0, None, 0, None) == capi.FG_ERR_INVALID_ARG
+    assert L.fg_gemm_f16(one, one, one, 8, 256, 100, KN, 0, 0, None, 0, None) == capi.FG_ERR_ALIGN128
+    assert L.fg_gemm_f16(one, one, one, 8, 256, 256, KN, 0, 4, None, 0, None) == capi.FG_ERR_WORKSPACE
+    assert L.fg_gemv_w8a16(one, one, None, 1.0, 0.0, one, 0, 256, 256, None) == capi.FG_ERR_INVALID_ARG
+    assert L.fg_gemv_w8a16(one, one, None, 1.0, 0.0, one, 1, 256, 130, None) == capi.FG_ERR_ALIGN128
+    assert L.fg_gemv_i8i8_i32(one, one, None, 1, 256, 256, None) == capi.FG_ERR_INVALID_ARG
+    assert L.fg_stream_read(one, 24, one, None) == capi.FG_ERR_INVALID_ARG
+    assert L.fg_stream_read_sink_bytes() >= 4
+    bad = capi.Plan()
+    bad.kernel, bad.tile_n, bad.m_block, bad.waves, bad.unroll, bad.splitk = capi.FG_KERNEL_NK_DOT2, 5, 1, 4, 1, 1
+    assert L.fg_gemm_f16_planned(one, one, one, 1, 256, 256, NK, 0, ctypes.byref(bad), None, 0, None) == capi.FG_ERR_UNSUPPORTED
+    bad.tile_n, bad.kernel = 8, capi.FG_KERNEL_KN_MFMA
+    assert L.fg_gemm_f16_planned(one, one, one, 1, 256, 256, NK, 0, ctypes.byref(bad), None, 0, None) == capi.FG_ERR_UNSUPPORTED
+
+
+# ---- pybind11 surface ---------------------------------------------------------------------------
+REFERENCE_NAMES = {
+    # backend/cuda/hk/edgemm.h:4-14
+    "edgemm", "edgemm_m8n256k64", "edgemm_m8n128k64", "edgemm_m8n128k128", "edgemv_m1n128k64x4",
+    "edgemm_m8n128k64x4", "edgemm_m8n128k64x4_bt", "edgemv_m1n256k64x4", "edgemm_m8n128k64x4_amd",
+    "edgemm_m8n256k32x8", "edgemm_m8n128k64x4_tr_amd",
+    # backend/cuda/hk/flatgemm.h:4-10
+    "flat_gemm_m8n128k64x4_bz1", "flat_gemm_m8n256k32x8_bz1", "flat_gemm_m8n256k64x8",
+    "flat_gemm_m8n256k32x16", "flat_gemm_m8n512k32x16", "flat_gemm_m8n64k128x8", "flat_gemm_m8n32k256x8",
+    # backend/cuda/hk/edgemm_tr.h:7-11
+    "gemm_m8n128k64x4_bt", "gemm_m8n32k128x8_bt", "gemm_m8n32k256x8_bt", "gemm_m8n32k256x8_bt_bz2",
+    "gemm_m8n64k128x8_bt_exp",
+    # backend/cuda/hk/fastgemv.h:4-7, backend/pybind.cpp:23-26
+    "fastgemv", "fastgemv_int8", "fastgemv_tuned", "fastgemv_extend", "hgemm", "fastgemm", "mma",
+}
+
+
+@pytest.fixture(scope="module")
+def sg():
+    import fastgate_amd
+
+    return fastgate_amd.speedgate
+
+
+def test_every_reference_name_is_bound(sg):
+    missing = sorted(n for n in REFERENCE_NAMES if not hasattr(sg, n))
+    assert not missing, missing
+
+
+def test_operator_table_matches_the_oracle_table(sg):
+    import oracle
+
+    for name, (layout, protocol, has_bz) in oracle.GEMM_OPS.items():
+        doc = getattr(sg, name).__doc__
+        assert (", bz:" in doc) == has_bz, name
+        assert ("C +=" in doc) == (protocol == "accumulate"), (name, doc)
+        assert ("B_t[N,K]" in doc) == (layout == oracle.W_NK), (name, doc)
+
+
+def test_alignment_error_is_value_error_and_comes_first(sg):
+    import torch
+
+    h = torch.half
+    C = torch.zeros((8, 128), dtype=h)
+    with pytest.raises(ValueError, match="must be multiple of 128"):
+        sg.edgemm_m8n128k64x4(torch.zeros((8, 100), dtype=h), torch.zeros((100, 128), dtype=h), C)
+    with pytest.raises(ValueError, match="transposed output row"):
+        sg.edgemm_m8n128k64x4_bt(torch.zeros((8, 128), dtype=h), torch.zeros((100, 128), dtype=h), C)
+    with pytest.raises(ValueError, match="must be multiple of 128"):
+        sg.flat_gemm_m8n256k64x8(torch.zeros((8, 100), dtype=h), torch.zeros((100, 128), dtype=h), C, 8)
+    with pytest.raises(ValueError, match="must be multiple of 128"):
+        sg.gemm_m8n128k64x4_bt(torch.zeros((8, 128), dtype=h), torch.zeros((64, 128), dtype=h), C)
+    with pytest.raises(ValueError, match="must be multiple of 128"):
+        sg.fastgemv(torch.zeros((128, 64), dtype=h), torch.zeros((1, 64), dtype=h), torch.zeros(128, dtype=h))
+
+
+def test_no_cpu_path(sg):
+    import torch
+
+    h = torch.half
+    A, B, C = torch.zeros((8, 128), dtype=h), torch.zeros((128, 128), dtype=h), torch.zeros((8, 128), dtype=h)
+    for name in ("edgemm_m8n128k64x4", "edgemm_m8n128k64x4_bt", "gemm_m8n128k64x4_bt", "flat_gemm_m8n256k32x16"):
+        with pytest.raises(RuntimeError, match="HIP device"):
+            getattr(sg, name)(A, B, C)
+    with pytest.raises(RuntimeError, match="HIP device"):
+        sg.fastgemv(B, A[:1], torch.zeros(128, dtype=h))
+    with pytest.raises(RuntimeError, match="HIP device"):
+        sg.fastgemv_int8(B.to(torch.int8), A[:1], torch.zeros(128, dtype=h))
+    with pytest.raises(TypeError):
+        sg.flat_gemm_m8n256k64x8(A, B, C)  # bz is a required argument, as in the reference
+
+
+def test_plan_is_reachable_from_python(sg):
+    d = sg.plan(16, 8192, 8192, sg.W_NK)
+    assert d["grid"][0] * d["grid"][2] >= 256 and d["block"] in (64, 128, 256)
+    with pytest.raises(ValueError):
+        sg.plan(16, 100, 8192, sg.W_NK)
+
+
+def test_product_never_touches_the_oracle():
+    pkg = ROOT / "fastgate_amd"
+    offenders = []
+    for path in list(pkg.rglob("*.py")) + list(pkg.rglob("*.hip")) + list(pkg.rglob("*.h")) + list(pkg.rglob("*.cpp")):
+        if re.search(r"\boracle\b", path.read_text()):
+            offenders.append(str(path.relative_to(ROOT)))
+    assert not offenders, offenders
