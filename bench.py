@@ -51,8 +51,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--cpu-repeats", type=int, default=3, help="repetitions of the step on the CPU oracle (0 = skip)")
-    ap.add_argument("--no-inner-events", action="store_true", help="do not record per-call events inside the timed region")
+    ap.add_argument("--cpu-repeats", type=int, default=8, help="repetitions of the step on the CPU oracle (0 = skip)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU; --gpus %d is not supported "
@@ -123,19 +122,13 @@ def main() -> int:
         for _, _, _, fn in calls:
             fn(it)
         it += 1
-    inner = not args.no_inner_events
-    marks = [[torch.cuda.Event(enable_timing=True) for _ in range(len(calls) + 1)] for _ in range(args.steps)] if inner else None
     ev_a, ev_b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     barrier()
     t0 = time.perf_counter()
     ev_a.record()
     for s in range(args.steps):
-        if inner:
-            marks[s][0].record()
-        for c, (_, _, _, fn) in enumerate(calls):
+        for _, _, _, fn in calls:
             fn(it)
-            if inner:
-                marks[s][c + 1].record()
         it += 1
     ev_b.record()
     barrier()
@@ -145,39 +138,44 @@ def main() -> int:
     ms_per_step = wall_ms / args.steps
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
 
+    # ---- per-call kernel time: `steps` back-to-back launches of one call between two HIP events
+    # on the launch stream (an event between every two calls of the step above would add about
+    # 3.5 us of bubble per call and distort `value`) --------------------------------------------------
     per_call = []
-    for c, (label, M, layout, _) in enumerate(calls):
+    for c, (label, M, layout, fn) in enumerate(calls):
         p = capi.plan(M, N, K, layout).as_dict()
-        if inner:
-            us = sum(marks[s][c].elapsed_time(marks[s][c + 1]) for s in range(args.steps)) * 1e3 / args.steps
-        else:
-            us = None
-        entry = {
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        barrier()
+        e0.record()
+        for s in range(args.steps):
+            fn(it + s)
+        e1.record()
+        barrier()
+        it += args.steps
+        us = e0.elapsed_time(e1) * 1e3 / args.steps
+        gbps = algorithmic_bytes(M) / (us * 1e-6) / 1e9
+        per_call.append({
             "op": label, "M": M, "w_layout": "[N,K]" if layout == capi.FG_W_NK else "[K,N]",
             "kernel": p["kernel_name"], "splitk": p["splitk"], "tile_n": p["tile_n"], "waves": p["waves"],
-            "unroll": p["unroll"], "launches": 1 + (p["splitk"] > 1),
-            "bytes": algorithmic_bytes(M),
-        }
-        if us is not None:
-            gbps = algorithmic_bytes(M) / (us * 1e-6) / 1e9
-            entry.update({"us_per_call": round(us, 2), "GBps": round(gbps, 1),
-                          "TFLOPs": round(2.0 * M * N * K / (us * 1e-6) / 1e12, 2),
-                          "frac_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4),
-                          "frac_read_ceiling": round(gbps / ceiling_gbps, 4)})
-        per_call.append(entry)
+            "unroll": p["unroll"], "launches": 1 + (p["splitk"] > 1 and not p["fused"]),
+            "bytes": algorithmic_bytes(M), "us_per_call": round(us, 2), "GBps": round(gbps, 1),
+            "TFLOPs": round(2.0 * M * N * K / (us * 1e-6) / 1e12, 2),
+            "frac_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4),
+            "frac_read_ceiling": round(gbps / ceiling_gbps, 4)})
 
-    roofline = None
-    if inner:
-        dom = max(per_call, key=lambda e: e["us_per_call"])
-        key = "%s_M%d" % (dom["kernel"], dom["M"])
-        roofline = {
-            "bound": "hbm", "achieved": dom["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-            "frac": round(dom["GBps"] / HBM_PEAK_GBPS, 4), "traffic": TRAFFIC_BYTES.get(key),
-            "kernel": "%s (%s M=%d %s)" % (dom["kernel"], dom["op"], dom["M"], dom["w_layout"]),
-            "launches_in_call": dom["launches"], "us": dom["us_per_call"],
-            "algorithmic_bytes": dom["bytes"], "measured_read_ceiling_GBps": round(ceiling_gbps, 1),
-            "frac_of_read_ceiling": dom["frac_read_ceiling"],
-        }
+    # The roofline entry describes the single-launch call that takes the longest: its time between
+    # the events is one kernel's launch-to-launch time, which the rocprofv3 kernel trace must match.
+    single = [e for e in per_call if e["launches"] == 1] or per_call
+    dom = max(single, key=lambda e: e["us_per_call"])
+    roofline = {
+        "bound": "hbm", "achieved": dom["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+        "frac": round(dom["GBps"] / HBM_PEAK_GBPS, 4),
+        "traffic": TRAFFIC_BYTES.get("%s_M%d" % (dom["kernel"], dom["M"])),
+        "kernel": "%s (%s M=%d %s)" % (dom["kernel"], dom["op"], dom["M"], dom["w_layout"]),
+        "launches_in_call": dom["launches"], "us": dom["us_per_call"],
+        "algorithmic_bytes": dom["bytes"], "measured_read_ceiling_GBps": round(ceiling_gbps, 1),
+        "frac_of_read_ceiling": dom["frac_read_ceiling"],
+    }
 
     # ---- CPU baseline: the oracle on the same step -------------------------------------------------
     cpu = None

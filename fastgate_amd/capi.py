@@ -29,7 +29,8 @@ FG_KERNEL_NK_MFMA = 2
 FG_KERNEL_KN_DOT2 = 3
 FG_KERNEL_KN_MFMA = 4
 FG_KERNEL_NK_MFMA4 = 5
-KERNEL_NAMES = {1: "nk_dot2", 2: "nk_mfma", 3: "kn_dot2", 4: "kn_mfma", 5: "nk_mfma4"}
+FG_KERNEL_NK_MFMA4S = 6
+KERNEL_NAMES = {1: "nk_dot2", 2: "nk_mfma", 3: "kn_dot2", 4: "kn_mfma", 5: "nk_mfma4", 6: "nk_mfma4s"}
 
 # Every symbol include/fastgate.h declares.
 EXPORTS = (
@@ -37,6 +38,8 @@ EXPORTS = (
     "fg_gemm_f16_planned",
     "fg_plan",
     "fg_workspace_bytes",
+    "fg_workspace_header_bytes",
+    "fg_workspace_init",
     "fg_gemv_w8a16",
     "fg_gemv_i8i8_i32",
     "fg_dequant_i32_f16",
@@ -53,6 +56,7 @@ class Plan(ctypes.Structure):
     _fields_ = [
         ("kernel", ctypes.c_int),
         ("splitk", ctypes.c_int),
+        ("fused", ctypes.c_int),
         ("tile_n", ctypes.c_int),
         ("m_block", ctypes.c_int),
         ("waves", ctypes.c_int),
@@ -98,6 +102,10 @@ def lib() -> ctypes.CDLL:
         L.fg_plan.argtypes = [ci, ci, ci, ci, ci, pp]
         L.fg_workspace_bytes.restype = sz
         L.fg_workspace_bytes.argtypes = [ci, ci, ci, ci, ci]
+        L.fg_workspace_header_bytes.restype = sz
+        L.fg_workspace_header_bytes.argtypes = []
+        L.fg_workspace_init.restype = ci
+        L.fg_workspace_init.argtypes = [vp, sz, vp]
         L.fg_gemv_w8a16.restype = ci
         L.fg_gemv_w8a16.argtypes = [vp, vp, vp, cf, cf, vp, ci, ci, ci, vp]
         L.fg_gemv_i8i8_i32.restype = ci

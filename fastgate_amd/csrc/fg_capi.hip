@@ -10,8 +10,7 @@
 namespace fg {
 namespace {
 
-constexpr int kCUs = 256;              // MI355X compute units
-constexpr int kTargetWaves = 8 * kCUs; // wavefronts wanted in flight for a weight stream
+constexpr int kCUs = 256;  // MI355X compute units
 
 int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
@@ -24,20 +23,19 @@ double balance(int items, int slots) {
   return (double)items / ((double)per * slots);
 }
 
-// Cross-workgroup split-K factor.  A split costs a second launch and S*M*N*8 bytes of
-// fp32 partial traffic, so it is only taken when the un-split grid leaves CUs idle.
-int pick_splitk(int tiles, int waves, int items, int M, int N, int K, int wbytes) {
+// Cross-workgroup split-K factor for the K-interleaved kernels.  A split costs S*M*N*8 bytes
+// of fp32 partial traffic and the arrival protocol, so it is only taken when the un-split
+// grid leaves CUs idle.
+int pick_splitk(int tiles, int waves, int items, int M, int N, int K, int target_wgs) {
   static const int cand[] = {1, 2, 3, 4, 6, 8, 12, 16};
   int best = 1;
   double best_score = -1.0;
   for (int S : cand) {
     if (S > 1 && items / (waves * S) < 2) continue;  // keep >= 2 steps per wave
-    const double fill = std::min(1.0, (double)tiles * S * waves / kTargetWaves);
-    const double cu_fill = std::min(1.0, (double)tiles * S / kCUs);
-    const double extra =
-        S > 1 ? (8.0 * S * M * N) / ((double)wbytes * K * N) : 0.0;  // partials vs weights
-    double score = balance(items, waves * S) * (0.5 * fill + 0.5 * cu_fill) / (1.0 + extra);
-    if (S > 1) score *= 0.92;  // second launch
+    const double fill = std::min(1.0, (double)tiles * S / target_wgs);
+    const double extra = S > 1 ? (8.0 * S * M * N) / (2.0 * K * N) : 0.0;  // partials vs weights
+    double score = balance(items, waves * S) * fill / (1.0 + extra);
+    if (S > 1) score *= 0.95;
     if (score > best_score + 1e-9) {
       best_score = score;
       best = S;
@@ -69,6 +67,11 @@ int finish_plan(int M, int N, int K, fg_plan_t* p) {
     case FG_KERNEL_NK_MFMA4:
       if (!nk_mfma4_supported(p->m_block, p->tile_n, p->unroll)) return FG_ERR_UNSUPPORTED;
       break;
+    case FG_KERNEL_NK_MFMA4S:
+      if (!nk_mfma4s_supported(p->m_block, p->tile_n, p->unroll)) return FG_ERR_UNSUPPORTED;
+      p->waves = 4;
+      p->splitk = ceil_div(K / 128, p->unroll);  // one workgroup per K slice of unroll*128
+      break;
     case FG_KERNEL_KN_DOT2:
       p->tile_n = 128;
       if (!kn_dot2_supported(p->m_block, p->unroll)) return FG_ERR_UNSUPPORTED;
@@ -87,36 +90,46 @@ int finish_plan(int M, int N, int K, fg_plan_t* p) {
   p->grid_y = ceil_div(M, p->m_block);
   p->grid_z = p->splitk;
   p->block = 64 * p->waves;
-  p->workspace_bytes = p->splitk > 1 ? (size_t)p->splitk * M * N * sizeof(float) : 0;
-  (void)K;
+  if (p->splitk > 1) {
+    if ((long long)p->grid_x * p->grid_y > kWsMaxTiles) p->fused = 0;
+    p->workspace_bytes = kWsHeaderBytes + (size_t)p->splitk * M * N * sizeof(float);
+  } else {
+    p->workspace_bytes = 0;
+  }
   return FG_OK;
 }
 
 int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
   std::memset(p, 0, sizeof(*p));
   p->stream_w = 1;
-  int items;
+  // Completing split-K inside the launch needs agent-scope fences, which write back and
+  // invalidate the per-XCD L2s: measured 8x slower than the second-pass kernel on MI355X
+  // (K = N = 8192, M = 16, S = 8: 205 us against 26 us).  The planner never picks it.
+  p->fused = 0;
+  int items = 1;
+  const bool interleaved = true;  // waves and splits interleave over K
   if (w_layout == FG_W_NK) {
-    if (M <= 7) {
+    // Measured on MI355X at K = N = 8192 (us per call): M=1 dot2 tile 4: 21.6-22.4; M=4 dot2
+    // 24.3 / mfma4 22.1; M=8 dot2 27.8 / mfma4 26.2 / mfma16 29.2; M=16 mfma4 36 / mfma16 31.7.
+    if (M <= 2) {
       p->kernel = FG_KERNEL_NK_DOT2;
-      p->m_block = M <= 1 ? 1 : (M <= 2 ? 2 : (M <= 4 ? 4 : 8));
-      const int rn_max = std::min(16, 64 / p->m_block);
+      p->m_block = M;
       p->tile_n = 4;
-      for (int rn = rn_max; rn >= 4; rn >>= 1) {
-        if (N / rn >= 2 * kCUs) {
-          p->tile_n = rn;
-          break;
-        }
-      }
-      const int nq = K / 8;
-      p->unroll = std::max(1, std::min(std::min(4, 16 / p->tile_n), nq / 64));
-      items = ceil_div(nq, 64 * p->unroll);
+      p->unroll = 1;
+      items = ceil_div(K / 8, 64);
+    } else if (M <= 8) {
+      p->kernel = FG_KERNEL_NK_MFMA4;
+      p->m_block = M <= 4 ? 4 : 8;
+      p->tile_n = 16;
+      while (p->tile_n > 4 && N / p->tile_n < 2 * kCUs) p->tile_n >>= 1;
+      p->unroll = (K / 128 >= 16) ? 2 : 1;
+      items = ceil_div(K / 128, p->unroll);
     } else {
       p->kernel = FG_KERNEL_NK_MFMA;
       p->m_block = 16;
-      p->tile_n = (N / 32 >= 2 * kCUs) ? 32 : 16;
-      p->unroll = p->tile_n == 32 ? 4 : 8;
-      if (K / 32 < 4 * p->unroll) p->unroll = 4;
+      p->tile_n = (N / 32 >= kCUs) ? 32 : 16;
+      p->unroll = p->tile_n == 32 ? 4 : 2;
+      if (K / 32 < 4 * p->unroll) p->unroll = 1;
       items = ceil_div(K / 32, p->unroll);
     }
   } else {
@@ -131,15 +144,15 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
     p->unroll = (K / 32 >= 64) ? 2 : 1;
     items = ceil_div(K / 32, p->unroll);
   }
-  p->waves = pick_waves(items);
-  const int tiles = (N / p->tile_n) * ceil_div(M, p->m_block);
-  p->splitk = splitk > 0 ? splitk : pick_splitk(tiles, p->waves, items, M, N, K, 2);
+  if (interleaved) {
+    p->waves = pick_waves(items);
+    const int tiles = (N / p->tile_n) * ceil_div(M, p->m_block);
+    p->splitk = splitk > 0 ? splitk : pick_splitk(tiles, p->waves, items, M, N, K, kCUs);
+  }
   return finish_plan(M, N, K, p);
 }
 
-int check_launch() {
-  return hipGetLastError() == hipSuccess ? FG_OK : FG_ERR_LAUNCH;
-}
+int check_launch() { return hipGetLastError() == hipSuccess ? FG_OK : FG_ERR_LAUNCH; }
 
 int run_gemm(const void* A, const void* W, void* C, int M, int N, int K, int accumulate,
              const fg_plan_t& p, void* ws, size_t ws_bytes, hipStream_t s) {
@@ -148,25 +161,36 @@ int run_gemm(const void* A, const void* W, void* C, int M, int N, int K, int acc
        reinterpret_cast<uintptr_t>(C) | reinterpret_cast<uintptr_t>(ws)) & 15) {
     return FG_ERR_INVALID_ARG;  // 16-byte loads and stores
   }
-  GemmArgs a{A, W, C, static_cast<float*>(ws), M, N, K, accumulate ? 1 : 0};
+  GemmArgs a{A, W, C, nullptr, nullptr, M, N, K, accumulate ? 1 : 0};
+  if (p.splitk > 1) {
+    a.ws = reinterpret_cast<float*>(static_cast<unsigned char*>(ws) + kWsHeaderBytes);
+    a.counters = p.fused ? static_cast<int*>(ws) : nullptr;
+  }
   (void)hipGetLastError();
   bool ok = false;
   switch (p.kernel) {
     case FG_KERNEL_NK_DOT2: ok = launch_nk_dot2(p, a, s); break;
     case FG_KERNEL_NK_MFMA: ok = launch_nk_mfma(p, a, s); break;
     case FG_KERNEL_NK_MFMA4: ok = launch_nk_mfma4(p, a, s); break;
+    case FG_KERNEL_NK_MFMA4S: ok = launch_nk_mfma4s(p, a, s); break;
     case FG_KERNEL_KN_DOT2: ok = launch_kn_dot2(p, a, s); break;
     case FG_KERNEL_KN_MFMA: ok = launch_kn_mfma(p, a, s); break;
     default: break;
   }
   if (!ok) return FG_ERR_UNSUPPORTED;
   if (check_launch() != FG_OK) return FG_ERR_LAUNCH;
-  if (p.splitk > 1) {
+  if (p.splitk > 1 && !p.fused) {
     launch_splitk_reduce(a.ws, C, p.splitk, M, N, a.accumulate, s);
     if (check_launch() != FG_OK) return FG_ERR_LAUNCH;
   }
   return FG_OK;
 }
+
+bool is_nk(int kernel) {
+  return kernel == FG_KERNEL_NK_DOT2 || kernel == FG_KERNEL_NK_MFMA ||
+         kernel == FG_KERNEL_NK_MFMA4 || kernel == FG_KERNEL_NK_MFMA4S;
+}
+bool is_kn(int kernel) { return kernel == FG_KERNEL_KN_DOT2 || kernel == FG_KERNEL_KN_MFMA; }
 
 }  // namespace
 }  // namespace fg
@@ -200,6 +224,17 @@ size_t fg_workspace_bytes(int M, int N, int K, int w_layout, int splitk) {
   return p.workspace_bytes;
 }
 
+size_t fg_workspace_header_bytes(void) { return fg::kWsHeaderBytes; }
+
+int fg_workspace_init(void* ws, size_t ws_bytes, void* stream) {
+  if (ws == nullptr || ws_bytes < fg::kWsHeaderBytes || (reinterpret_cast<uintptr_t>(ws) & 15)) {
+    return FG_ERR_INVALID_ARG;
+  }
+  (void)hipGetLastError();
+  fg::launch_fill_zero(ws, fg::kWsHeaderBytes, static_cast<hipStream_t>(stream));
+  return fg::check_launch();
+}
+
 int fg_gemm_f16(const void* A, const void* W, void* C, int M, int N, int K, int w_layout,
                 int accumulate, int splitk, void* ws, size_t ws_bytes, void* stream) {
   if (A == nullptr || W == nullptr || C == nullptr) return FG_ERR_INVALID_ARG;
@@ -215,10 +250,10 @@ int fg_gemm_f16_planned(const void* A, const void* W, void* C, int M, int N, int
   if (A == nullptr || W == nullptr || C == nullptr || plan == nullptr) return FG_ERR_INVALID_ARG;
   int st = fg::validate_shape(M, N, K, w_layout);
   if (st != FG_OK) return st;
-  const bool nk = plan->kernel == FG_KERNEL_NK_DOT2 || plan->kernel == FG_KERNEL_NK_MFMA ||
-                  plan->kernel == FG_KERNEL_NK_MFMA4;
-  const bool kn = plan->kernel == FG_KERNEL_KN_DOT2 || plan->kernel == FG_KERNEL_KN_MFMA;
-  if ((w_layout == FG_W_NK && !nk) || (w_layout == FG_W_KN && !kn)) return FG_ERR_UNSUPPORTED;
+  if ((w_layout == FG_W_NK && !fg::is_nk(plan->kernel)) ||
+      (w_layout == FG_W_KN && !fg::is_kn(plan->kernel))) {
+    return FG_ERR_UNSUPPORTED;
+  }
   st = fg::finish_plan(M, N, K, plan);
   if (st != FG_OK) return st;
   return fg::run_gemm(A, W, C, M, N, K, accumulate, *plan, ws, ws_bytes,

@@ -72,4 +72,73 @@ __device__ __forceinline__ float f16_bits_to_f32(uint16_t b) {
   return static_cast<float>(__builtin_bit_cast(half_t, b));
 }
 
+// Orders LDS traffic among the lanes of one wavefront (data handed from lane to lane through
+// a wave-private LDS region).  The LDS unit serves a wave's requests in order; this only keeps
+// the compiler from moving the accesses across the hand-over point.  No s_barrier is issued.
+__device__ __forceinline__ void wave_lds_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// ---------------------------------------------------------------------------------------
+// Split-K completion inside one launch.  Every workgroup of a tile stores its fp32 partial
+// to part[z][m][n], then arrives at the tile's counter; the workgroup that arrives last sums
+// the S partials in ascending z (so the result does not depend on arrival order), writes C
+// and puts the counter back to zero for the next call.  The only atomic is on the counter.
+// ---------------------------------------------------------------------------------------
+__device__ __forceinline__ bool splitk_last_arriver(int* counter, int S) {
+  __shared__ int s_last;
+  __threadfence();  // release: this workgroup's partial stores are visible device-wide
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const int old = atomicAdd(counter, 1);
+    const int last = old == S - 1;
+    if (last) atomicExch(counter, 0);
+    s_last = last;
+  }
+  __syncthreads();
+  const bool last = s_last != 0;
+  if (last) __threadfence();  // acquire: see the other workgroups' partials
+  return last;
+}
+
+// C[m0..m0+mcnt)[n0..n0+ncnt) = fp16( Σ_z part[z] (+ C) ); ncnt and n0 are multiples of 4.
+__device__ __forceinline__ void splitk_reduce_tile(const float* __restrict__ part, half_t* C, int S,
+                                                   int M, int N, int m0, int mcnt, int n0, int ncnt,
+                                                   int accumulate) {
+  typedef half_t half4v __attribute__((ext_vector_type(4)));
+  const int nq = ncnt >> 2;
+  const size_t MN = (size_t)M * N;
+  for (int e = threadIdx.x; e < mcnt * nq; e += blockDim.x) {
+    const int m = m0 + e / nq, n = n0 + (e % nq) * 4;
+    if (m >= M) continue;
+    const size_t off = (size_t)m * N + n;
+    float4_t sum = *reinterpret_cast<const float4_t*>(part + off);
+    for (int z = 1; z < S; ++z) sum += *reinterpret_cast<const float4_t*>(part + (size_t)z * MN + off);
+    half4v* c = reinterpret_cast<half4v*>(C + off);
+    if (accumulate) {
+      const half4v old = *c;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) sum[k] += static_cast<float>(old[k]);
+    }
+    half4v out;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) out[k] = static_cast<half_t>(sum[k]);
+    *c = out;
+  }
+}
+
+// Shared tail of every GEMM kernel: the workgroup has stored its fp32 partial of the tile
+// (m0.., n0..) when gridDim.z > 1; with counters it also completes the split-K sum in place,
+// without counters a second kernel does.
+template <int MROWS, int NCOLS>
+__device__ __forceinline__ void finish_splitk(float* ws, int* counters, half_t* C, int M, int N,
+                                              int m0, int n0, int accumulate) {
+  if (gridDim.z > 1 && counters != nullptr) {
+    if (splitk_last_arriver(counters + blockIdx.y * gridDim.x + blockIdx.x, gridDim.z))
+      splitk_reduce_tile(ws, C, gridDim.z, M, N, m0, MROWS, n0, NCOLS, accumulate);
+  }
+}
+
 }  // namespace fg

@@ -16,6 +16,7 @@ struct GemmArgs {
   const void* W;  // fp16 [N,K] or [K,N]
   void* C;        // fp16 [M,N]
   float* ws;      // fp32 [S,M,N] partials when plan.splitk > 1
+  int* counters;  // per-tile arrival counters (fused split-K) or null (second-pass kernel)
   int M, N, K;
   int accumulate;
 };
@@ -24,12 +25,14 @@ struct GemmArgs {
 bool nk_dot2_supported(int m_block, int tile_n, int unroll);
 bool nk_mfma_supported(int tile_n, int unroll);
 bool nk_mfma4_supported(int m_block, int tile_n, int unroll);
+bool nk_mfma4s_supported(int m_block, int tile_n, int chunks);
 bool kn_dot2_supported(int m_block, int unroll);
 bool kn_mfma_supported(int unroll);
 
 bool launch_nk_dot2(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
 bool launch_nk_mfma(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
 bool launch_nk_mfma4(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
+bool launch_nk_mfma4s(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
 bool launch_kn_dot2(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
 bool launch_kn_mfma(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
 
@@ -50,6 +53,11 @@ bool launch_i8i8_i32(const void* Wq, const void* xq, int32_t* acc, int M, int N,
                      hipStream_t s);
 void launch_dequant_i32_f16(const int32_t* acc, const void* scale, float x_scale, void* y, int M,
                             int N, hipStream_t s);
+
+// Split-K workspace: a header of arrival counters (zero between calls), then the partials.
+constexpr size_t kWsHeaderBytes = 65536;
+constexpr int kWsMaxTiles = (int)(kWsHeaderBytes / sizeof(int));
+void launch_fill_zero(void* p, size_t bytes, hipStream_t s);
 
 constexpr int kStreamReadBlocks = 2048;
 void launch_stream_read(const void* src, size_t bytes, void* sink, hipStream_t s);

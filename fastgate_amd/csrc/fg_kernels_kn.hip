@@ -41,8 +41,8 @@ template <int U, bool STREAM>
 __global__ __launch_bounds__(256) void kn_mfma_kernel(const half_t* __restrict__ A,
                                                       const half_t* __restrict__ W,
                                                       half_t* __restrict__ C,
-                                                      float* __restrict__ ws, int M, int N, int K,
-                                                      int accumulate) {
+                                                      float* __restrict__ ws, int* counters, int M, int N,
+                                                      int K, int accumulate) {
   __shared__ float red[4][16][128];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -120,6 +120,7 @@ __global__ __launch_bounds__(256) void kn_mfma_kernel(const half_t* __restrict__
       }
     }
   }
+  finish_splitk<16, 128>(ws, counters, C, M, N, m0, n0, accumulate);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -131,8 +132,8 @@ template <int MB, int U, bool STREAM>
 __global__ __launch_bounds__(256) void kn_dot2_kernel(const half_t* __restrict__ A,
                                                       const half_t* __restrict__ W,
                                                       half_t* __restrict__ C,
-                                                      float* __restrict__ ws, int M, int N, int K,
-                                                      int accumulate) {
+                                                      float* __restrict__ ws, int* counters, int M, int N,
+                                                      int K, int accumulate) {
   __shared__ float red[16][MB][128];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -200,6 +201,7 @@ __global__ __launch_bounds__(256) void kn_dot2_kernel(const half_t* __restrict__
       }
     }
   }
+  finish_splitk<MB, 128>(ws, counters, C, M, N, m0, n0, accumulate);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -218,10 +220,10 @@ static void kn_dot2_go(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
   auto* W = static_cast<const half_t*>(a.W);
   auto* C = static_cast<half_t*>(a.C);
   if (p.stream_w)
-    hipLaunchKernelGGL((kn_dot2_kernel<MB, U, true>), grid, block, 0, s, A, W, C, a.ws, a.M, a.N,
+    hipLaunchKernelGGL((kn_dot2_kernel<MB, U, true>), grid, block, 0, s, A, W, C, a.ws, a.counters, a.M, a.N,
                        a.K, a.accumulate);
   else
-    hipLaunchKernelGGL((kn_dot2_kernel<MB, U, false>), grid, block, 0, s, A, W, C, a.ws, a.M, a.N,
+    hipLaunchKernelGGL((kn_dot2_kernel<MB, U, false>), grid, block, 0, s, A, W, C, a.ws, a.counters, a.M, a.N,
                        a.K, a.accumulate);
 }
 
@@ -254,10 +256,10 @@ static void kn_mfma_go(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
   auto* W = static_cast<const half_t*>(a.W);
   auto* C = static_cast<half_t*>(a.C);
   if (p.stream_w)
-    hipLaunchKernelGGL((kn_mfma_kernel<U, true>), grid, block, 0, s, A, W, C, a.ws, a.M, a.N, a.K,
+    hipLaunchKernelGGL((kn_mfma_kernel<U, true>), grid, block, 0, s, A, W, C, a.ws, a.counters, a.M, a.N, a.K,
                        a.accumulate);
   else
-    hipLaunchKernelGGL((kn_mfma_kernel<U, false>), grid, block, 0, s, A, W, C, a.ws, a.M, a.N, a.K,
+    hipLaunchKernelGGL((kn_mfma_kernel<U, false>), grid, block, 0, s, A, W, C, a.ws, a.counters, a.M, a.N, a.K,
                        a.accumulate);
 }
 

@@ -1,10 +1,9 @@
 // fp16 kernels for weights stored [N,K] (each output column's weights contiguous along K).
 //
-// Both kernels stream W exactly once with 16-byte loads and keep the M x K activation
-// panel out of the way: every wave re-reads only the slice of A that matches the K
-// positions it owns (an L2 hit, 1/tile_n of the weight traffic) straight into registers,
-// so the main loop has no LDS traffic and no barrier.  The wavefronts of a workgroup (and,
-// with split-K, of gridDim.z workgroups) interleave over K; their partial sums meet in LDS.
+// All kernels stream W exactly once with 16-byte loads.  Rows of W are K*2 bytes apart -- a
+// power of two for the usual K -- so every kernel here is built to keep the set of rows it
+// has in flight small and to start different workgroups at different K positions; otherwise
+// all workgroups sit on the same few HBM channels at the same time.
 //
 // Replaces the device side of gemv_fp16 / gemm_fp16 (backend/cuda/hk/fastgemv.cuh:503-561,
 // 244-311), eed_hgemm_m8n128k64x4_v7_bt (hk/edgemm.cuh:1467-1667) and
@@ -17,14 +16,16 @@ namespace fg {
 // ---------------------------------------------------------------------------------------
 // v_dot2 kernel.  Workgroup = blockDim.x/64 waves, tile = RN columns of C x MB rows of A.
 // Lane l of wave slot s owns the 16-byte chunks q = (step*slots + s)*64*U + u*64 + l of
-// every row of its tile: 1 KB contiguous per row and load instruction.
+// every row of its tile: 1 KB contiguous per row and load instruction.  The matching slice
+// of A is re-read per step (an L2 hit, 1/RN of the weight traffic) straight into registers,
+// so the main loop has no LDS traffic and no barrier.
 // ---------------------------------------------------------------------------------------
 template <int MB, int RN, int U, bool STREAM>
 __global__ __launch_bounds__(256) void nk_dot2_kernel(const half_t* __restrict__ A,
                                                       const half_t* __restrict__ W,
                                                       half_t* __restrict__ C,
-                                                      float* __restrict__ ws, int M, int N, int K,
-                                                      int accumulate) {
+                                                      float* __restrict__ ws, int* counters, int M,
+                                                      int N, int K, int accumulate) {
   __shared__ float red[16][RN * MB];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -45,10 +46,8 @@ __global__ __launch_bounds__(256) void nk_dot2_kernel(const half_t* __restrict__
   const half_t* At = A + (size_t)m0 * K;
   const u32x4 zero = {0u, 0u, 0u, 0u};
 
-  // Rows are K*2 bytes apart, a power of two for the usual K, so workgroups that walk K in
-  // lockstep would all sit on the same HBM channels; each workgroup starts at its own step.
   const int nsteps = (nq + slots * (64 * U) - 1) / (slots * (64 * U));
-  int step = (blockIdx.x + blockIdx.y) % nsteps;
+  int step = (blockIdx.x + blockIdx.y) % nsteps;  // staggered start
   for (int it = 0; it < nsteps; ++it) {
     const int q0 = (step * slots + slot) * (64 * U);
     step = step + 1 == nsteps ? 0 : step + 1;
@@ -97,20 +96,22 @@ __global__ __launch_bounds__(256) void nk_dot2_kernel(const half_t* __restrict__
       }
     }
   }
+  finish_splitk<MB, RN>(ws, counters, C, M, N, m0, n0, accumulate);
 }
 
 // ---------------------------------------------------------------------------------------
-// MFMA kernel.  Workgroup tile = 16*TNW columns of C x 16 rows of A.  A 16-byte weight load
-// of lane l (j = l%16, g = l/16) lands directly in the B-operand layout of
+// MFMA 16x16x32 kernel.  Workgroup tile = 16*TNW columns of C x 16 rows of A.  A 16-byte
+// weight load of lane l (j = l%16, g = l/16) lands directly in the B-operand layout of
 // v_mfma_f32_16x16x32_f16: column n0+16t+j, k = 32*unit + 8g .. +7; the matching A operand is
-// row m0+j at the same k.  One MFMA consumes one load instruction of the wave.
+// row m0+j at the same k.  One MFMA consumes one load instruction of the wave, but that
+// instruction touches 16 rows x 64 bytes.
 // ---------------------------------------------------------------------------------------
 template <int TNW, int U, bool STREAM>
 __global__ __launch_bounds__(256) void nk_mfma_kernel(const half_t* __restrict__ A,
                                                       const half_t* __restrict__ W,
                                                       half_t* __restrict__ C,
-                                                      float* __restrict__ ws, int M, int N, int K,
-                                                      int accumulate) {
+                                                      float* __restrict__ ws, int* counters, int M,
+                                                      int N, int K, int accumulate) {
   __shared__ float red[4][TNW][256];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -132,7 +133,7 @@ __global__ __launch_bounds__(256) void nk_mfma_kernel(const half_t* __restrict__
   const u32x4 zero = {0u, 0u, 0u, 0u};
 
   const int nsteps = (nunits + slots * U - 1) / (slots * U);
-  int step = (blockIdx.x + blockIdx.y) % nsteps;  // staggered start, see nk_dot2_kernel
+  int step = (blockIdx.x + blockIdx.y) % nsteps;  // staggered start
   for (int it = 0; it < nsteps; ++it) {
     const int u0 = (step * slots + slot) * U;
     step = step + 1 == nsteps ? 0 : step + 1;
@@ -176,29 +177,32 @@ __global__ __launch_bounds__(256) void nk_mfma_kernel(const half_t* __restrict__
       }
     }
   }
+  finish_splitk<16, 16 * TNW>(ws, counters, C, M, N, m0, n0, accumulate);
 }
 
 // ---------------------------------------------------------------------------------------
-// MFMA 4x4x4 kernel.  v_mfma_f32_4x4x4_16B_f16 multiplies 16 independent 4x4x4 blocks; here
+// MFMA 4x4x4 kernels.  v_mfma_f32_4x4x4_16B_f16 multiplies 16 independent 4x4x4 blocks; here
 // block b = lane/4 owns the 8 k positions 128*chunk + 8b..8b+7 (two MFMAs of 4 k each) and its
 // four lanes j = lane%4 own four neighbouring weight rows.  One 16-byte load instruction of a
 // wave therefore reads 4 weight rows x 256 contiguous bytes -- the same row-friendly pattern as
 // the v_dot2 kernel with a 4-row tile, instead of the 16 rows x 64 bytes the 16x16x32 operand
 // layout forces -- and one instruction per 4 rows of A replaces 4*4 v_dot2.
-// Workgroup tile = 4*R4 columns of C x 4*MG rows of A; acc[r][g][i] at lane (b,j) is the
-// partial C[m0+4g+i][n0+4r+j] over the k positions of block b, summed over b at the end.
+// acc[g][i] at lane (b,j) is the partial C[m0+4g+i][n+j] over the k positions of block b; the
+// 16 blocks are summed once per output.
 // ---------------------------------------------------------------------------------------
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ half4_t lo4(u32x4 v) { return __builtin_bit_cast(half4_t, u32x2{v.x, v.y}); }
 __device__ __forceinline__ half4_t hi4(u32x4 v) { return __builtin_bit_cast(half4_t, u32x2{v.z, v.w}); }
 
+// Interleaved variant: the waves of a workgroup interleave over K, every wave covers all
+// 4*R4 columns of the tile and re-reads its slice of A from L2.  Best for M <= 8.
 template <int MG, int R4, int U, bool STREAM>
 __global__ __launch_bounds__(256) void nk_mfma4_kernel(const half_t* __restrict__ A,
                                                        const half_t* __restrict__ W,
                                                        half_t* __restrict__ C,
-                                                       float* __restrict__ ws, int M, int N, int K,
-                                                       int accumulate) {
+                                                       float* __restrict__ ws, int* counters, int M,
+                                                       int N, int K, int accumulate) {
   __shared__ float red[16][R4 * MG * 16];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -221,7 +225,7 @@ __global__ __launch_bounds__(256) void nk_mfma4_kernel(const half_t* __restrict_
   const u32x4 zero = {0u, 0u, 0u, 0u};
 
   const int nsteps = (nchunks + slots * U - 1) / (slots * U);
-  int step = (blockIdx.x + blockIdx.y) % nsteps;  // staggered start, see nk_dot2_kernel
+  int step = (blockIdx.x + blockIdx.y) % nsteps;  // staggered start
   for (int it = 0; it < nsteps; ++it) {
     const int c0 = (step * slots + slot) * U;
     step = step + 1 == nsteps ? 0 : step + 1;
@@ -280,11 +284,123 @@ __global__ __launch_bounds__(256) void nk_mfma4_kernel(const half_t* __restrict_
       }
     }
   }
+  finish_splitk<4 * MG, 4 * R4>(ws, counters, C, M, N, m0, n0, accumulate);
+}
+
+// Sliced variant for M = 8..16.  Re-reading A per 4*R4 columns costs as much L1 traffic as the
+// weights themselves once M reaches 16, so here a workgroup owns a K slice of CW*128 positions
+// (blockIdx.z selects it), stages the 4*MG x slice panel of A in LDS once, and its waves split
+// the TN columns of the tile: wave w walks RG = TN/16 groups of 4 rows, each group CW loads of
+// 4 rows x 256 B (4 rows x CW*256 B contiguous), with the next group's loads issued before
+// the current group's MFMAs.  A operands come from LDS (ds_read_b128).  gridDim.z = number of
+// K slices; the slices meet through the split-K workspace.
+template <int MG, int CW, int RG, bool STREAM>
+__global__ __launch_bounds__(256) void nk_mfma4s_kernel(const half_t* __restrict__ A,
+                                                        const half_t* __restrict__ W,
+                                                        half_t* __restrict__ C,
+                                                        float* __restrict__ ws, int* counters, int M,
+                                                        int N, int K, int accumulate) {
+  constexpr int TN = 16 * RG;     // columns per workgroup (4 waves x RG x 4)
+  constexpr int AROWB = CW * 256;  // bytes per LDS row of A
+  // LDS: A panel [4*MG][CW*256 B], then red[4 waves][4 dpp rows][MG*16] floats.  The 16-byte
+  // pieces of A row r are stored at piece ^ ((r&3) << 2): the four rows j a ds_read_b128 touches
+  // then fall on different banks without padding.
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  unsigned char* a_lds = smem;
+  float(*red)[4][MG * 16] = reinterpret_cast<float(*)[4][MG * 16]>(smem + 4 * MG * AROWB);
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int j = lane & 3, b = lane >> 2;
+  const int n0 = blockIdx.x * TN;
+  const int m0 = blockIdx.y * (4 * MG);
+  const int nchunks = K >> 7;
+  const int c_lo = blockIdx.z * CW;  // first 128-wide K chunk of this slice
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+
+  // Stage A[m0 .. m0+4MG)[c_lo*128 .. +CW*128) in LDS, zero where the row or chunk is absent.
+  for (int e = threadIdx.x; e < 4 * MG * CW * 16; e += 256) {
+    const int row = e / (CW * 16), q = e % (CW * 16);  // q: 16-byte piece within the slice row
+    const int chunk = c_lo + (q >> 4);
+    const bool ok = (m0 + row) < M && chunk < nchunks;
+    const u32x4 v =
+        ok ? load16<false>(A + (size_t)(m0 + row) * K + (size_t)c_lo * 128 + q * 8) : zero;
+    *reinterpret_cast<u32x4*>(a_lds + row * AROWB + ((q ^ ((row & 3) << 2)) << 4)) = v;
+  }
+
+  // Weight loads of the first row group are in flight while A lands in LDS.
+  const half_t* Wp = W + (size_t)(n0 + wave * (4 * RG) + j) * K + (size_t)c_lo * 128 + b * 8;
+  u32x4 wcur[CW], wnxt[CW];
+#pragma unroll
+  for (int c = 0; c < CW; ++c)
+    wcur[c] = (c_lo + c) < nchunks ? load16<STREAM>(Wp + (size_t)c * 128) : zero;
+  __syncthreads();
+
+#pragma unroll
+  for (int rg = 0; rg < RG; ++rg) {
+    if (rg + 1 < RG) {
+#pragma unroll
+      for (int c = 0; c < CW; ++c)
+        wnxt[c] = (c_lo + c) < nchunks
+                      ? load16<STREAM>(Wp + (size_t)(4 * (rg + 1)) * K + (size_t)c * 128)
+                      : zero;
+    }
+    float4_t acc[MG];
+#pragma unroll
+    for (int g = 0; g < MG; ++g) acc[g] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int c = 0; c < CW; ++c) {
+#pragma unroll
+      for (int g = 0; g < MG; ++g) {
+        const u32x4 a = *reinterpret_cast<const u32x4*>(a_lds + (4 * g + j) * AROWB +
+                                                        (((c * 16 + b) ^ (j << 2)) << 4));
+        acc[g] = __builtin_amdgcn_mfma_f32_4x4x4f16(lo4(a), lo4(wcur[c]), acc[g], 0, 0, 0);
+        acc[g] = __builtin_amdgcn_mfma_f32_4x4x4f16(hi4(a), hi4(wcur[c]), acc[g], 0, 0, 0);
+      }
+    }
+    // 16 blocks -> one value: row_ror within the DPP row, the 4 rows through wave-private LDS.
+#pragma unroll
+    for (int g = 0; g < MG; ++g)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float v = acc[g][i];
+        v += dpp_f32<0x124>(v);
+        v += dpp_f32<0x128>(v);
+        if ((lane & 12) == 0) red[wave][lane >> 4][(g * 4 + i) * 4 + j] = v;
+      }
+    wave_lds_sync();  // red[wave] is private to this wave: ordering only, no s_barrier
+    if (lane < MG * 16) {
+      const float sum =
+          red[wave][0][lane] + red[wave][1][lane] + red[wave][2][lane] + red[wave][3][lane];
+      const int mg = m0 + (lane >> 2), n = n0 + wave * (4 * RG) + 4 * rg + (lane & 3);
+      if (mg < M) {
+        if (gridDim.z == 1) {
+          half_t* c = C + (size_t)mg * N + n;
+          float out = sum;
+          if (accumulate) out += static_cast<float>(*c);
+          *c = static_cast<half_t>(out);
+        } else {
+          ws[((size_t)blockIdx.z * M + mg) * N + n] = sum;
+        }
+      }
+    }
+    wave_lds_sync();
+    if (rg + 1 < RG) {
+#pragma unroll
+      for (int c = 0; c < CW; ++c) wcur[c] = wnxt[c];
+    }
+  }
+  finish_splitk<4 * MG, TN>(ws, counters, C, M, N, m0, n0, accumulate);
 }
 
 // ---------------------------------------------------------------------------------------
 // Host launchers
 // ---------------------------------------------------------------------------------------
+#define FG_LAUNCH(KERNEL, p, a, s)                                                            \
+  hipLaunchKernelGGL(KERNEL, dim3((p).grid_x, (p).grid_y, (p).grid_z), dim3((p).block), 0, s, \
+                     static_cast<const half_t*>((a).A), static_cast<const half_t*>((a).W),    \
+                     static_cast<half_t*>((a).C), (a).ws, (a).counters, (a).M, (a).N, (a).K,  \
+                     (a).accumulate)
+
 bool nk_dot2_supported(int mb, int rn, int u) {
   const bool mb_ok = mb == 1 || mb == 2 || mb == 4 || mb == 8;
   const bool rn_ok = rn == 4 || rn == 8 || rn == 16;
@@ -298,16 +414,8 @@ bool nk_mfma_supported(int tile_n, int u) {
 
 template <int MB, int RN, int U>
 static void nk_dot2_go(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
-  const dim3 grid(p.grid_x, p.grid_y, p.grid_z), block(p.block);
-  auto* A = static_cast<const half_t*>(a.A);
-  auto* W = static_cast<const half_t*>(a.W);
-  auto* C = static_cast<half_t*>(a.C);
-  if (p.stream_w)
-    hipLaunchKernelGGL((nk_dot2_kernel<MB, RN, U, true>), grid, block, 0, s, A, W, C, a.ws, a.M,
-                       a.N, a.K, a.accumulate);
-  else
-    hipLaunchKernelGGL((nk_dot2_kernel<MB, RN, U, false>), grid, block, 0, s, A, W, C, a.ws, a.M,
-                       a.N, a.K, a.accumulate);
+  if (p.stream_w) FG_LAUNCH((nk_dot2_kernel<MB, RN, U, true>), p, a, s);
+  else FG_LAUNCH((nk_dot2_kernel<MB, RN, U, false>), p, a, s);
 }
 
 template <int MB, int RN>
@@ -350,16 +458,8 @@ bool launch_nk_dot2(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
 
 template <int TNW, int U>
 static void nk_mfma_go(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
-  const dim3 grid(p.grid_x, p.grid_y, p.grid_z), block(p.block);
-  auto* A = static_cast<const half_t*>(a.A);
-  auto* W = static_cast<const half_t*>(a.W);
-  auto* C = static_cast<half_t*>(a.C);
-  if (p.stream_w)
-    hipLaunchKernelGGL((nk_mfma_kernel<TNW, U, true>), grid, block, 0, s, A, W, C, a.ws, a.M, a.N,
-                       a.K, a.accumulate);
-  else
-    hipLaunchKernelGGL((nk_mfma_kernel<TNW, U, false>), grid, block, 0, s, A, W, C, a.ws, a.M, a.N,
-                       a.K, a.accumulate);
+  if (p.stream_w) FG_LAUNCH((nk_mfma_kernel<TNW, U, true>), p, a, s);
+  else FG_LAUNCH((nk_mfma_kernel<TNW, U, false>), p, a, s);
 }
 
 template <int TNW>
@@ -369,6 +469,14 @@ static bool nk_mfma_u(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
     case 2: nk_mfma_go<TNW, 2>(p, a, s); return true;
     case 4: nk_mfma_go<TNW, 4>(p, a, s); return true;
     case 8: nk_mfma_go<TNW, 8>(p, a, s); return true;
+    default: return false;
+  }
+}
+
+bool launch_nk_mfma(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
+  switch (p.tile_n) {
+    case 16: return nk_mfma_u<1>(p, a, s);
+    case 32: return nk_mfma_u<2>(p, a, s);
     default: return false;
   }
 }
@@ -384,16 +492,8 @@ bool nk_mfma4_supported(int m_block, int tile_n, int u) {
 
 template <int MG, int R4, int U>
 static void nk_mfma4_go(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
-  const dim3 grid(p.grid_x, p.grid_y, p.grid_z), block(p.block);
-  auto* A = static_cast<const half_t*>(a.A);
-  auto* W = static_cast<const half_t*>(a.W);
-  auto* C = static_cast<half_t*>(a.C);
-  if (p.stream_w)
-    hipLaunchKernelGGL((nk_mfma4_kernel<MG, R4, U, true>), grid, block, 0, s, A, W, C, a.ws, a.M,
-                       a.N, a.K, a.accumulate);
-  else
-    hipLaunchKernelGGL((nk_mfma4_kernel<MG, R4, U, false>), grid, block, 0, s, A, W, C, a.ws, a.M,
-                       a.N, a.K, a.accumulate);
+  if (p.stream_w) FG_LAUNCH((nk_mfma4_kernel<MG, R4, U, true>), p, a, s);
+  else FG_LAUNCH((nk_mfma4_kernel<MG, R4, U, false>), p, a, s);
 }
 
 template <int MG, int R4>
@@ -435,10 +535,59 @@ bool launch_nk_mfma4(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
   }
 }
 
-bool launch_nk_mfma(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
+// Sliced variant: unroll = chunks of 128 K positions per slice (8 or 16), tile_n = 16*RG.
+bool nk_mfma4s_supported(int m_block, int tile_n, int cw) {
+  const bool mg_ok = m_block == 8 || m_block == 12 || m_block == 16;
+  const bool tn_ok = tile_n == 16 || tile_n == 32 || tile_n == 64;
+  return mg_ok && tn_ok && (cw == 8 || cw == 16);
+}
+
+template <int MG, int CW, int RG, bool STREAM>
+static void nk_mfma4s_launch(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
+  constexpr unsigned lds = 4 * MG * CW * 256 + 4 * 4 * MG * 16 * sizeof(float);
+  static bool raised = false;  // more than 64 KB of LDS per workgroup has to be asked for once
+  if (!raised) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&nk_mfma4s_kernel<MG, CW, RG, STREAM>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    raised = true;
+  }
+  hipLaunchKernelGGL((nk_mfma4s_kernel<MG, CW, RG, STREAM>), dim3(p.grid_x, p.grid_y, p.grid_z),
+                     dim3(256), lds, s, static_cast<const half_t*>(a.A),
+                     static_cast<const half_t*>(a.W), static_cast<half_t*>(a.C), a.ws, a.counters,
+                     a.M, a.N, a.K, a.accumulate);
+}
+
+template <int MG, int CW, int RG>
+static void nk_mfma4s_go(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
+  if (p.stream_w) nk_mfma4s_launch<MG, CW, RG, true>(p, a, s);
+  else nk_mfma4s_launch<MG, CW, RG, false>(p, a, s);
+}
+
+template <int MG, int CW>
+static bool nk_mfma4s_rg(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
   switch (p.tile_n) {
-    case 16: return nk_mfma_u<1>(p, a, s);
-    case 32: return nk_mfma_u<2>(p, a, s);
+    case 16: nk_mfma4s_go<MG, CW, 1>(p, a, s); return true;
+    case 32: nk_mfma4s_go<MG, CW, 2>(p, a, s); return true;
+    case 64: nk_mfma4s_go<MG, CW, 4>(p, a, s); return true;
+    default: return false;
+  }
+}
+
+template <int MG>
+static bool nk_mfma4s_cw(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
+  switch (p.unroll) {
+    case 8: return nk_mfma4s_rg<MG, 8>(p, a, s);
+    case 16: return nk_mfma4s_rg<MG, 16>(p, a, s);
+    default: return false;
+  }
+}
+
+bool launch_nk_mfma4s(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
+  if (p.block != 256) return false;
+  switch (p.m_block) {
+    case 8: return nk_mfma4s_cw<2>(p, a, s);
+    case 12: return nk_mfma4s_cw<3>(p, a, s);
+    case 16: return nk_mfma4s_cw<4>(p, a, s);
     default: return false;
   }
 }

@@ -49,7 +49,9 @@ void check_tensor(const at::Tensor& t, const char* name, at::ScalarType dtype, c
 }
 
 // Split-K scratch, one buffer per (device, stream), grown on demand through the caching
-// allocator so that reuse is ordered on the stream that last used it.
+// allocator so that reuse is ordered on the stream that last used it.  Allocated zeroed: the
+// arrival counters at its start must be zero before the first call and every call leaves
+// them zero.
 at::Tensor workspace(const at::Tensor& like, size_t bytes) {
   static std::mutex mu;
   static std::map<std::pair<int, void*>, at::Tensor> cache;
@@ -58,7 +60,7 @@ at::Tensor workspace(const at::Tensor& like, size_t bytes) {
   auto it = cache.find(key);
   if (it == cache.end() || (size_t)it->second.numel() < bytes) {
     size_t want = std::max<size_t>(bytes, (size_t)8 << 20);
-    cache[key] = at::empty({(int64_t)want}, like.options().dtype(at::kByte));
+    cache[key] = at::zeros({(int64_t)want}, like.options().dtype(at::kByte));
     it = cache.find(key);
   }
   return it->second;
@@ -290,6 +292,7 @@ py::dict plan(int M, int N, int K, int w_layout, int splitk) {
   py::dict d;
   d["kernel"] = p.kernel;
   d["splitk"] = p.splitk;
+  d["fused"] = p.fused;
   d["tile_n"] = p.tile_n;
   d["m_block"] = p.m_block;
   d["waves"] = p.waves;

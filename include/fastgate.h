@@ -50,7 +50,9 @@ enum {
   FG_KERNEL_NK_MFMA = 2, /* [N,K] weights, v_mfma_f32_16x16x32_f16, 16 rows of A a block */
   FG_KERNEL_KN_DOT2 = 3, /* [K,N] weights, 8x8 register transpose + v_dot2_f32_f16       */
   FG_KERNEL_KN_MFMA = 4, /* [K,N] weights, 8x8 register transpose + MFMA                 */
-  FG_KERNEL_NK_MFMA4 = 5 /* [N,K] weights, v_mfma_f32_4x4x4_16B_f16: 4 rows x 256 B a load */
+  FG_KERNEL_NK_MFMA4 = 5, /* [N,K] weights, v_mfma_f32_4x4x4_16B_f16: 4 rows x 256 B a load */
+  FG_KERNEL_NK_MFMA4S = 6 /* same instruction; a workgroup owns a K slice of unroll*128, keeps
+                             that slice of A in LDS, its waves split tile_n (16/32/64) columns */
 };
 
 /*
@@ -60,9 +62,12 @@ enum {
  */
 typedef struct fg_plan_t {
   int kernel;   /* FG_KERNEL_*                                                        */
-  int splitk;   /* S >= 1: K is interleaved over S workgroups per output tile; S > 1
-                   writes fp32 partials [S,M,N] to the workspace and runs the second-pass
-                   reduction kernel (no data atomics)                                */
+  int splitk;   /* S >= 1: K is divided over S workgroups per output tile; S > 1 writes
+                   fp32 partials [S,M,N] to the workspace; they are summed in ascending
+                   order of S, so results are reproducible (no data atomics)          */
+  int fused;    /* with S > 1: 1 = the workgroup that finishes a tile last sums the
+                   partials in the same launch (one counter atomic per workgroup),
+                   0 = a second kernel does                                            */
   int tile_n;   /* output columns per workgroup                                       */
   int m_block;  /* rows of A per workgroup (grid.y = ceil(M / m_block))               */
   int waves;    /* wavefronts per workgroup; they interleave over K, reduced in LDS   */
@@ -77,7 +82,10 @@ typedef struct fg_plan_t {
  * is formed in fp32 before the single rounding).
  *   splitk  0 = library heuristic, S >= 1 = forced (the reference's trailing `int bz`).
  *   ws      device scratch of at least fg_workspace_bytes() bytes when the plan's
- *           splitk > 1, else may be NULL.  Contents need no initialisation.
+ *           splitk > 1, else may be NULL.  Its first fg_workspace_header_bytes() bytes hold
+ *           arrival counters: zero them once with fg_workspace_init() (or allocate zeroed
+ *           memory); every call leaves them zero again.  Calls that share a workspace must
+ *           be ordered on one stream.
  * Services, with w_layout = FG_W_KN: edgemm_m8n128k64x4 (backend/cuda/hk/edgemm.cu:102-156),
  * edgemm_m8n128k64x4_amd (:159-213), edgemm_m8n256k32x8 (:363-385, accumulate),
  * flat_gemm_m8n128k64x4_bz1, flat_gemm_m8n256k32x8_bz1, flat_gemm_m8n256k64x8,
@@ -104,6 +112,13 @@ int fg_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* out);
 /* Workspace bytes fg_gemm_f16 needs for this shape and splitk argument (0 when the plan
  * does not split across workgroups).  Host only. */
 size_t fg_workspace_bytes(int M, int N, int K, int w_layout, int splitk);
+
+/* Size of the counter header at the start of a split-K workspace, and the call that zeroes it
+ * (a fill kernel on `stream`, safe to capture in a HIP graph).  Needed once per workspace, not
+ * per call.  The reference has no counterpart: its split-K adds fp16 atomically into a C the
+ * host zeroed with an extra memset launch (backend/cuda/hk/edgemm.cu:138-142). */
+size_t fg_workspace_header_bytes(void);
+int fg_workspace_init(void* ws, size_t ws_bytes, void* stream);
 
 /*
  * W8A16 GEMV: y[m,n] = s_n · ( Σ_k x[m,k]·float(Wq[n,k]) − zero_point·Σ_k x[m,k] ),

@@ -57,13 +57,19 @@ def capi_gemm(A, W, C, w_layout, accumulate=False, splitk=0, plan=None):
     L = capi.lib()
     M, K = A.shape
     N = W.shape[1] if w_layout == capi.FG_W_KN else W.shape[0]
+    hdr = L.fg_workspace_header_bytes()
     if plan is None:
         p = capi.plan(M, N, K, w_layout, splitk)
         wsb = p.workspace_bytes
     else:
         p = plan
-        wsb = max(1, p.splitk) * M * N * 4 if p.splitk > 1 else 0
-    ws = torch.empty(max(wsb, 16), dtype=torch.uint8, device=A.device) if wsb else None
+        # the sliced kernel derives its split from K; leave room for any split up to K/128
+        wsb = hdr + max(p.splitk, K // 128) * M * N * 4
+    ws = None
+    if wsb:
+        # poisoned partials, then the counter header zeroed through the C ABI
+        ws = torch.full((wsb,), 0xFF, dtype=torch.uint8, device=A.device)
+        capi.check(L.fg_workspace_init(ptr(ws), wsb, stream_ptr()), "fg_workspace_init")
     if plan is None:
         st = L.fg_gemm_f16(ptr(A), ptr(W), ptr(C), M, N, K, w_layout, int(accumulate), splitk,
                            ptr(ws), wsb, stream_ptr())
@@ -74,8 +80,8 @@ def capi_gemm(A, W, C, w_layout, accumulate=False, splitk=0, plan=None):
     return p
 
 
-def make_plan(kernel, tile_n=0, m_block=0, waves=4, unroll=1, splitk=1, stream_w=1):
+def make_plan(kernel, tile_n=0, m_block=0, waves=4, unroll=1, splitk=1, stream_w=1, fused=1):
     p = capi.Plan()
     p.kernel, p.tile_n, p.m_block, p.waves = kernel, tile_n, m_block, waves
-    p.unroll, p.splitk, p.stream_w = unroll, splitk, stream_w
+    p.unroll, p.splitk, p.stream_w, p.fused = unroll, splitk, stream_w, fused
     return p

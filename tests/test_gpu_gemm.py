@@ -71,6 +71,65 @@ def test_every_instantiation(device, name, layout, kw):
             assert_close_f16(got, ref, "%s M=%d waves=%d S=%d" % (name, M, waves, splitk))
 
 
+@pytest.mark.parametrize("m_block", [8, 12, 16])
+@pytest.mark.parametrize("tile_n", [16, 32, 64])
+@pytest.mark.parametrize("chunks", [8, 16])
+def test_sliced_mfma4_kernel(device, m_block, tile_n, chunks):
+    # K = 2176 = 17 chunks of 128: two or three K slices, the last one ragged
+    N = 384
+    for K in (640, 2176):
+        for M in sorted({1, m_block - 3, m_block, 2 * m_block + 1}):
+            A, W = _case(M, N, K, NK, 40 + M + K)
+            ref, _ = oracle.gemm_f16(A.numpy(), W.numpy(), NK)
+            C0 = normal((M, N), gen(41), 2.0)
+            refa, _ = oracle.gemm_f16(A.numpy(), W.numpy(), NK, C=C0.numpy(), accumulate=True)
+            for fused in (1, 0):
+                kw = dict(kernel=capi.FG_KERNEL_NK_MFMA4S, tile_n=tile_n, m_block=m_block, unroll=chunks, fused=fused)
+                got, p = _run(A, W, NK, device, plan=make_plan(**kw))
+                assert p.splitk == -(-(K // 128) // chunks)
+                assert_close_f16(got, ref, "mfma4s M=%d K=%d fused=%d" % (M, K, fused))
+                got, _ = _run(A, W, NK, device, accumulate=True, C0=C0, plan=make_plan(**kw))
+                assert_close_f16(got, refa, "mfma4s accumulate M=%d K=%d fused=%d" % (M, K, fused))
+
+
+@pytest.mark.parametrize("layout", [KN, NK])
+@pytest.mark.parametrize("fused", [0, 1])
+def test_split_k_two_pass_and_fused_agree_bitwise(device, layout, fused):
+    # both completions sum the same fp32 partials in ascending split order
+    M, N, K = 8, 512, 4096
+    A, W = _case(M, N, K, layout, 61)
+    kernel = capi.FG_KERNEL_KN_MFMA if layout == KN else capi.FG_KERNEL_NK_MFMA4
+    base = dict(kernel=kernel, tile_n=16, m_block=8, unroll=2)
+    ref_bits = None
+    for splitk in (2, 4, 8):
+        got, _ = _run(A, W, layout, device, plan=make_plan(splitk=splitk, fused=fused, **base))
+        other, _ = _run(A, W, layout, device, plan=make_plan(splitk=splitk, fused=1 - fused, **base))
+        assert (got.view(np.uint16) == other.view(np.uint16)).all()
+        ref, _ = oracle.gemm_f16(A.numpy(), W.numpy(), layout)
+        assert_close_f16(got, ref, "S=%d fused=%d" % (splitk, fused))
+
+
+def test_workspace_counters_return_to_zero(device):
+    # the arrival counters must be zero again after every call so the workspace can be reused
+    from helpers import ptr, stream_ptr
+    L = capi.lib()
+    M, N, K = 16, 1024, 2048
+    hdr = L.fg_workspace_header_bytes()
+    ws = torch.full((hdr + 16 * M * N * 4,), 0xFF, dtype=torch.uint8, device=device)
+    capi.check(L.fg_workspace_init(ptr(ws), ws.numel(), stream_ptr()), "init")
+    for layout in (KN, NK):
+        A, W = _case(M, N, K, layout, 71)
+        ref, _ = oracle.gemm_f16(A.numpy(), W.numpy(), layout)
+        Ad, Wd = A.to(device), W.to(device)
+        C = torch.empty((M, N), dtype=torch.half, device=device)
+        for splitk in (4, 2, 8, 4):
+            capi.check(L.fg_gemm_f16(ptr(Ad), ptr(Wd), ptr(C), M, N, K, layout, 0, splitk, ptr(ws),
+                                     ws.numel(), stream_ptr()), "gemm")
+            torch.cuda.synchronize()
+            assert int(ws[:hdr].view(torch.int32).abs().sum()) == 0
+            assert_close_f16(C.cpu().numpy(), ref, "reuse S=%d" % splitk)
+
+
 @pytest.mark.parametrize("layout", [KN, NK])
 @pytest.mark.parametrize("M", [1, 2, 3, 4, 5, 7, 8, 9, 15, 16, 17, 33])
 def test_auto_plan_small(device, layout, M):

@@ -49,19 +49,25 @@ def test_plan_is_consistent(layout, M, N, K):
     p = capi.plan(M, N, K, layout)
     d = p.as_dict()
     assert p.kernel in ((capi.FG_KERNEL_KN_DOT2, capi.FG_KERNEL_KN_MFMA) if layout == KN
-                        else (capi.FG_KERNEL_NK_DOT2, capi.FG_KERNEL_NK_MFMA)), d
+                        else (capi.FG_KERNEL_NK_DOT2, capi.FG_KERNEL_NK_MFMA, capi.FG_KERNEL_NK_MFMA4,
+                              capi.FG_KERNEL_NK_MFMA4S)), d
     assert N % p.tile_n == 0 and p.grid_x == N // p.tile_n, d
     assert p.grid_y == -(-M // p.m_block) and p.grid_z == p.splitk >= 1, d
     assert p.block == 64 * p.waves and p.waves in (1, 2, 4), d
-    assert p.workspace_bytes == (p.splitk * M * N * 4 if p.splitk > 1 else 0), d
+    hdr = capi.lib().fg_workspace_header_bytes()
+    assert p.workspace_bytes == (hdr + p.splitk * M * N * 4 if p.splitk > 1 else 0), d
     assert capi.workspace_bytes(M, N, K, layout) == p.workspace_bytes
-    # the MFMA kernels are reserved for M >= 8
-    if M < 8:
+    if p.splitk > 1 and p.fused:
+        assert p.grid_x * p.grid_y * 4 <= hdr, d   # one counter per output tile
+    # v_dot2 is the default for the smallest batches; the MFMA kernels take over above
+    if M <= 2:
         assert p.kernel in (capi.FG_KERNEL_KN_DOT2, capi.FG_KERNEL_NK_DOT2), d
+    if p.kernel == capi.FG_KERNEL_NK_MFMA4S:
+        assert p.splitk == -(-(K // 128) // p.unroll) and p.waves == 4, d
     # a forced split is honoured
     for s in (1, 2, 7):
         q = capi.plan(M, N, K, layout, s)
-        assert q.splitk == s and q.workspace_bytes == (s * M * N * 4 if s > 1 else 0)
+        assert q.splitk == s and q.workspace_bytes == (hdr + s * M * N * 4 if s > 1 else 0)
 
 
 def test_plan_fills_the_chip_on_the_metric_shapes():
