@@ -30,7 +30,8 @@ FG_KERNEL_KN_DOT2 = 3
 FG_KERNEL_KN_MFMA = 4
 FG_KERNEL_NK_MFMA4 = 5
 FG_KERNEL_NK_MFMA4S = 6
-KERNEL_NAMES = {1: "nk_dot2", 2: "nk_mfma", 3: "kn_dot2", 4: "kn_mfma", 5: "nk_mfma4", 6: "nk_mfma4s"}
+FG_KERNEL_NK_MFMA_T = 7
+KERNEL_NAMES = {1: "nk_dot2", 2: "nk_mfma", 3: "kn_dot2", 4: "kn_mfma", 5: "nk_mfma4", 6: "nk_mfma4s", 7: "nk_mfma_t"}
 
 # Every symbol include/fastgate.h declares.
 EXPORTS = (
@@ -62,6 +63,7 @@ class Plan(ctypes.Structure):
         ("waves", ctypes.c_int),
         ("unroll", ctypes.c_int),
         ("stream_w", ctypes.c_int),
+        ("stagger", ctypes.c_int),
         ("grid_x", ctypes.c_int),
         ("grid_y", ctypes.c_int),
         ("grid_z", ctypes.c_int),

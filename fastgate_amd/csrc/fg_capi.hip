@@ -72,6 +72,12 @@ int finish_plan(int M, int N, int K, fg_plan_t* p) {
       p->waves = 4;
       p->splitk = ceil_div(K / 128, p->unroll);  // one workgroup per K slice of unroll*128
       break;
+    case FG_KERNEL_NK_MFMA_T:
+      if (!nk_mfma_t_supported(p->unroll, p->tile_n)) return FG_ERR_UNSUPPORTED;
+      p->m_block = 16;
+      p->waves = 4;
+      p->splitk = nk_mfma_t_slices(K);  // each wave owns a fixed K range of at most 512
+      break;
     case FG_KERNEL_KN_DOT2:
       p->tile_n = 128;
       if (!kn_dot2_supported(p->m_block, p->unroll)) return FG_ERR_UNSUPPORTED;
@@ -107,47 +113,89 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
   // (K = N = 8192, M = 16, S = 8: 205 us against 26 us).  The planner never picks it.
   p->fused = 0;
   int items = 1;
-  const bool interleaved = true;  // waves and splits interleave over K
+  bool interleaved = true;  // waves and splits interleave over K (not the transposing kernel)
   if (w_layout == FG_W_NK) {
     // Measured on MI355X at K = N = 8192 (us per call): M=1 dot2 tile 4: 21.6-22.4; M=4 dot2
     // 24.3 / mfma4 22.1; M=8 dot2 27.8 / mfma4 26.2 / mfma16 29.2; M=16 mfma4 36 / mfma16 31.7.
-    if (M <= 2) {
+    // The shape sweep (K = N in 1024..16384 and the LLaMA / DiT shapes) behind these choices is
+    // summarised in profiles/; every rule below is the measured winner for its range.
+    if (M <= 2 || (M <= 4 && N <= 4096 && K >= 8192)) {
+      // (few, long rows at M = 3..4: v_dot2 16.3 us against 19.8 for N = 3072, K = 12288)
       p->kernel = FG_KERNEL_NK_DOT2;
-      p->m_block = M;
+      p->m_block = M <= 2 ? M : 4;
       p->tile_n = 4;
-      p->unroll = 1;
-      items = ceil_div(K / 8, 64);
-    } else if (M <= 8) {
+      p->unroll = (K >= 16384 || M > 2) ? 2 : 1;
+      items = ceil_div(K / 8, 64 * p->unroll);
+      p->stagger = items <= 16;  // at most 4 steps for 4 waves
+    } else if (M <= 4 || (M <= 8 && (splitk > 0 || K < 4096 || N / 16 >= kCUs))) {
       p->kernel = FG_KERNEL_NK_MFMA4;
       p->m_block = M <= 4 ? 4 : 8;
-      p->tile_n = 16;
-      while (p->tile_n > 4 && N / p->tile_n < 2 * kCUs) p->tile_n >>= 1;
-      p->unroll = (K / 128 >= 16) ? 2 : 1;
+      if (K >= 16384) {
+        p->tile_n = 32, p->unroll = 1;
+      } else if (K == 8192 || N <= 4096) {
+        // two chunks per wave and step: 8 steps at K = 8192, one K band per XCD
+        p->tile_n = N <= 4096 ? 8 : 16, p->unroll = K >= 256 ? 2 : 1, p->stagger = K <= 8192;
+      } else {
+        p->tile_n = 16, p->unroll = 1;
+      }
       items = ceil_div(K / 128, p->unroll);
-    } else {
+    } else if (splitk > 0) {
+      // a caller-chosen split-K factor only exists for the K-interleaved kernels
       p->kernel = FG_KERNEL_NK_MFMA;
       p->m_block = 16;
       p->tile_n = (N / 32 >= kCUs) ? 32 : 16;
       p->unroll = p->tile_n == 32 ? 4 : 2;
       if (K / 32 < 4 * p->unroll) p->unroll = 1;
       items = ceil_div(K / 32, p->unroll);
+    } else {
+      // M = 9..16 (and 5..8 for mid-sized K): 16x16x32 MFMA behind the LDS transpose
+      // (K = N = 8192, M = 16: 27.6 us against 31.7 for the direct 16x16x32 kernel)
+      p->kernel = FG_KERNEL_NK_MFMA_T;
+      p->m_block = 16;
+      p->unroll = 16;
+      p->tile_n = (N / 128) * nk_mfma_t_slices(K) >= kCUs / 2 ? 128 : 32;
+      interleaved = false;
     }
   } else {
-    if (M <= 7) {
+    if (M <= 2) {
       p->kernel = FG_KERNEL_KN_DOT2;
-      p->m_block = M <= 1 ? 1 : (M <= 2 ? 2 : (M <= 4 ? 4 : 8));
+      p->m_block = M;
     } else {
-      p->kernel = FG_KERNEL_KN_MFMA;
+      p->kernel = FG_KERNEL_KN_MFMA;  // 26.3 us against 29.8 for v_dot2 at M = 4, K = N = 8192
       p->m_block = 16;
     }
     p->tile_n = 128;
-    p->unroll = (K / 32 >= 64) ? 2 : 1;
+    p->unroll = (p->kernel == FG_KERNEL_KN_DOT2 && K >= 2048) ? 2 : 1;
     items = ceil_div(K / 32, p->unroll);
   }
   if (interleaved) {
     p->waves = pick_waves(items);
     const int tiles = (N / p->tile_n) * ceil_div(M, p->m_block);
-    p->splitk = splitk > 0 ? splitk : pick_splitk(tiles, p->waves, items, M, N, K, kCUs);
+    if (splitk > 0) {
+      p->splitk = splitk;
+    } else if (w_layout == FG_W_KN) {
+      // [K,N] tiles are 128 columns wide, so the grid needs split-K to cover the chip: the
+      // factor that brings tiles*S closest to one workgroup per CU, none for tiny weights.
+      int best = 1;
+      if ((size_t)N * K >= ((size_t)2 << 20)) {
+        double best_ratio = 1e30;
+        for (int S = 1; S <= 16; S *= 2) {
+          if (items / (p->waves * S) < 1) break;
+          const double r = (double)tiles * S / kCUs;
+          const double ratio = r > 1.0 ? r : 1.0 / (r * r);  // idle CUs cost more than a deeper split
+          if (ratio < best_ratio - 1e-9) {
+            best_ratio = ratio;
+            best = S;
+          }
+        }
+      }
+      p->splitk = best;
+    } else {
+      p->splitk = pick_splitk(tiles, p->waves, items, M, N, K, kCUs);
+    }
+  } else {
+    p->waves = 4;
+    p->splitk = 1;  // finish_plan derives it from K
   }
   return finish_plan(M, N, K, p);
 }
@@ -161,7 +209,7 @@ int run_gemm(const void* A, const void* W, void* C, int M, int N, int K, int acc
        reinterpret_cast<uintptr_t>(C) | reinterpret_cast<uintptr_t>(ws)) & 15) {
     return FG_ERR_INVALID_ARG;  // 16-byte loads and stores
   }
-  GemmArgs a{A, W, C, nullptr, nullptr, M, N, K, accumulate ? 1 : 0};
+  GemmArgs a{A, W, C, nullptr, nullptr, M, N, K, (accumulate ? 1 : 0) | (p.stagger ? 2 : 0)};
   if (p.splitk > 1) {
     a.ws = reinterpret_cast<float*>(static_cast<unsigned char*>(ws) + kWsHeaderBytes);
     a.counters = p.fused ? static_cast<int*>(ws) : nullptr;
@@ -173,6 +221,7 @@ int run_gemm(const void* A, const void* W, void* C, int M, int N, int K, int acc
     case FG_KERNEL_NK_MFMA: ok = launch_nk_mfma(p, a, s); break;
     case FG_KERNEL_NK_MFMA4: ok = launch_nk_mfma4(p, a, s); break;
     case FG_KERNEL_NK_MFMA4S: ok = launch_nk_mfma4s(p, a, s); break;
+    case FG_KERNEL_NK_MFMA_T: ok = launch_nk_mfma_t(p, a, s); break;
     case FG_KERNEL_KN_DOT2: ok = launch_kn_dot2(p, a, s); break;
     case FG_KERNEL_KN_MFMA: ok = launch_kn_mfma(p, a, s); break;
     default: break;
@@ -180,7 +229,7 @@ int run_gemm(const void* A, const void* W, void* C, int M, int N, int K, int acc
   if (!ok) return FG_ERR_UNSUPPORTED;
   if (check_launch() != FG_OK) return FG_ERR_LAUNCH;
   if (p.splitk > 1 && !p.fused) {
-    launch_splitk_reduce(a.ws, C, p.splitk, M, N, a.accumulate, s);
+    launch_splitk_reduce(a.ws, C, p.splitk, M, N, a.accumulate & 1, s);
     if (check_launch() != FG_OK) return FG_ERR_LAUNCH;
   }
   return FG_OK;
@@ -188,7 +237,8 @@ int run_gemm(const void* A, const void* W, void* C, int M, int N, int K, int acc
 
 bool is_nk(int kernel) {
   return kernel == FG_KERNEL_NK_DOT2 || kernel == FG_KERNEL_NK_MFMA ||
-         kernel == FG_KERNEL_NK_MFMA4 || kernel == FG_KERNEL_NK_MFMA4S;
+         kernel == FG_KERNEL_NK_MFMA4 || kernel == FG_KERNEL_NK_MFMA4S ||
+         kernel == FG_KERNEL_NK_MFMA_T;
 }
 bool is_kn(int kernel) { return kernel == FG_KERNEL_KN_DOT2 || kernel == FG_KERNEL_KN_MFMA; }
 

@@ -72,6 +72,20 @@ __device__ __forceinline__ float f16_bits_to_f32(uint16_t b) {
   return static_cast<float>(__builtin_bit_cast(half_t, b));
 }
 
+// First K step of a workgroup whose waves walk K in `nsteps` steps (wrapping around).
+// Weight rows are K*2 bytes apart -- a power of two for the usual K -- so workgroups that
+// walk K in lockstep sit on the same HBM and L2 channels at the same time.  Workgroups are
+// dealt to the 8 XCDs round-robin by linear id; numbering them within their XCD (id / 8)
+// spreads the start positions evenly over each XCD's L2 channels as well as over the chip
+// (starting at id % nsteps instead leaves each XCD on 1/8 of the positions: 2.2x slower at
+// K = 8192 with 16 steps).
+// Flag bit 1 selects id % nsteps: with exactly 8 steps every XCD then owns one K band at a time,
+// which measured 9% faster at K = N = 8192 and must not be used with other step counts.
+__device__ __forceinline__ int stagger_start(int nsteps, int flags) {
+  const unsigned lid = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+  return (int)(((flags & 2) ? lid : (lid >> 3)) % (unsigned)nsteps);
+}
+
 // Orders LDS traffic among the lanes of one wavefront (data handed from lane to lane through
 // a wave-private LDS region).  The LDS unit serves a wave's requests in order; this only keeps
 // the compiler from moving the accesses across the hand-over point.  No s_barrier is issued.
@@ -85,27 +99,40 @@ __device__ __forceinline__ void wave_lds_sync() {
 // Split-K completion inside one launch.  Every workgroup of a tile stores its fp32 partial
 // to part[z][m][n], then arrives at the tile's counter; the workgroup that arrives last sums
 // the S partials in ascending z (so the result does not depend on arrival order), writes C
-// and puts the counter back to zero for the next call.  The only atomic is on the counter.
+// and puts the counter back to zero for the next call.  The only atomic RMW is on the counter.
+//
+// The workgroups of a tile run on different XCDs, whose L2s are not coherent with each other.
+// Agent-scope fences would fix that by writing back / invalidating a whole L2 (measured: 2-8x
+// slower kernels), so the partials never live in L2 instead: they are written and read with
+// relaxed agent-scope atomic accesses (write-through stores, L2-bypassing loads), and a
+// workgroup-scope release (s_waitcnt on those stores) orders them before the counter update.
 // ---------------------------------------------------------------------------------------
+__device__ __forceinline__ void store_partial(float* p, float v, bool coherent) {
+  if (coherent) __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  else *p = v;
+}
+__device__ __forceinline__ float load_partial(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 __device__ __forceinline__ bool splitk_last_arriver(int* counter, int S) {
   __shared__ int s_last;
-  __threadfence();  // release: this workgroup's partial stores are visible device-wide
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // partial stores have completed
   __syncthreads();
   if (threadIdx.x == 0) {
-    const int old = atomicAdd(counter, 1);
+    const int old = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     const int last = old == S - 1;
-    if (last) atomicExch(counter, 0);
+    if (last) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     s_last = last;
   }
   __syncthreads();
-  const bool last = s_last != 0;
-  if (last) __threadfence();  // acquire: see the other workgroups' partials
-  return last;
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+  return s_last != 0;
 }
 
 // C[m0..m0+mcnt)[n0..n0+ncnt) = fp16( Σ_z part[z] (+ C) ); ncnt and n0 are multiples of 4.
-__device__ __forceinline__ void splitk_reduce_tile(const float* __restrict__ part, half_t* C, int S,
-                                                   int M, int N, int m0, int mcnt, int n0, int ncnt,
+__device__ __forceinline__ void splitk_reduce_tile(const float* part, half_t* C, int S, int M, int N,
+                                                   int m0, int mcnt, int n0, int ncnt,
                                                    int accumulate) {
   typedef half_t half4v __attribute__((ext_vector_type(4)));
   const int nq = ncnt >> 2;
@@ -114,8 +141,10 @@ __device__ __forceinline__ void splitk_reduce_tile(const float* __restrict__ par
     const int m = m0 + e / nq, n = n0 + (e % nq) * 4;
     if (m >= M) continue;
     const size_t off = (size_t)m * N + n;
-    float4_t sum = *reinterpret_cast<const float4_t*>(part + off);
-    for (int z = 1; z < S; ++z) sum += *reinterpret_cast<const float4_t*>(part + (size_t)z * MN + off);
+    float sum[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int z = 0; z < S; ++z)
+#pragma unroll
+      for (int k = 0; k < 4; ++k) sum[k] += load_partial(part + (size_t)z * MN + off + k);
     half4v* c = reinterpret_cast<half4v*>(C + off);
     if (accumulate) {
       const half4v old = *c;

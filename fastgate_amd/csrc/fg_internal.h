@@ -18,7 +18,7 @@ struct GemmArgs {
   float* ws;      // fp32 [S,M,N] partials when plan.splitk > 1
   int* counters;  // per-tile arrival counters (fused split-K) or null (second-pass kernel)
   int M, N, K;
-  int accumulate;
+  int accumulate;  // bit 0: C += A*W; bit 1: plan.stagger (start step = workgroup id % steps)
 };
 
 // Tile sets that exist as instantiations (the planner and the validators share these).
@@ -26,6 +26,8 @@ bool nk_dot2_supported(int m_block, int tile_n, int unroll);
 bool nk_mfma_supported(int tile_n, int unroll);
 bool nk_mfma4_supported(int m_block, int tile_n, int unroll);
 bool nk_mfma4s_supported(int m_block, int tile_n, int chunks);
+bool nk_mfma_t_supported(int rows, int tile_n);
+int nk_mfma_t_slices(int K);
 bool kn_dot2_supported(int m_block, int unroll);
 bool kn_mfma_supported(int unroll);
 
@@ -33,6 +35,7 @@ bool launch_nk_dot2(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
 bool launch_nk_mfma(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
 bool launch_nk_mfma4(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
 bool launch_nk_mfma4s(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
+bool launch_nk_mfma_t(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
 bool launch_kn_dot2(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
 bool launch_kn_mfma(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
 

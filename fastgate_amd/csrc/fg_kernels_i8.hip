@@ -22,13 +22,13 @@ __device__ __forceinline__ void i8x4_to_half2x2(uint32_t w, half2_t& lo, half2_t
 }
 
 template <int MB, int RN, int U>
-__global__ __launch_bounds__(256) void w8a16_kernel(const int8_t* __restrict__ Wq,
+__global__ __launch_bounds__(512) void w8a16_kernel(const int8_t* __restrict__ Wq,
                                                     const half_t* __restrict__ X,
                                                     const half_t* __restrict__ scale,
                                                     float scalar_scale, float zero_point,
                                                     half_t* __restrict__ Y, int M, int N, int K) {
-  __shared__ float red[16][RN * MB];
-  __shared__ float redx[16][MB];
+  __shared__ float red[32][RN * MB];
+  __shared__ float redx[32][MB];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int nw = blockDim.x >> 6;
@@ -48,7 +48,11 @@ __global__ __launch_bounds__(256) void w8a16_kernel(const int8_t* __restrict__ W
   const u32x4 zero = {0u, 0u, 0u, 0u};
   const half2_t ones = {static_cast<half_t>(1.f), static_cast<half_t>(1.f)};
 
-  for (int q0 = wave * (64 * U); q0 < nq; q0 += nw * (64 * U)) {
+  const int nsteps = (nq + nw * (64 * U) - 1) / (nw * (64 * U));
+  int step = stagger_start(nsteps, 0);
+  for (int it = 0; it < nsteps; ++it) {
+    const int q0 = (step * nw + wave) * (64 * U);
+    step = step + 1 == nsteps ? 0 : step + 1;
     u32x4 wr[U][RN];
     u32x4 xr[U][MB][2];
 #pragma unroll
@@ -141,7 +145,11 @@ __global__ __launch_bounds__(256) void i8i8_kernel(const int8_t* __restrict__ Wq
   const int8_t* Wt = Wq + (size_t)n0 * K;
   const u32x4 zero = {0u, 0u, 0u, 0u};
 
-  for (int q0 = wave * (64 * U); q0 < nq; q0 += nw * (64 * U)) {
+  const int nsteps = (nq + nw * (64 * U) - 1) / (nw * (64 * U));
+  int step = stagger_start(nsteps, 0);
+  for (int it = 0; it < nsteps; ++it) {
+    const int q0 = (step * nw + wave) * (64 * U);
+    step = step + 1 == nsteps ? 0 : step + 1;
     u32x4 wr[U][RN];
     u32x4 xr[U][MB];
 #pragma unroll
@@ -211,6 +219,11 @@ static void w8a16_go(const W8A16Args& a, hipStream_t s) {
   auto* sc = static_cast<const half_t*>(a.scale);
   auto* Y = static_cast<half_t*>(a.y);
   const dim3 block(64 * i8_waves(a.K));
+  if (MB == 1) {  // measured best at K = N = 8192 (12.6 us): 4 rows, one load group in flight
+    hipLaunchKernelGGL((w8a16_kernel<1, 4, 1>), dim3(a.N / 4), block, 0, s, Wq, X, sc,
+                       a.scalar_scale, a.zero_point, Y, a.M, a.N, a.K);
+    return;
+  }
   if (a.N / 8 >= 512 && MB <= 4) {
     hipLaunchKernelGGL((w8a16_kernel<MB, 8, 2>), dim3(a.N / 8), block, 0, s, Wq, X, sc,
                        a.scalar_scale, a.zero_point, Y, a.M, a.N, a.K);
@@ -235,6 +248,10 @@ static void i8i8_go(const void* Wq, const void* xq, int32_t* acc, int M, int N, 
   auto* W = static_cast<const int8_t*>(Wq);
   auto* X = static_cast<const int8_t*>(xq);
   const dim3 block(64 * i8_waves(K));
+  if (MB == 1) {
+    hipLaunchKernelGGL((i8i8_kernel<1, 4, 1>), dim3(N / 4), block, 0, s, W, X, acc, M, N, K);
+    return;
+  }
   if (N / 8 >= 512 && MB <= 4) {
     hipLaunchKernelGGL((i8i8_kernel<MB, 8, 2>), dim3(N / 8), block, 0, s, W, X, acc, M, N, K);
   } else {

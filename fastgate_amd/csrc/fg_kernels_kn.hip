@@ -43,6 +43,7 @@ __global__ __launch_bounds__(256) void kn_mfma_kernel(const half_t* __restrict__
                                                       half_t* __restrict__ C,
                                                       float* __restrict__ ws, int* counters, int M, int N,
                                                       int K, int accumulate) {
+  accumulate &= 1;  // the flag word also carries the stagger mode of the [N,K] kernels
   __shared__ float red[4][16][128];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -115,8 +116,13 @@ __global__ __launch_bounds__(256) void kn_mfma_kernel(const half_t* __restrict__
         *reinterpret_cast<half8_t*>(c) = out;
       } else {
         float* o = ws + ((size_t)blockIdx.z * M + mg) * N + n0 + c0;
-        *reinterpret_cast<float4_t*>(o) = float4_t{sum[0], sum[1], sum[2], sum[3]};
-        *reinterpret_cast<float4_t*>(o + 4) = float4_t{sum[4], sum[5], sum[6], sum[7]};
+        if (counters != nullptr) {
+#pragma unroll
+          for (int i = 0; i < 8; ++i) store_partial(o + i, sum[i], true);
+        } else {
+          *reinterpret_cast<float4_t*>(o) = float4_t{sum[0], sum[1], sum[2], sum[3]};
+          *reinterpret_cast<float4_t*>(o + 4) = float4_t{sum[4], sum[5], sum[6], sum[7]};
+        }
       }
     }
   }
@@ -134,6 +140,7 @@ __global__ __launch_bounds__(256) void kn_dot2_kernel(const half_t* __restrict__
                                                       half_t* __restrict__ C,
                                                       float* __restrict__ ws, int* counters, int M, int N,
                                                       int K, int accumulate) {
+  accumulate &= 1;  // the flag word also carries the stagger mode of the [N,K] kernels
   __shared__ float red[16][MB][128];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -197,7 +204,7 @@ __global__ __launch_bounds__(256) void kn_dot2_kernel(const half_t* __restrict__
         if (accumulate) sum += static_cast<float>(*c);
         *c = static_cast<half_t>(sum);
       } else {
-        ws[((size_t)blockIdx.z * M + mg) * N + n] = sum;
+        store_partial(ws + ((size_t)blockIdx.z * M + mg) * N + n, sum, counters != nullptr);
       }
     }
   }

@@ -25,7 +25,8 @@ __global__ __launch_bounds__(256) void nk_dot2_kernel(const half_t* __restrict__
                                                       const half_t* __restrict__ W,
                                                       half_t* __restrict__ C,
                                                       float* __restrict__ ws, int* counters, int M,
-                                                      int N, int K, int accumulate) {
+                                                      int N, int K, int flags) {
+  const int accumulate = flags & 1;  // bit 1 of flags selects the start stagger
   __shared__ float red[16][RN * MB];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -47,7 +48,7 @@ __global__ __launch_bounds__(256) void nk_dot2_kernel(const half_t* __restrict__
   const u32x4 zero = {0u, 0u, 0u, 0u};
 
   const int nsteps = (nq + slots * (64 * U) - 1) / (slots * (64 * U));
-  int step = (blockIdx.x + blockIdx.y) % nsteps;  // staggered start
+  int step = stagger_start(nsteps, flags);
   for (int it = 0; it < nsteps; ++it) {
     const int q0 = (step * slots + slot) * (64 * U);
     step = step + 1 == nsteps ? 0 : step + 1;
@@ -92,7 +93,7 @@ __global__ __launch_bounds__(256) void nk_dot2_kernel(const half_t* __restrict__
         if (accumulate) sum += static_cast<float>(*c);
         *c = static_cast<half_t>(sum);
       } else {
-        ws[((size_t)blockIdx.z * M + mg) * N + n] = sum;
+        store_partial(ws + ((size_t)blockIdx.z * M + mg) * N + n, sum, counters != nullptr);
       }
     }
   }
@@ -111,7 +112,8 @@ __global__ __launch_bounds__(256) void nk_mfma_kernel(const half_t* __restrict__
                                                       const half_t* __restrict__ W,
                                                       half_t* __restrict__ C,
                                                       float* __restrict__ ws, int* counters, int M,
-                                                      int N, int K, int accumulate) {
+                                                      int N, int K, int flags) {
+  const int accumulate = flags & 1;  // bit 1 of flags selects the start stagger
   __shared__ float red[4][TNW][256];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -133,7 +135,7 @@ __global__ __launch_bounds__(256) void nk_mfma_kernel(const half_t* __restrict__
   const u32x4 zero = {0u, 0u, 0u, 0u};
 
   const int nsteps = (nunits + slots * U - 1) / (slots * U);
-  int step = (blockIdx.x + blockIdx.y) % nsteps;  // staggered start
+  int step = stagger_start(nsteps, flags);
   for (int it = 0; it < nsteps; ++it) {
     const int u0 = (step * slots + slot) * U;
     step = step + 1 == nsteps ? 0 : step + 1;
@@ -173,7 +175,7 @@ __global__ __launch_bounds__(256) void nk_mfma_kernel(const half_t* __restrict__
         if (accumulate) sum += static_cast<float>(*c);
         *c = static_cast<half_t>(sum);
       } else {
-        ws[((size_t)blockIdx.z * M + mg) * N + n] = sum;
+        store_partial(ws + ((size_t)blockIdx.z * M + mg) * N + n, sum, counters != nullptr);
       }
     }
   }
@@ -202,7 +204,8 @@ __global__ __launch_bounds__(256) void nk_mfma4_kernel(const half_t* __restrict_
                                                        const half_t* __restrict__ W,
                                                        half_t* __restrict__ C,
                                                        float* __restrict__ ws, int* counters, int M,
-                                                       int N, int K, int accumulate) {
+                                                       int N, int K, int flags) {
+  const int accumulate = flags & 1;  // bit 1 of flags selects the start stagger
   __shared__ float red[16][R4 * MG * 16];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -225,7 +228,7 @@ __global__ __launch_bounds__(256) void nk_mfma4_kernel(const half_t* __restrict_
   const u32x4 zero = {0u, 0u, 0u, 0u};
 
   const int nsteps = (nchunks + slots * U - 1) / (slots * U);
-  int step = (blockIdx.x + blockIdx.y) % nsteps;  // staggered start
+  int step = stagger_start(nsteps, flags);
   for (int it = 0; it < nsteps; ++it) {
     const int c0 = (step * slots + slot) * U;
     step = step + 1 == nsteps ? 0 : step + 1;
@@ -280,7 +283,7 @@ __global__ __launch_bounds__(256) void nk_mfma4_kernel(const half_t* __restrict_
         if (accumulate) sum += static_cast<float>(*c);
         *c = static_cast<half_t>(sum);
       } else {
-        ws[((size_t)blockIdx.z * M + mg) * N + n] = sum;
+        store_partial(ws + ((size_t)blockIdx.z * M + mg) * N + n, sum, counters != nullptr);
       }
     }
   }
@@ -299,7 +302,8 @@ __global__ __launch_bounds__(256) void nk_mfma4s_kernel(const half_t* __restrict
                                                         const half_t* __restrict__ W,
                                                         half_t* __restrict__ C,
                                                         float* __restrict__ ws, int* counters, int M,
-                                                        int N, int K, int accumulate) {
+                                                        int N, int K, int flags) {
+  const int accumulate = flags & 1;  // bit 1 of flags selects the start stagger
   constexpr int TN = 16 * RG;     // columns per workgroup (4 waves x RG x 4)
   constexpr int AROWB = CW * 256;  // bytes per LDS row of A
   // LDS: A panel [4*MG][CW*256 B], then red[4 waves][4 dpp rows][MG*16] floats.  The 16-byte
@@ -379,7 +383,7 @@ __global__ __launch_bounds__(256) void nk_mfma4s_kernel(const half_t* __restrict
           if (accumulate) out += static_cast<float>(*c);
           *c = static_cast<half_t>(out);
         } else {
-          ws[((size_t)blockIdx.z * M + mg) * N + n] = sum;
+          store_partial(ws + ((size_t)blockIdx.z * M + mg) * N + n, sum, counters != nullptr);
         }
       }
     }
@@ -393,9 +397,117 @@ __global__ __launch_bounds__(256) void nk_mfma4s_kernel(const half_t* __restrict
 }
 
 // ---------------------------------------------------------------------------------------
+// MFMA 16x16x32 kernel with row-friendly loads ("transposing" variant) for M = 5..16.
+// The 16x16x32 B operand wants 16 rows x 64 B per instruction, which is the worst shape for
+// HBM.  Here a wave instead loads ROWS rows x 1 KB (one row per instruction, 64 lanes x 16 B
+// along K), parks them in a wave-private LDS buffer and reads them back in operand order
+// (lane (j,g): row j, 16-byte piece 4u+g); rows are padded to 1040 B so both directions are
+// free of bank conflicts.  No workgroup barrier is involved.
+// Each wave owns a fixed K range of ur*32 positions (ur <= 16) for the whole kernel, so its
+// A operands are loaded once into 16 registers-quads and reused for every row tile: the A
+// traffic is 1/(ROWS*T) of the weight traffic instead of 1/1.  The wave walks T tiles of ROWS
+// rows, next tile's loads in flight during the current tile's LDS round trip and MFMAs; the
+// 4 waves of a workgroup (adjacent K ranges) meet in LDS at the end, the gridDim.z workgroups
+// of a tile in the split-K workspace.  ROWS = 8 leaves half of each MFMA idle (it is nowhere
+// near the limit) in exchange for half as many rows in flight.
+// ---------------------------------------------------------------------------------------
+template <int ROWS, int T, bool FULL, bool STREAM>
+__global__ __launch_bounds__(256) void nk_mfma_t_kernel(const half_t* __restrict__ A,
+                                                        const half_t* __restrict__ W,
+                                                        half_t* __restrict__ C,
+                                                        float* __restrict__ ws, int* counters, int M,
+                                                        int N, int K, int accumulate, int ur) {
+  // FULL: every wave range is complete (ur == 16 and K a multiple of 2048), no K masks needed.
+  accumulate &= 1;  // the flag word also carries the stagger mode of the interleaved kernels
+  constexpr int RS = 1040;  // LDS bytes per staged row: 1 KB + 16 B
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int j = lane & 15, g = lane >> 4;
+  const int n0 = blockIdx.x * (ROWS * T);
+  const int m0 = blockIdx.y * 16;
+  const int nunits = K >> 5;
+  if (FULL) ur = 16;
+  const int u_lo = (blockIdx.z * 4 + wave) * ur;  // first 32-wide K unit of this wave
+  unsigned char* wb = smem + wave * (ROWS * RS);
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+
+  // lane l streams the 16-byte piece l of the wave's K range, for every row; first tile first
+  const bool lane_ok = FULL || (lane < 4 * ur && (u_lo * 4 + lane) < nunits * 4);
+  const half_t* Wp = W + (size_t)n0 * K + (size_t)u_lo * 32 + lane * 8;
+  u32x4 wcur[ROWS], wnxt[ROWS];
+#pragma unroll
+  for (int r = 0; r < ROWS; ++r) wcur[r] = lane_ok ? load16<STREAM>(Wp + (size_t)r * K) : zero;
+
+  // A operands of the whole K range: a[u] = A[m0+j][32*(u_lo+u) + 8g .. +7], zero where the
+  // row or the unit does not exist (the staged weights of such units are zero as well)
+  u32x4 a[16];
+  const bool arow = (m0 + j) < M;
+  const half_t* Ap = A + (size_t)(m0 + (arow ? j : 0)) * K + (size_t)u_lo * 32 + g * 8;
+#pragma unroll
+  for (int u = 0; u < 16; ++u)
+    a[u] = (arow && (FULL || (u < ur && (u_lo + u) < nunits))) ? load16<false>(Ap + u * 32) : zero;
+
+  float4_t acc[T];
+#pragma unroll
+  for (int t = 0; t < T; ++t) {
+    acc[t] = float4_t{0.f, 0.f, 0.f, 0.f};
+    if (t + 1 < T) {
+#pragma unroll
+      for (int r = 0; r < ROWS; ++r)
+        wnxt[r] = lane_ok ? load16<STREAM>(Wp + (size_t)((t + 1) * ROWS + r) * K) : zero;
+    }
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) *reinterpret_cast<u32x4*>(wb + r * RS + lane * 16) = wcur[r];
+    wave_lds_sync();
+    u32x4 b[16];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+      b[u] = zero;
+      if (ROWS == 16 || j < ROWS) b[u] = *reinterpret_cast<const u32x4*>(wb + j * RS + (4 * u + g) * 16);
+    }
+#pragma unroll
+    for (int u = 0; u < 16; ++u)
+      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(a[u]), as_half8(b[u]), acc[t], 0, 0, 0);
+    wave_lds_sync();
+    if (t + 1 < T) {
+#pragma unroll
+      for (int r = 0; r < ROWS; ++r) wcur[r] = wnxt[r];
+    }
+  }
+
+  // acc[t][r] = D[m = 4g + r][row j of tile t]; the 4 waves' partials meet in LDS
+  __syncthreads();
+  float(*red)[T][16 * ROWS] = reinterpret_cast<float(*)[T][16 * ROWS]>(smem);
+  if (j < ROWS) {
+#pragma unroll
+    for (int t = 0; t < T; ++t)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) red[wave][t][(4 * g + r) * ROWS + j] = acc[t][r];
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < T * 16 * ROWS; e += 256) {
+    const int m = e / (T * ROWS), c = e % (T * ROWS), t = c / ROWS, jj = c % ROWS;
+    float sum = red[0][t][m * ROWS + jj] + red[1][t][m * ROWS + jj] + red[2][t][m * ROWS + jj] +
+                red[3][t][m * ROWS + jj];
+    const int mg = m0 + m, n = n0 + c;
+    if (mg < M) {
+      if (gridDim.z == 1) {
+        half_t* cp = C + (size_t)mg * N + n;
+        if (accumulate) sum += static_cast<float>(*cp);
+        *cp = static_cast<half_t>(sum);
+      } else {
+        store_partial(ws + ((size_t)blockIdx.z * M + mg) * N + n, sum, counters != nullptr);
+      }
+    }
+  }
+  finish_splitk<16, ROWS * T>(ws, counters, C, M, N, m0, n0, accumulate);
+}
+
+// ---------------------------------------------------------------------------------------
 // Host launchers
 // ---------------------------------------------------------------------------------------
-#define FG_LAUNCH(KERNEL, p, a, s)                                                            \
+#define FG_LAUNCH(KERNEL, p, a, s)                                                           \
   hipLaunchKernelGGL(KERNEL, dim3((p).grid_x, (p).grid_y, (p).grid_z), dim3((p).block), 0, s, \
                      static_cast<const half_t*>((a).A), static_cast<const half_t*>((a).W),    \
                      static_cast<half_t*>((a).C), (a).ws, (a).counters, (a).M, (a).N, (a).K,  \
@@ -578,6 +690,64 @@ static bool nk_mfma4s_cw(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
   switch (p.unroll) {
     case 8: return nk_mfma4s_rg<MG, 8>(p, a, s);
     case 16: return nk_mfma4s_rg<MG, 16>(p, a, s);
+    default: return false;
+  }
+}
+
+// Transposing variant: unroll = rows per tile (8 or 16), tile_n = rows * T with T in {2,4,8}.
+bool nk_mfma_t_supported(int rows, int tile_n) {
+  if (rows != 8 && rows != 16) return false;
+  const int t = tile_n / rows;
+  return tile_n % rows == 0 && (t == 2 || t == 4 || t == 8);
+}
+
+int nk_mfma_t_slices(int K) { return ((K >> 5) + 63) / 64; }  // workgroups along K (4 waves x <=16 units)
+
+template <int ROWS, int T, bool FULL, bool STREAM>
+static void nk_mfma_t_launch(const fg_plan_t& p, const GemmArgs& a, hipStream_t s, int ur) {
+  constexpr unsigned lds = 4 * ROWS * 1040;
+  static bool raised = false;  // more than 64 KB of LDS per workgroup has to be asked for once
+  if (!raised) {
+    (void)hipFuncSetAttribute(
+        reinterpret_cast<const void*>(&nk_mfma_t_kernel<ROWS, T, FULL, STREAM>),
+        hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    raised = true;
+  }
+  hipLaunchKernelGGL((nk_mfma_t_kernel<ROWS, T, FULL, STREAM>),
+                     dim3(p.grid_x, p.grid_y, p.grid_z), dim3(256), lds, s,
+                     static_cast<const half_t*>(a.A), static_cast<const half_t*>(a.W),
+                     static_cast<half_t*>(a.C), a.ws, a.counters, a.M, a.N, a.K, a.accumulate, ur);
+}
+
+template <int ROWS, int T>
+static void nk_mfma_t_go(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
+  const int nunits = a.K >> 5;
+  const int ur = (nunits + 4 * p.grid_z - 1) / (4 * p.grid_z);  // K units per wave, <= 16
+  const bool full = ur == 16 && nunits == 64 * p.grid_z;
+  if (full) {
+    if (p.stream_w) nk_mfma_t_launch<ROWS, T, true, true>(p, a, s, ur);
+    else nk_mfma_t_launch<ROWS, T, true, false>(p, a, s, ur);
+  } else {
+    if (p.stream_w) nk_mfma_t_launch<ROWS, T, false, true>(p, a, s, ur);
+    else nk_mfma_t_launch<ROWS, T, false, false>(p, a, s, ur);
+  }
+}
+
+template <int ROWS>
+static bool nk_mfma_t_t(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
+  switch (p.tile_n / ROWS) {
+    case 2: nk_mfma_t_go<ROWS, 2>(p, a, s); return true;
+    case 4: nk_mfma_t_go<ROWS, 4>(p, a, s); return true;
+    case 8: nk_mfma_t_go<ROWS, 8>(p, a, s); return true;
+    default: return false;
+  }
+}
+
+bool launch_nk_mfma_t(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
+  if (p.block != 256 || p.grid_z != nk_mfma_t_slices(a.K)) return false;
+  switch (p.unroll) {
+    case 8: return nk_mfma_t_t<8>(p, a, s);
+    case 16: return nk_mfma_t_t<16>(p, a, s);
     default: return false;
   }
 }

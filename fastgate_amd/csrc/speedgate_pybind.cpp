@@ -298,6 +298,7 @@ py::dict plan(int M, int N, int K, int w_layout, int splitk) {
   d["waves"] = p.waves;
   d["unroll"] = p.unroll;
   d["stream_w"] = p.stream_w;
+  d["stagger"] = p.stagger;
   d["grid"] = py::make_tuple(p.grid_x, p.grid_y, p.grid_z);
   d["block"] = p.block;
   d["workspace_bytes"] = p.workspace_bytes;

@@ -51,8 +51,11 @@ enum {
   FG_KERNEL_KN_DOT2 = 3, /* [K,N] weights, 8x8 register transpose + v_dot2_f32_f16       */
   FG_KERNEL_KN_MFMA = 4, /* [K,N] weights, 8x8 register transpose + MFMA                 */
   FG_KERNEL_NK_MFMA4 = 5, /* [N,K] weights, v_mfma_f32_4x4x4_16B_f16: 4 rows x 256 B a load */
-  FG_KERNEL_NK_MFMA4S = 6 /* same instruction; a workgroup owns a K slice of unroll*128, keeps
-                             that slice of A in LDS, its waves split tile_n (16/32/64) columns */
+  FG_KERNEL_NK_MFMA4S = 6, /* same instruction; a workgroup owns a K slice of unroll*128, keeps
+                              that slice of A in LDS, its waves split tile_n (16/32/64) columns */
+  FG_KERNEL_NK_MFMA_T = 7  /* [N,K] weights, 16x16x32 MFMA fed through a wave-private LDS
+                              transpose: loads are `unroll` (8/16) rows x 1 KB, every wave keeps
+                              the A operands of its fixed K range in registers               */
 };
 
 /*
@@ -73,6 +76,9 @@ typedef struct fg_plan_t {
   int waves;    /* wavefronts per workgroup; they interleave over K, reduced in LDS   */
   int unroll;   /* independent 16-byte load groups in flight per lane and step        */
   int stream_w; /* 1 = weight loads carry the non-temporal hint                       */
+  int stagger;  /* K-interleaved [N,K] kernels start each workgroup at its own K step:
+                   0 = (workgroup id / 8) % steps, spread within every XCD (default);
+                   1 = workgroup id % steps, one K band per XCD (only with 8 steps)  */
   int grid_x, grid_y, grid_z, block; /* filled by fg_plan / fg_gemm_f16_planned       */
   size_t workspace_bytes;            /* 0 when splitk == 1                            */
 } fg_plan_t;

@@ -92,6 +92,33 @@ def test_sliced_mfma4_kernel(device, m_block, tile_n, chunks):
                 assert_close_f16(got, refa, "mfma4s accumulate M=%d K=%d fused=%d" % (M, K, fused))
 
 
+@pytest.mark.parametrize("rows", [8, 16])
+@pytest.mark.parametrize("tiles", [2, 4, 8])
+def test_transposing_mfma_kernel(device, rows, tiles):
+    # K = 128 (4 units: one wave busy, three idle), 640 (5 units per wave), 2176 (two K slices,
+    # 9 units per wave, the last wave ragged), 6144 (three slices of 16 units)
+    N = 384 if (rows * tiles) in (16, 32, 64, 128) else 512
+    for K in (128, 640, 2176, 6144):
+        for M in (1, 5, 8, 16, 19):
+            A, W = _case(M, N, K, NK, 50 + M + K)
+            ref, _ = oracle.gemm_f16(A.numpy(), W.numpy(), NK)
+            C0 = normal((M, N), gen(51), 2.0)
+            refa, _ = oracle.gemm_f16(A.numpy(), W.numpy(), NK, C=C0.numpy(), accumulate=True)
+            kw = dict(kernel=capi.FG_KERNEL_NK_MFMA_T, tile_n=rows * tiles, unroll=rows)
+            got, p = _run(A, W, NK, device, plan=make_plan(**kw))
+            assert p.splitk == -(-(K // 32) // 64) and p.block == 256
+            assert_close_f16(got, ref, "mfma_t M=%d K=%d" % (M, K))
+            got, _ = _run(A, W, NK, device, accumulate=True, C0=C0, plan=make_plan(**kw))
+            assert_close_f16(got, refa, "mfma_t accumulate M=%d K=%d" % (M, K))
+    # exact small integers: any operand-layout mistake in the LDS round trip changes the bits
+    g = gen(52)
+    A = torch.randint(-2, 3, (16, 512), generator=g).half()
+    W = torch.randint(-3, 4, (N, 512), generator=g).half()
+    ref, _ = oracle.gemm_f16(A.numpy(), W.numpy(), NK)
+    got, _ = _run(A, W, NK, device, plan=make_plan(kernel=capi.FG_KERNEL_NK_MFMA_T, tile_n=rows * tiles, unroll=rows))
+    assert (got == ref).all()
+
+
 @pytest.mark.parametrize("layout", [KN, NK])
 @pytest.mark.parametrize("fused", [0, 1])
 def test_split_k_two_pass_and_fused_agree_bitwise(device, layout, fused):
