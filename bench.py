@@ -37,9 +37,24 @@ MS = (1, 8, 16)
 R = 5  # weight buffers per layout
 HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E peak
 
-# HBM bytes per launch of the roofline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE,
-# keyed by kernel family and M; see profiles/ for the runs.  None = not measured.
-TRAFFIC_BYTES = {}
+# HBM bytes per launch from two rocprofv3 --pmc runs of this script (FETCH_SIZE, then WRITE_SIZE,
+# KiB per dispatch), keyed by kernel family and M.  Each counter is scaled by what it reads for
+# kernels of known traffic (--calibrate-traffic: a 1 GiB read and a 256 MiB copy): FETCH_SIZE
+# reports half the bytes on this part (factor 2.0), WRITE_SIZE all of them (factor 1.0).
+# The summaries are under profiles/.  A kernel/M not listed reports null.
+FETCH_SCALE, WRITE_SCALE = 2.0, 1.0
+
+
+def _traffic(fetch_kib: float, write_kib: float) -> int:
+    return int(round((fetch_kib * FETCH_SCALE + write_kib * WRITE_SCALE) * 1024))
+
+
+TRAFFIC_BYTES = {
+    "nk_dot2_M1": _traffic(65621.2, 64.0),
+    "nk_mfma4_M8": _traffic(66096.5, 128.0),
+    "nk_mfma_t_M16": _traffic(66629.0, 2048.0),   # main kernel only; the 2 MiB written are split-K partials
+    "kn_dot2_M1": _traffic(65635.6, 128.0),
+}
 
 
 def algorithmic_bytes(M: int) -> int:
@@ -51,6 +66,9 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--calibrate-traffic", action="store_true",
+                    help="only run kernels of known traffic (1 GiB read probe, 256 MiB device copy) for "
+                         "scaling rocprofv3's FETCH_SIZE / WRITE_SIZE counters, then exit")
     ap.add_argument("--cpu-repeats", type=int, default=8, help="repetitions of the step on the CPU oracle (0 = skip)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -71,6 +89,24 @@ def main() -> int:
     sg = fastgate_amd.speedgate  # ImportError if the extension was not built
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+
+    if args.calibrate_traffic:
+        import ctypes
+        L = capi.lib()
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).random_(0, 256)
+        sink = torch.empty(L.fg_stream_read_sink_bytes(), dtype=torch.uint8, device=dev)
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        for _ in range(5):
+            L.fg_stream_read(ctypes.c_void_p(src.data_ptr()), 1 << 30, ctypes.c_void_p(sink.data_ptr()), stream)
+        a = src[: 256 << 20].view(torch.int32)
+        b = torch.empty_like(a)
+        for _ in range(5):
+            b.copy_(a)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibration": {"stream_read_kernel": {"read_bytes": 1 << 30, "write_bytes": 0, "launches": 5},
+                                          "device_copy_kernel": {"read_bytes": 256 << 20, "write_bytes": 256 << 20,
+                                                                 "launches": 5}}}))
+        return 0
 
     # ---- synthetic inputs, seeded on the CPU so the CPU baseline sees the same bits ----------
     g = torch.Generator().manual_seed(8192)
