@@ -73,7 +73,7 @@ def main() -> int:
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU; --gpus %d is not supported "
-              "(the path shards by output columns without any collective, see DESIGN.md)" % args.gpus,
+              "(the path shards by output columns without any collective; each GPU would run this same kernel on its share)" % args.gpus,
               file=sys.stderr)
         return 2
 
