@@ -61,6 +61,93 @@ def algorithmic_bytes(M: int) -> int:
     return 2 * K * N + 2 * M * K + 2 * M * N
 
 
+def run_sweep(torch, sg, capi, dev, steps, warmup):
+    """Per-shape timing of the benchmark configurations: us per call, GB/s on algorithmic bytes,
+    fraction of the 8 TB/s peak, and the plan (kernel, split-K, tile) the library chose."""
+    import ctypes
+    L = capi.lib()
+
+    def time_us(fn):
+        for i in range(warmup):
+            fn(i)
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(steps):
+            fn(i)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / steps
+
+    # read ceiling for the "fraction of the measured ceiling" column
+    probe = [torch.empty(1 << 30, dtype=torch.uint8, device=dev).random_(0, 256) for _ in range(2)]
+    sink = torch.empty(L.fg_stream_read_sink_bytes(), dtype=torch.uint8, device=dev)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    us = time_us(lambda i: L.fg_stream_read(ctypes.c_void_p(probe[i % 2].data_ptr()), 1 << 30,
+                                            ctypes.c_void_p(sink.data_ptr()), stream))
+    ceiling = (1 << 30) / us / 1e3
+    del probe
+
+    rows = []
+
+    def fp16_case(name, op, M, Kk, Nn, layout, seed):
+        g = torch.Generator(device=dev).manual_seed(seed)
+        nbuf = max(2, min(320, -(-(640 << 20) // (2 * Kk * Nn))))  # rotate over > 512 MiB of weights
+        shape = (Nn, Kk) if layout == capi.FG_W_NK else (Kk, Nn)
+        ws = [(torch.randn(shape, device=dev, generator=g) * 0.02).half() for _ in range(nbuf)]
+        a = torch.randn((M, Kk), device=dev, generator=g).half()
+        c = torch.zeros((M, Nn), dtype=torch.half, device=dev)
+        fn = getattr(sg, op)
+        if op.startswith("fastgemv"):
+            call = lambda i: fn(ws[i % nbuf], a, c)
+        else:
+            call = lambda i: fn(a, ws[i % nbuf], c)
+        us_call = time_us(call)
+        by = 2 * Kk * Nn + 2 * M * Kk + 2 * M * Nn
+        p = capi.plan(M, Nn, Kk, layout, 0).as_dict()
+        rows.append({"config": name, "op": op, "M": M, "K": Kk, "N": Nn,
+                     "w_layout": "[N,K]" if layout == capi.FG_W_NK else "[K,N]", "seed": seed,
+                     "kernel": p["kernel_name"], "splitk": p["splitk"], "in_launch_reduce": p["fused"],
+                     "tile_n": p["tile_n"], "bytes": by, "us_per_call": round(us_call, 2),
+                     "GBps": round(by / us_call / 1e3, 1), "TFLOPs": round(2.0 * M * Nn * Kk / us_call / 1e6, 2),
+                     "frac_hbm_peak": round(by / us_call / 1e3 / HBM_PEAK_GBPS, 4),
+                     "frac_read_ceiling": round(by / us_call / 1e3 / ceiling, 4)})
+
+    fp16_case("C1 fastgemv", "fastgemv", 1, 4096, 4096, capi.FG_W_NK, 1001)
+    fp16_case("C2 edgemm", "edgemm_m8n128k64x4", 8, 4096, 11008, capi.FG_W_KN, 1002)
+    fp16_case("C2 edgemm_bt", "edgemm_m8n128k64x4_bt", 8, 4096, 11008, capi.FG_W_NK, 1002)
+    fp16_case("C3a flat up-projection", "gemm_m8n128k64x4_bt", 16, 3072, 12288, capi.FG_W_NK, 1003)
+    fp16_case("C3b flat down-projection", "gemm_m8n128k64x4_bt", 16, 12288, 3072, capi.FG_W_NK, 1003)
+    for ki, kn in enumerate((1024, 4096, 8192, 16384)):
+        for mi, M in enumerate((1, 2, 4, 8, 16)):
+            seed = 2000 + 16 * ki + mi
+            fp16_case("C5 sweep", "edgemm_m8n128k64x4_bt", M, kn, kn, capi.FG_W_NK, seed)
+            fp16_case("C5 sweep", "edgemm_m8n128k64x4", M, kn, kn, capi.FG_W_KN, seed)
+
+    # C4: int8 weights, fp16 activations, per-channel scale
+    g = torch.Generator(device=dev).manual_seed(1004)
+    Kk = Nn = 8192
+    wq = [torch.randint(-127, 128, (Nn, Kk), device=dev, generator=g, dtype=torch.int8) for _ in range(10)]
+    x = torch.randn((1, Kk), device=dev, generator=g).half()
+    scale = (torch.rand(Nn, device=dev, generator=g) * 0.009 + 0.001).half()
+    y = torch.empty(Nn, dtype=torch.half, device=dev)
+    us_i8 = time_us(lambda i: sg.fastgemv_int8(wq[i % 10], x, y, scale=scale))
+    by = Kk * Nn + 2 * Kk + 2 * Nn + 2 * Nn
+    us_f16 = next(r["us_per_call"] for r in rows if r["config"] == "C5 sweep" and r["M"] == 1 and r["K"] == 8192
+                  and r["w_layout"] == "[N,K]")
+    rows.append({"config": "C4 int8 fastgemv", "op": "fastgemv_int8", "M": 1, "K": Kk, "N": Nn, "w_layout": "[N,K] int8",
+                 "seed": 1004, "kernel": "w8a16", "splitk": 1, "bytes": by, "us_per_call": round(us_i8, 2),
+                 "GBps": round(by / us_i8 / 1e3, 1), "frac_hbm_peak": round(by / us_i8 / 1e3 / HBM_PEAK_GBPS, 4),
+                 "frac_read_ceiling": round(by / us_i8 / 1e3 / ceiling, 4),
+                 "weights_per_ns": round(Kk * Nn / us_i8 / 1e3, 3),
+                 "fp16_M1_weights_per_ns": round(Kk * Nn / us_f16 / 1e3, 3),
+                 "weight_throughput_vs_fp16": round(us_f16 / us_i8, 3)})
+    return {"sweep": rows, "read_ceiling_GBps": round(ceiling, 1), "hbm_peak_GBps": HBM_PEAK_GBPS,
+            "steps": steps, "warmup": warmup, "data": "synthetic", "dtype": "f16",
+            "device": torch.cuda.get_device_name(0)}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -69,6 +156,10 @@ def main() -> int:
     ap.add_argument("--calibrate-traffic", action="store_true",
                     help="only run kernels of known traffic (1 GiB read probe, 256 MiB device copy) for "
                          "scaling rocprofv3's FETCH_SIZE / WRITE_SIZE counters, then exit")
+    ap.add_argument("--sweep", action="store_true",
+                    help="instead of the headline step, time every benchmark configuration (the fastgemv, "
+                         "edgemm, flat-GEMM and int8 shapes and the M x K=N shape sweep on both weight "
+                         "layouts) and print one JSON object with the plan and roofline figures per shape")
     ap.add_argument("--cpu-repeats", type=int, default=8, help="repetitions of the step on the CPU oracle (0 = skip)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -106,6 +197,10 @@ def main() -> int:
         print(json.dumps({"calibration": {"stream_read_kernel": {"read_bytes": 1 << 30, "write_bytes": 0, "launches": 5},
                                           "device_copy_kernel": {"read_bytes": 256 << 20, "write_bytes": 256 << 20,
                                                                  "launches": 5}}}))
+        return 0
+
+    if args.sweep:
+        print(json.dumps(run_sweep(torch, sg, capi, dev, args.steps, args.warmup)))
         return 0
 
     # ---- synthetic inputs, seeded on the CPU so the CPU baseline sees the same bits ----------

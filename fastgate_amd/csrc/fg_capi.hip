@@ -98,6 +98,8 @@ int finish_plan(int M, int N, int K, fg_plan_t* p) {
   p->block = 64 * p->waves;
   if (p->splitk > 1) {
     if ((long long)p->grid_x * p->grid_y > kWsMaxTiles) p->fused = 0;
+    // the in-launch completion addresses the partials with 32-bit byte offsets
+    if ((unsigned long long)p->splitk * M * N * sizeof(float) > 0x7fffffffull) p->fused = 0;
     p->workspace_bytes = kWsHeaderBytes + (size_t)p->splitk * M * N * sizeof(float);
   } else {
     p->workspace_bytes = 0;
@@ -108,10 +110,12 @@ int finish_plan(int M, int N, int K, fg_plan_t* p) {
 int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
   std::memset(p, 0, sizeof(*p));
   p->stream_w = 1;
-  // Completing split-K inside the launch needs agent-scope fences, which write back and
-  // invalidate the per-XCD L2s: measured 8x slower than the second-pass kernel on MI355X
-  // (K = N = 8192, M = 16, S = 8: 205 us against 26 us).  The planner never picks it.
-  p->fused = 0;
+  // Split-K can finish inside the launch (the last workgroup of a tile sums the partials) or
+  // in a second kernel.  Measured at K = N = 8192, S = 4 (us per call, second kernel / in-launch):
+  // [K,N] M=1 26.4 / 25.7, M=8 26.2 / 25.5, M=16 26.4 / 27.0; [N,K] transposing kernel M=8
+  // 26.2 / 25.6, M=16 27.4 / 27.8.  Either way the dependent tail costs 3-4 us; in-launch wins
+  // while the partials of a tile are small.
+  p->fused = M <= 8;
   int items = 1;
   bool interleaved = true;  // waves and splits interleave over K (not the transposing kernel)
   if (w_layout == FG_W_NK) {

@@ -115,6 +115,27 @@ __device__ __forceinline__ float load_partial(const float* p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// 16-byte forms of the same two accesses (HIP has no 16-byte atomics): raw buffer accesses on
+// the partials buffer with the agent-scope cache policy bit (sc1) -- the encoding the 4-byte
+// agent-scope atomics above compile to, four columns per instruction instead of one.  `idx` is
+// the element index into `base`, a multiple of 4; the buffer is at most 2 GiB.
+constexpr int kCachePolicyAgent = 16;  // sc1
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t partials_rsrc(const float* base) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(base), 0, 0x7fffffff, 0x00020000);
+}
+__device__ __forceinline__ void store_partial4(float* base, size_t idx, float4_t v, bool coherent) {
+  if (coherent) {
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), partials_rsrc(base),
+                                           (int)(idx * 4), 0, kCachePolicyAgent);
+  } else {
+    *reinterpret_cast<float4_t*>(base + idx) = v;
+  }
+}
+__device__ __forceinline__ float4_t load_partial4(const float* base, size_t idx) {
+  return __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(
+                                          partials_rsrc(base), (int)(idx * 4), 0, kCachePolicyAgent));
+}
+
 __device__ __forceinline__ bool splitk_last_arriver(int* counter, int S) {
   __shared__ int s_last;
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // partial stores have completed
@@ -141,10 +162,8 @@ __device__ __forceinline__ void splitk_reduce_tile(const float* part, half_t* C,
     const int m = m0 + e / nq, n = n0 + (e % nq) * 4;
     if (m >= M) continue;
     const size_t off = (size_t)m * N + n;
-    float sum[4] = {0.f, 0.f, 0.f, 0.f};
-    for (int z = 0; z < S; ++z)
-#pragma unroll
-      for (int k = 0; k < 4; ++k) sum[k] += load_partial(part + (size_t)z * MN + off + k);
+    float4_t sum = {0.f, 0.f, 0.f, 0.f};
+    for (int z = 0; z < S; ++z) sum += load_partial4(part, (size_t)z * MN + off);
     half4v* c = reinterpret_cast<half4v*>(C + off);
     if (accumulate) {
       const half4v old = *c;

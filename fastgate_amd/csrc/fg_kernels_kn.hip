@@ -115,14 +115,9 @@ __global__ __launch_bounds__(256) void kn_mfma_kernel(const half_t* __restrict__
         for (int i = 0; i < 8; ++i) out[i] = static_cast<half_t>(sum[i]);
         *reinterpret_cast<half8_t*>(c) = out;
       } else {
-        float* o = ws + ((size_t)blockIdx.z * M + mg) * N + n0 + c0;
-        if (counters != nullptr) {
-#pragma unroll
-          for (int i = 0; i < 8; ++i) store_partial(o + i, sum[i], true);
-        } else {
-          *reinterpret_cast<float4_t*>(o) = float4_t{sum[0], sum[1], sum[2], sum[3]};
-          *reinterpret_cast<float4_t*>(o + 4) = float4_t{sum[4], sum[5], sum[6], sum[7]};
-        }
+        const size_t o = ((size_t)blockIdx.z * M + mg) * N + n0 + c0;
+        store_partial4(ws, o, float4_t{sum[0], sum[1], sum[2], sum[3]}, counters != nullptr);
+        store_partial4(ws, o + 4, float4_t{sum[4], sum[5], sum[6], sum[7]}, counters != nullptr);
       }
     }
   }
