@@ -72,6 +72,11 @@ int finish_plan(int M, int N, int K, fg_plan_t* p) {
       p->waves = 4;
       p->splitk = ceil_div(K / 128, p->unroll);  // one workgroup per K slice of unroll*128
       break;
+    case FG_KERNEL_NK_MFMA_R:
+      p->tile_n = 16;
+      p->m_block = 16;
+      p->unroll = 1;
+      break;
     case FG_KERNEL_NK_MFMA_T:
       if (!nk_mfma_t_supported(p->unroll, p->tile_n)) return FG_ERR_UNSUPPORTED;
       p->m_block = 16;
@@ -118,6 +123,7 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
   p->fused = M <= 8;
   int items = 1;
   bool interleaved = true;  // waves and splits interleave over K (not the transposing kernel)
+  bool row_tiles = false;   // the 16-column row-load kernel picks its own split
   if (w_layout == FG_W_NK) {
     // Measured on MI355X at K = N = 8192 (us per call): M=1 dot2 tile 4: 21.6-22.4; M=4 dot2
     // 24.3 / mfma4 22.1; M=8 dot2 27.8 / mfma4 26.2 / mfma16 29.2; M=16 mfma4 36 / mfma16 31.7.
@@ -131,7 +137,9 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
       p->unroll = (K >= 16384 || M > 2) ? 2 : 1;
       items = ceil_div(K / 8, 64 * p->unroll);
       p->stagger = items <= 16;  // at most 4 steps for 4 waves
-    } else if (M <= 4 || (M <= 8 && (splitk > 0 || K < 4096 || N / 16 >= kCUs))) {
+    } else if (M <= 6 || (M <= 8 && K >= 16384)) {
+      // (M = 5 at K = N = 8192: 22.9 us against 24.6 for the row-load kernel; M = 8: 25.6 / 24.1;
+      //  K = N = 16384, M = 8: 77.9 / 80.7)
       p->kernel = FG_KERNEL_NK_MFMA4;
       p->m_block = M <= 4 ? 4 : 8;
       if (K >= 16384) {
@@ -143,6 +151,17 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
         p->tile_n = 16, p->unroll = 1;
       }
       items = ceil_div(K / 128, p->unroll);
+    } else if (M <= 8 || N / 16 >= kCUs) {
+      // 16-column tiles, weights and activations as contiguous row pieces through LDS.  Measured
+      // against the kernels below (us): K = N = 8192 M=8 24.1 / 25.6, M=16 25.8 / 27.3;
+      // K = N = 16384 M=16 85 / 92; K=3072 N=12288 M=16 17.7 / 21.0; K=4096 N=11008 M=8 17.7 / 20.1.
+      // Few tiles (N < 4096) only pay off for M <= 8, with a split that gives >= 512 workgroups.
+      p->kernel = FG_KERNEL_NK_MFMA_R;
+      p->m_block = 16;
+      p->tile_n = 16;
+      p->unroll = 1;
+      items = ceil_div(K, 256);
+      row_tiles = true;
     } else if (splitk > 0) {
       // a caller-chosen split-K factor only exists for the K-interleaved kernels
       p->kernel = FG_KERNEL_NK_MFMA;
@@ -179,9 +198,9 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
       p->splitk = splitk;
     } else if (w_layout == FG_W_KN) {
       // [K,N] tiles are 128 columns wide, so the grid needs split-K to cover the chip: the
-      // factor that brings tiles*S closest to one workgroup per CU, none for tiny weights.
+      // factor that brings tiles*S closest to one workgroup per CU.
       int best = 1;
-      if ((size_t)N * K >= ((size_t)2 << 20)) {
+      if ((size_t)N * K >= ((size_t)1 << 18)) {  // 1024 x 1024: 7.7 us with S = 8 against 9.0 without
         double best_ratio = 1e30;
         for (int S = 1; S <= 16; S *= 2) {
           if (items / (p->waves * S) < 1) break;
@@ -194,6 +213,10 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
         }
       }
       p->splitk = best;
+    } else if (row_tiles) {
+      int S = tiles >= kCUs ? 1 : ceil_div(2 * kCUs, tiles);
+      while (S > 1 && items / (p->waves * S) < 2) --S;  // keep two bands per wave
+      p->splitk = S;
     } else {
       p->splitk = pick_splitk(tiles, p->waves, items, M, N, K, kCUs);
     }
@@ -226,6 +249,7 @@ int run_gemm(const void* A, const void* W, void* C, int M, int N, int K, int acc
     case FG_KERNEL_NK_MFMA4: ok = launch_nk_mfma4(p, a, s); break;
     case FG_KERNEL_NK_MFMA4S: ok = launch_nk_mfma4s(p, a, s); break;
     case FG_KERNEL_NK_MFMA_T: ok = launch_nk_mfma_t(p, a, s); break;
+    case FG_KERNEL_NK_MFMA_R: ok = launch_nk_mfma_r(p, a, s); break;
     case FG_KERNEL_KN_DOT2: ok = launch_kn_dot2(p, a, s); break;
     case FG_KERNEL_KN_MFMA: ok = launch_kn_mfma(p, a, s); break;
     default: break;
@@ -242,7 +266,7 @@ int run_gemm(const void* A, const void* W, void* C, int M, int N, int K, int acc
 bool is_nk(int kernel) {
   return kernel == FG_KERNEL_NK_DOT2 || kernel == FG_KERNEL_NK_MFMA ||
          kernel == FG_KERNEL_NK_MFMA4 || kernel == FG_KERNEL_NK_MFMA4S ||
-         kernel == FG_KERNEL_NK_MFMA_T;
+         kernel == FG_KERNEL_NK_MFMA_T || kernel == FG_KERNEL_NK_MFMA_R;
 }
 bool is_kn(int kernel) { return kernel == FG_KERNEL_KN_DOT2 || kernel == FG_KERNEL_KN_MFMA; }
 

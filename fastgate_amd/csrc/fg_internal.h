@@ -36,6 +36,7 @@ bool launch_nk_mfma(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
 bool launch_nk_mfma4(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
 bool launch_nk_mfma4s(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
 bool launch_nk_mfma_t(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
+bool launch_nk_mfma_r(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
 bool launch_kn_dot2(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
 bool launch_kn_mfma(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
 

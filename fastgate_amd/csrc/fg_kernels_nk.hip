@@ -505,6 +505,124 @@ __global__ __launch_bounds__(256) void nk_mfma_t_kernel(const half_t* __restrict
 }
 
 // ---------------------------------------------------------------------------------------
+// MFMA 16x16x32 kernel with row-friendly loads for BOTH operands, no split-K needed.
+// What makes re-reading A expensive is the shape of the loads, not their volume: read as
+// 16 rows x 64 B (operand order) or 4 rows x 256 B, a 16-row A costs as much as the weights;
+// read as whole contiguous row pieces it costs under 10 % (a load-only probe with 16 weight rows
+// and 16 activation rows per step: 24.5 us against 22.7 us without the activation rows, at
+// K = N = 8192).  So here a wave loads, per step, a 512-byte band (256 k) of the tile's 16 weight
+// rows and of the A rows -- two rows per instruction, 32 lanes x 16 B each -- parks both in
+// wave-private LDS strips (rows padded to 528 B: conflict-free in both directions) and reads them
+// back in operand order for 8 MFMAs.  The tile is only 16 columns wide, so N/16 workgroups fill
+// the chip without split-K and there is no second pass; the 4 waves of a workgroup interleave
+// over the bands of K and meet in LDS once at the end.  MH = instructions per step for A:
+// 4 covers M <= 8, 8 covers M <= 16.
+// ---------------------------------------------------------------------------------------
+template <int MH, bool FULL>
+__global__ __launch_bounds__(256) void nk_mfma_r_kernel(const half_t* __restrict__ A,
+                                                        const half_t* __restrict__ W,
+                                                        half_t* __restrict__ C,
+                                                        float* __restrict__ ws, int* counters, int M,
+                                                        int N, int K, int flags) {
+  // FULL: K is a multiple of 256 and the bands divide evenly over the waves -- no masks needed.
+  const int accumulate = flags & 1;  // bit 1 of flags selects the start stagger
+  constexpr int RS = 528;            // LDS bytes per staged row: 512 B + 16 B
+  constexpr int WSTRIP = 16 * RS;    // weights of one wave
+  constexpr int ASTRIP = 2 * MH * RS;  // activations of one wave (rows beyond 2*MH read as row 0)
+  constexpr int WAVE_LDS = WSTRIP + ASTRIP;
+  static_assert(4 * WAVE_LDS >= 4 * 256 * (int)sizeof(float), "reduction scratch fits");
+  __shared__ __attribute__((aligned(16))) unsigned char smem[4 * WAVE_LDS];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int nw = blockDim.x >> 6;
+  const int j = lane & 15, g = lane >> 4;   // operand order: row j, 8 k at 8g within a 32-wide unit
+  const int h = lane >> 5, c = lane & 31;   // load order: row 2i+h, 16-byte piece c of the band
+  const int n0 = blockIdx.x * 16;
+  const int m0 = blockIdx.y * 16;
+  const int slots = nw * gridDim.z;
+  const int slot = blockIdx.z * nw + wave;
+  const int nbands = (K + 255) >> 8;  // K % 128 == 0: the last band may be half
+  unsigned char* wstrip = smem + wave * WAVE_LDS;
+  unsigned char* astrip = wstrip + WSTRIP;
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+
+  const half_t* Wp = W + (size_t)(n0 + h) * K + c * 8;
+  const half_t* Ap = A + (size_t)(m0 + h) * K + c * 8;
+  bool arow[MH];
+#pragma unroll
+  for (int i = 0; i < MH; ++i) arow[i] = (m0 + 2 * i + h) < M;
+  // LDS byte offsets: where this lane parks its pieces, and where it reads its operands.  With
+  // an 8-row A strip the MFMA rows 8..15 re-read rows 0..7; their results are never stored.
+  const int st_off = h * RS + c * 16;
+  const int ldw_off = j * RS + g * 16;
+  const int lda_off = (MH == 8 ? j : (j & 7)) * RS + g * 16;
+
+  auto load_band = [&](int band, u32x4(&w)[8], u32x4(&a)[MH]) {
+    const bool ok = FULL || (band < nbands && (band * 256 + c * 8) < K);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) w[i] = ok ? load16<true>(Wp + (size_t)(2 * i) * K + (size_t)band * 256) : zero;
+#pragma unroll
+    for (int i = 0; i < MH; ++i)
+      a[i] = (ok && arow[i]) ? load16<false>(Ap + (size_t)(2 * i) * K + (size_t)band * 256) : zero;
+  };
+  float4_t acc = {0.f, 0.f, 0.f, 0.f};
+  auto multiply = [&](const u32x4(&w)[8], const u32x4(&a)[MH]) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4*>(wstrip + st_off + 2 * i * RS) = w[i];
+#pragma unroll
+    for (int i = 0; i < MH; ++i) *reinterpret_cast<u32x4*>(astrip + st_off + 2 * i * RS) = a[i];
+    wave_lds_sync();
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const u32x4 av = *reinterpret_cast<const u32x4*>(astrip + lda_off + u * 64);
+      const u32x4 bv = *reinterpret_cast<const u32x4*>(wstrip + ldw_off + u * 64);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(av), as_half8(bv), acc, 0, 0, 0);
+    }
+    wave_lds_sync();
+  };
+
+  // Two register sets, alternating: the next band is in flight while this one is multiplied.
+  u32x4 w0[8], w1[8], a0[MH], a1[MH];
+  const int nsteps = (nbands + slots - 1) / slots;
+  int step = stagger_start(nsteps, flags);
+  auto next_band = [&]() {
+    const int band = step * slots + slot;
+    step = step + 1 == nsteps ? 0 : step + 1;
+    return band;
+  };
+  load_band(next_band(), w0, a0);
+  for (int it = 0; it < nsteps; it += 2) {
+    if (it + 1 < nsteps) load_band(next_band(), w1, a1);
+    multiply(w0, a0);
+    if (it + 1 >= nsteps) break;
+    if (it + 2 < nsteps) load_band(next_band(), w0, a0);
+    multiply(w1, a1);
+  }
+
+  // acc[r] = D[m = 4g + r][column j]; the waves' partials meet in LDS
+  __syncthreads();
+  float(*red)[256] = reinterpret_cast<float(*)[256]>(smem);
+#pragma unroll
+  for (int r = 0; r < 4; ++r) red[wave][(4 * g + r) * 16 + j] = acc[r];
+  __syncthreads();
+  for (int e = threadIdx.x; e < 256; e += blockDim.x) {
+    float sum = 0.f;
+    for (int wv = 0; wv < nw; ++wv) sum += red[wv][e];
+    const int mg = m0 + (e >> 4), n = n0 + (e & 15);
+    if ((e >> 4) < 2 * MH && mg < M) {
+      if (gridDim.z == 1) {
+        half_t* cp = C + (size_t)mg * N + n;
+        if (accumulate) sum += static_cast<float>(*cp);
+        *cp = static_cast<half_t>(sum);
+      } else {
+        store_partial(ws + ((size_t)blockIdx.z * M + mg) * N + n, sum, counters != nullptr);
+      }
+    }
+  }
+  finish_splitk<16, 16>(ws, counters, C, M, N, m0, n0, accumulate);
+}
+
+// ---------------------------------------------------------------------------------------
 // Host launchers
 // ---------------------------------------------------------------------------------------
 #define FG_LAUNCH(KERNEL, p, a, s)                                                           \
@@ -760,6 +878,21 @@ bool launch_nk_mfma4s(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
     case 16: return nk_mfma4s_cw<4>(p, a, s);
     default: return false;
   }
+}
+
+bool launch_nk_mfma_r(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
+  if (p.tile_n != 16 || p.m_block != 16) return false;
+  const int slots = p.waves * p.grid_z;
+  const bool full = a.K % 256 == 0 && (a.K / 256) % slots == 0;
+  const bool half_m = a.M <= 8;  // one block row whose A strip needs only 8 rows
+  if (half_m) {
+    if (full) FG_LAUNCH((nk_mfma_r_kernel<4, true>), p, a, s);
+    else FG_LAUNCH((nk_mfma_r_kernel<4, false>), p, a, s);
+  } else {
+    if (full) FG_LAUNCH((nk_mfma_r_kernel<8, true>), p, a, s);
+    else FG_LAUNCH((nk_mfma_r_kernel<8, false>), p, a, s);
+  }
+  return true;
 }
 
 }  // namespace fg
