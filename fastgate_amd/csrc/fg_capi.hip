@@ -75,7 +75,7 @@ int finish_plan(int M, int N, int K, fg_plan_t* p) {
     case FG_KERNEL_NK_MFMA_R:
       p->tile_n = 16;
       p->m_block = 16;
-      p->unroll = 1;
+      if (p->unroll != 1 && p->unroll != 2) return FG_ERR_UNSUPPORTED;
       break;
     case FG_KERNEL_NK_MFMA_T:
       if (!nk_mfma_t_supported(p->unroll, p->tile_n)) return FG_ERR_UNSUPPORTED;
@@ -159,8 +159,11 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
       p->kernel = FG_KERNEL_NK_MFMA_R;
       p->m_block = 16;
       p->tile_n = 16;
-      p->unroll = 1;
-      items = ceil_div(K, 256);
+      // 256-byte bands (more, lighter workgroups per CU) once there are plenty of tiles:
+      // K=3072 N=12288 M=16 16.3 us against 18.3 with 512-byte bands, K=N=8192 M=16 25.4 / 26.0;
+      // with few tiles the wider band wins (K=12288 N=3072 M=8: 18.3 / 21.3).
+      p->unroll = (K < 16384 && (N / 16 >= 2 * kCUs || (M > 8 && N / 16 >= kCUs))) ? 1 : 2;
+      items = ceil_div(K, 128 * p->unroll);
       row_tiles = true;
     } else if (splitk > 0) {
       // a caller-chosen split-K factor only exists for the K-interleaved kernels

@@ -518,62 +518,71 @@ __global__ __launch_bounds__(256) void nk_mfma_t_kernel(const half_t* __restrict
 // over the bands of K and meet in LDS once at the end.  MH = instructions per step for A:
 // 4 covers M <= 8, 8 covers M <= 16.
 // ---------------------------------------------------------------------------------------
-template <int MH, bool FULL>
+template <int AROWS, int BAND, bool FULL>
 __global__ __launch_bounds__(256) void nk_mfma_r_kernel(const half_t* __restrict__ A,
                                                         const half_t* __restrict__ W,
                                                         half_t* __restrict__ C,
                                                         float* __restrict__ ws, int* counters, int M,
                                                         int N, int K, int flags) {
-  // FULL: K is a multiple of 256 and the bands divide evenly over the waves -- no masks needed.
+  // AROWS: rows of A staged per step (8 covers M <= 8, 16 covers M <= 16).  BAND: bytes of K per
+  // row and step (512 or 256).  FULL: K is a multiple of the band and the bands divide evenly
+  // over the waves -- no masks needed.
   const int accumulate = flags & 1;  // bit 1 of flags selects the start stagger
-  constexpr int RS = 528;            // LDS bytes per staged row: 512 B + 16 B
-  constexpr int WSTRIP = 16 * RS;    // weights of one wave
-  constexpr int ASTRIP = 2 * MH * RS;  // activations of one wave (rows beyond 2*MH read as row 0)
+  constexpr int LPR = BAND / 16;       // lanes per row piece
+  constexpr int RPI = 64 / LPR;        // rows per load instruction
+  constexpr int WI = 16 / RPI;         // load instructions per step for the weights
+  constexpr int AI = AROWS / RPI;      // ... for the activations
+  constexpr int UNITS = BAND / 64;     // 32-wide MFMA K units per band
+  constexpr int BK = BAND / 2;         // K positions per band
+  constexpr int RS = BAND + 16;        // LDS bytes per staged row
+  constexpr int WSTRIP = 16 * RS;      // weights of one wave
+  constexpr int ASTRIP = AROWS * RS;   // activations of one wave (rows beyond AROWS re-read row j%8)
   constexpr int WAVE_LDS = WSTRIP + ASTRIP;
   static_assert(4 * WAVE_LDS >= 4 * 256 * (int)sizeof(float), "reduction scratch fits");
   __shared__ __attribute__((aligned(16))) unsigned char smem[4 * WAVE_LDS];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int nw = blockDim.x >> 6;
-  const int j = lane & 15, g = lane >> 4;   // operand order: row j, 8 k at 8g within a 32-wide unit
-  const int h = lane >> 5, c = lane & 31;   // load order: row 2i+h, 16-byte piece c of the band
+  const int j = lane & 15, g = lane >> 4;       // operand order: row j, 8 k at 8g within a unit
+  const int h = lane / LPR, c = lane % LPR;     // load order: row RPI*i + h, 16-byte piece c
   const int n0 = blockIdx.x * 16;
   const int m0 = blockIdx.y * 16;
   const int slots = nw * gridDim.z;
   const int slot = blockIdx.z * nw + wave;
-  const int nbands = (K + 255) >> 8;  // K % 128 == 0: the last band may be half
+  const int nbands = (K + BK - 1) / BK;  // K % 128 == 0: the last band may be partial
   unsigned char* wstrip = smem + wave * WAVE_LDS;
   unsigned char* astrip = wstrip + WSTRIP;
   const u32x4 zero = {0u, 0u, 0u, 0u};
 
   const half_t* Wp = W + (size_t)(n0 + h) * K + c * 8;
   const half_t* Ap = A + (size_t)(m0 + h) * K + c * 8;
-  bool arow[MH];
+  bool arow[AI];
 #pragma unroll
-  for (int i = 0; i < MH; ++i) arow[i] = (m0 + 2 * i + h) < M;
+  for (int i = 0; i < AI; ++i) arow[i] = (m0 + RPI * i + h) < M;
   // LDS byte offsets: where this lane parks its pieces, and where it reads its operands.  With
   // an 8-row A strip the MFMA rows 8..15 re-read rows 0..7; their results are never stored.
   const int st_off = h * RS + c * 16;
   const int ldw_off = j * RS + g * 16;
-  const int lda_off = (MH == 8 ? j : (j & 7)) * RS + g * 16;
+  const int lda_off = (AROWS == 16 ? j : (j & 7)) * RS + g * 16;
 
-  auto load_band = [&](int band, u32x4(&w)[8], u32x4(&a)[MH]) {
-    const bool ok = FULL || (band < nbands && (band * 256 + c * 8) < K);
+  auto load_band = [&](int band, u32x4(&w)[WI], u32x4(&a)[AI]) {
+    const bool ok = FULL || (band < nbands && (band * BK + c * 8) < K);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) w[i] = ok ? load16<true>(Wp + (size_t)(2 * i) * K + (size_t)band * 256) : zero;
+    for (int i = 0; i < WI; ++i)
+      w[i] = ok ? load16<true>(Wp + (size_t)(RPI * i) * K + (size_t)band * BK) : zero;
 #pragma unroll
-    for (int i = 0; i < MH; ++i)
-      a[i] = (ok && arow[i]) ? load16<false>(Ap + (size_t)(2 * i) * K + (size_t)band * 256) : zero;
+    for (int i = 0; i < AI; ++i)
+      a[i] = (ok && arow[i]) ? load16<false>(Ap + (size_t)(RPI * i) * K + (size_t)band * BK) : zero;
   };
   float4_t acc = {0.f, 0.f, 0.f, 0.f};
-  auto multiply = [&](const u32x4(&w)[8], const u32x4(&a)[MH]) {
+  auto multiply = [&](const u32x4(&w)[WI], const u32x4(&a)[AI]) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4*>(wstrip + st_off + 2 * i * RS) = w[i];
+    for (int i = 0; i < WI; ++i) *reinterpret_cast<u32x4*>(wstrip + st_off + RPI * i * RS) = w[i];
 #pragma unroll
-    for (int i = 0; i < MH; ++i) *reinterpret_cast<u32x4*>(astrip + st_off + 2 * i * RS) = a[i];
+    for (int i = 0; i < AI; ++i) *reinterpret_cast<u32x4*>(astrip + st_off + RPI * i * RS) = a[i];
     wave_lds_sync();
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
+    for (int u = 0; u < UNITS; ++u) {
       const u32x4 av = *reinterpret_cast<const u32x4*>(astrip + lda_off + u * 64);
       const u32x4 bv = *reinterpret_cast<const u32x4*>(wstrip + ldw_off + u * 64);
       acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(av), as_half8(bv), acc, 0, 0, 0);
@@ -582,7 +591,7 @@ __global__ __launch_bounds__(256) void nk_mfma_r_kernel(const half_t* __restrict
   };
 
   // Two register sets, alternating: the next band is in flight while this one is multiplied.
-  u32x4 w0[8], w1[8], a0[MH], a1[MH];
+  u32x4 w0[WI], w1[WI], a0[AI], a1[AI];
   const int nsteps = (nbands + slots - 1) / slots;
   int step = stagger_start(nsteps, flags);
   auto next_band = [&]() {
@@ -609,7 +618,7 @@ __global__ __launch_bounds__(256) void nk_mfma_r_kernel(const half_t* __restrict
     float sum = 0.f;
     for (int wv = 0; wv < nw; ++wv) sum += red[wv][e];
     const int mg = m0 + (e >> 4), n = n0 + (e & 15);
-    if ((e >> 4) < 2 * MH && mg < M) {
+    if ((e >> 4) < AROWS && mg < M) {
       if (gridDim.z == 1) {
         half_t* cp = C + (size_t)mg * N + n;
         if (accumulate) sum += static_cast<float>(*cp);
@@ -880,17 +889,27 @@ bool launch_nk_mfma4s(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
   }
 }
 
+template <int AROWS, int BAND>
+static void nk_mfma_r_go(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
+  const int slots = p.waves * p.grid_z;
+  const int bk = BAND / 2;
+  const bool full = a.K % bk == 0 && (a.K / bk) % slots == 0;
+  if (full) FG_LAUNCH((nk_mfma_r_kernel<AROWS, BAND, true>), p, a, s);
+  else FG_LAUNCH((nk_mfma_r_kernel<AROWS, BAND, false>), p, a, s);
+}
+
+// unroll = 2: 512-byte bands (two rows per load instruction); unroll = 1: 256-byte bands.
 bool launch_nk_mfma_r(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
   if (p.tile_n != 16 || p.m_block != 16) return false;
-  const int slots = p.waves * p.grid_z;
-  const bool full = a.K % 256 == 0 && (a.K / 256) % slots == 0;
   const bool half_m = a.M <= 8;  // one block row whose A strip needs only 8 rows
-  if (half_m) {
-    if (full) FG_LAUNCH((nk_mfma_r_kernel<4, true>), p, a, s);
-    else FG_LAUNCH((nk_mfma_r_kernel<4, false>), p, a, s);
+  if (p.unroll == 2) {
+    if (half_m) nk_mfma_r_go<8, 512>(p, a, s);
+    else nk_mfma_r_go<16, 512>(p, a, s);
+  } else if (p.unroll == 1) {
+    if (half_m) nk_mfma_r_go<8, 256>(p, a, s);
+    else nk_mfma_r_go<16, 256>(p, a, s);
   } else {
-    if (full) FG_LAUNCH((nk_mfma_r_kernel<8, true>), p, a, s);
-    else FG_LAUNCH((nk_mfma_r_kernel<8, false>), p, a, s);
+    return false;
   }
   return true;
 }
