@@ -53,7 +53,8 @@ int validate_shape(int M, int N, int K, int w_layout) {
 
 // Fills grid/block/workspace from the tile fields; rejects tiles that were not built.
 int finish_plan(int M, int N, int K, fg_plan_t* p) {
-  if (p->splitk < 1 || p->waves < 1 || p->waves > 4 || (p->waves & (p->waves - 1))) {
+  const int max_waves = (p->kernel == FG_KERNEL_NK_MFMA_R && p->unroll == 1) ? 8 : 4;
+  if (p->splitk < 1 || p->waves < 1 || p->waves > max_waves || (p->waves & (p->waves - 1))) {
     return FG_ERR_INVALID_ARG;
   }
   switch (p->kernel) {
@@ -122,7 +123,6 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
   // while the partials of a tile are small.
   p->fused = M <= 8;
   int items = 1;
-  bool interleaved = true;  // waves and splits interleave over K (not the transposing kernel)
   bool row_tiles = false;   // the 16-column row-load kernel picks its own split
   if (w_layout == FG_W_NK) {
     // Measured on MI355X at K = N = 8192 (us per call): M=1 dot2 tile 4: 21.6-22.4; M=4 dot2
@@ -137,9 +137,8 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
       p->unroll = (K >= 16384 || M > 2) ? 2 : 1;
       items = ceil_div(K / 8, 64 * p->unroll);
       p->stagger = items <= 16;  // at most 4 steps for 4 waves
-    } else if (M <= 6 || (M <= 8 && K >= 16384)) {
-      // (M = 5 at K = N = 8192: 22.9 us against 24.6 for the row-load kernel; M = 8: 25.6 / 24.1;
-      //  K = N = 16384, M = 8: 77.9 / 80.7)
+    } else if (M <= 4 || (M <= 8 && K >= 16384)) {
+      // (K = N = 16384, M = 8: 77.5 us against 78.9 for the row-load kernel)
       p->kernel = FG_KERNEL_NK_MFMA4;
       p->m_block = M <= 4 ? 4 : 8;
       if (K >= 16384) {
@@ -151,36 +150,18 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
         p->tile_n = 16, p->unroll = 1;
       }
       items = ceil_div(K / 128, p->unroll);
-    } else if (M <= 8 || N / 16 >= kCUs) {
-      // 16-column tiles, weights and activations as contiguous row pieces through LDS.  Measured
-      // against the kernels below (us): K = N = 8192 M=8 24.1 / 25.6, M=16 25.8 / 27.3;
-      // K = N = 16384 M=16 85 / 92; K=3072 N=12288 M=16 17.7 / 21.0; K=4096 N=11008 M=8 17.7 / 20.1.
-      // Few tiles (N < 4096) only pay off for M <= 8, with a split that gives >= 512 workgroups.
+    } else {
+      // M >= 5: 16-column tiles, weights and activations as contiguous row pieces through LDS,
+      // 8 waves on 256-byte bands.  Measured against the best of the other [N,K] kernels (us):
+      // K = N = 8192 M=8 23.2 / 25.6, M=16 24.6 / 27.3; K=3072 N=12288 M=16 15.6 / 21.0;
+      // K=12288 N=3072 M=16 19.1 / 20.3; K = N = 4096 M=8 7.8 / 9.5; K=4096 N=11008 M=8 16.5 / 20.1.
+      // At K = 16384 four waves on 512-byte bands are level or slightly ahead (M=16 84.3 / 85.8).
       p->kernel = FG_KERNEL_NK_MFMA_R;
       p->m_block = 16;
       p->tile_n = 16;
-      // 256-byte bands (more, lighter workgroups per CU) once there are plenty of tiles:
-      // K=3072 N=12288 M=16 16.3 us against 18.3 with 512-byte bands, K=N=8192 M=16 25.4 / 26.0;
-      // with few tiles the wider band wins (K=12288 N=3072 M=8: 18.3 / 21.3).
-      p->unroll = (K < 16384 && (N / 16 >= 2 * kCUs || (M > 8 && N / 16 >= kCUs))) ? 1 : 2;
+      p->unroll = K >= 16384 ? 2 : 1;
       items = ceil_div(K, 128 * p->unroll);
       row_tiles = true;
-    } else if (splitk > 0) {
-      // a caller-chosen split-K factor only exists for the K-interleaved kernels
-      p->kernel = FG_KERNEL_NK_MFMA;
-      p->m_block = 16;
-      p->tile_n = (N / 32 >= kCUs) ? 32 : 16;
-      p->unroll = p->tile_n == 32 ? 4 : 2;
-      if (K / 32 < 4 * p->unroll) p->unroll = 1;
-      items = ceil_div(K / 32, p->unroll);
-    } else {
-      // M = 9..16 (and 5..8 for mid-sized K): 16x16x32 MFMA behind the LDS transpose
-      // (K = N = 8192, M = 16: 27.6 us against 31.7 for the direct 16x16x32 kernel)
-      p->kernel = FG_KERNEL_NK_MFMA_T;
-      p->m_block = 16;
-      p->unroll = 16;
-      p->tile_n = (N / 128) * nk_mfma_t_slices(K) >= kCUs / 2 ? 128 : 32;
-      interleaved = false;
     }
   } else {
     if (M <= 2) {
@@ -194,8 +175,8 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
     p->unroll = (p->kernel == FG_KERNEL_KN_DOT2 && K >= 2048) ? 2 : 1;
     items = ceil_div(K / 32, p->unroll);
   }
-  if (interleaved) {
-    p->waves = pick_waves(items);
+  {
+    p->waves = (row_tiles && p->unroll == 1 && items >= 16) ? 8 : pick_waves(items);
     const int tiles = (N / p->tile_n) * ceil_div(M, p->m_block);
     if (splitk > 0) {
       p->splitk = splitk;
@@ -217,15 +198,13 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
       }
       p->splitk = best;
     } else if (row_tiles) {
-      int S = tiles >= kCUs ? 1 : ceil_div(2 * kCUs, tiles);
+      // (K=12288 N=3072, 192 tiles, M=8: 16.0 us unsplit against 19.3 with S = 3)
+      int S = tiles >= kCUs / 2 ? 1 : ceil_div(kCUs, tiles);
       while (S > 1 && items / (p->waves * S) < 2) --S;  // keep two bands per wave
       p->splitk = S;
     } else {
       p->splitk = pick_splitk(tiles, p->waves, items, M, N, K, kCUs);
     }
-  } else {
-    p->waves = 4;
-    p->splitk = 1;  // finish_plan derives it from K
   }
   return finish_plan(M, N, K, p);
 }

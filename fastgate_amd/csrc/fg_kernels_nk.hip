@@ -518,8 +518,8 @@ __global__ __launch_bounds__(256) void nk_mfma_t_kernel(const half_t* __restrict
 // over the bands of K and meet in LDS once at the end.  MH = instructions per step for A:
 // 4 covers M <= 8, 8 covers M <= 16.
 // ---------------------------------------------------------------------------------------
-template <int AROWS, int BAND, bool FULL>
-__global__ __launch_bounds__(256) void nk_mfma_r_kernel(const half_t* __restrict__ A,
+template <int AROWS, int BAND, bool FULL, int NW>
+__global__ __launch_bounds__(64 * NW) void nk_mfma_r_kernel(const half_t* __restrict__ A,
                                                         const half_t* __restrict__ W,
                                                         half_t* __restrict__ C,
                                                         float* __restrict__ ws, int* counters, int M,
@@ -538,8 +538,8 @@ __global__ __launch_bounds__(256) void nk_mfma_r_kernel(const half_t* __restrict
   constexpr int WSTRIP = 16 * RS;      // weights of one wave
   constexpr int ASTRIP = AROWS * RS;   // activations of one wave (rows beyond AROWS re-read row j%8)
   constexpr int WAVE_LDS = WSTRIP + ASTRIP;
-  static_assert(4 * WAVE_LDS >= 4 * 256 * (int)sizeof(float), "reduction scratch fits");
-  __shared__ __attribute__((aligned(16))) unsigned char smem[4 * WAVE_LDS];
+  static_assert(WAVE_LDS >= 256 * (int)sizeof(float), "reduction scratch fits");
+  __shared__ __attribute__((aligned(16))) unsigned char smem[NW * WAVE_LDS];  // NW = most waves
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int nw = blockDim.x >> 6;
@@ -894,13 +894,21 @@ static void nk_mfma_r_go(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
   const int slots = p.waves * p.grid_z;
   const int bk = BAND / 2;
   const bool full = a.K % bk == 0 && (a.K / bk) % slots == 0;
-  if (full) FG_LAUNCH((nk_mfma_r_kernel<AROWS, BAND, true>), p, a, s);
-  else FG_LAUNCH((nk_mfma_r_kernel<AROWS, BAND, false>), p, a, s);
+  if constexpr (BAND == 256) {
+    if (p.waves == 8) {
+      if (full) FG_LAUNCH((nk_mfma_r_kernel<AROWS, BAND, true, 8>), p, a, s);
+      else FG_LAUNCH((nk_mfma_r_kernel<AROWS, BAND, false, 8>), p, a, s);
+      return;
+    }
+  }
+  if (full) FG_LAUNCH((nk_mfma_r_kernel<AROWS, BAND, true, 4>), p, a, s);
+  else FG_LAUNCH((nk_mfma_r_kernel<AROWS, BAND, false, 4>), p, a, s);
 }
 
 // unroll = 2: 512-byte bands (two rows per load instruction); unroll = 1: 256-byte bands.
 bool launch_nk_mfma_r(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
   if (p.tile_n != 16 || p.m_block != 16) return false;
+  if (p.waves > 4 && !(p.waves == 8 && p.unroll == 1)) return false;
   const bool half_m = a.M <= 8;  // one block row whose A strip needs only 8 rows
   if (p.unroll == 2) {
     if (half_m) nk_mfma_r_go<8, 512>(p, a, s);
