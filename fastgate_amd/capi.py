@@ -29,10 +29,9 @@ FG_KERNEL_NK_MFMA = 2
 FG_KERNEL_KN_DOT2 = 3
 FG_KERNEL_KN_MFMA = 4
 FG_KERNEL_NK_MFMA4 = 5
-FG_KERNEL_NK_MFMA4S = 6
 FG_KERNEL_NK_MFMA_T = 7
 FG_KERNEL_NK_MFMA_R = 8
-KERNEL_NAMES = {1: "nk_dot2", 2: "nk_mfma", 3: "kn_dot2", 4: "kn_mfma", 5: "nk_mfma4", 6: "nk_mfma4s", 7: "nk_mfma_t", 8: "nk_mfma_r"}
+KERNEL_NAMES = {1: "nk_dot2", 2: "nk_mfma", 3: "kn_dot2", 4: "kn_mfma", 5: "nk_mfma4", 7: "nk_mfma_t", 8: "nk_mfma_r"}
 
 # Every symbol include/fastgate.h declares.
 EXPORTS = (

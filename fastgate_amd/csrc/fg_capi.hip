@@ -68,11 +68,6 @@ int finish_plan(int M, int N, int K, fg_plan_t* p) {
     case FG_KERNEL_NK_MFMA4:
       if (!nk_mfma4_supported(p->m_block, p->tile_n, p->unroll)) return FG_ERR_UNSUPPORTED;
       break;
-    case FG_KERNEL_NK_MFMA4S:
-      if (!nk_mfma4s_supported(p->m_block, p->tile_n, p->unroll)) return FG_ERR_UNSUPPORTED;
-      p->waves = 4;
-      p->splitk = ceil_div(K / 128, p->unroll);  // one workgroup per K slice of unroll*128
-      break;
     case FG_KERNEL_NK_MFMA_R:
       p->tile_n = 16;
       p->m_block = 16;
@@ -229,7 +224,6 @@ int run_gemm(const void* A, const void* W, void* C, int M, int N, int K, int acc
     case FG_KERNEL_NK_DOT2: ok = launch_nk_dot2(p, a, s); break;
     case FG_KERNEL_NK_MFMA: ok = launch_nk_mfma(p, a, s); break;
     case FG_KERNEL_NK_MFMA4: ok = launch_nk_mfma4(p, a, s); break;
-    case FG_KERNEL_NK_MFMA4S: ok = launch_nk_mfma4s(p, a, s); break;
     case FG_KERNEL_NK_MFMA_T: ok = launch_nk_mfma_t(p, a, s); break;
     case FG_KERNEL_NK_MFMA_R: ok = launch_nk_mfma_r(p, a, s); break;
     case FG_KERNEL_KN_DOT2: ok = launch_kn_dot2(p, a, s); break;
@@ -247,7 +241,7 @@ int run_gemm(const void* A, const void* W, void* C, int M, int N, int K, int acc
 
 bool is_nk(int kernel) {
   return kernel == FG_KERNEL_NK_DOT2 || kernel == FG_KERNEL_NK_MFMA ||
-         kernel == FG_KERNEL_NK_MFMA4 || kernel == FG_KERNEL_NK_MFMA4S ||
+         kernel == FG_KERNEL_NK_MFMA4 ||
          kernel == FG_KERNEL_NK_MFMA_T || kernel == FG_KERNEL_NK_MFMA_R;
 }
 bool is_kn(int kernel) { return kernel == FG_KERNEL_KN_DOT2 || kernel == FG_KERNEL_KN_MFMA; }

@@ -25,7 +25,6 @@ struct GemmArgs {
 bool nk_dot2_supported(int m_block, int tile_n, int unroll);
 bool nk_mfma_supported(int tile_n, int unroll);
 bool nk_mfma4_supported(int m_block, int tile_n, int unroll);
-bool nk_mfma4s_supported(int m_block, int tile_n, int chunks);
 bool nk_mfma_t_supported(int rows, int tile_n);
 int nk_mfma_t_slices(int K);
 bool kn_dot2_supported(int m_block, int unroll);
@@ -34,7 +33,6 @@ bool kn_mfma_supported(int unroll);
 bool launch_nk_dot2(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
 bool launch_nk_mfma(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
 bool launch_nk_mfma4(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
-bool launch_nk_mfma4s(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
 bool launch_nk_mfma_t(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
 bool launch_nk_mfma_r(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
 bool launch_kn_dot2(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);

@@ -183,7 +183,7 @@ __global__ __launch_bounds__(256) void nk_mfma_kernel(const half_t* __restrict__
 }
 
 // ---------------------------------------------------------------------------------------
-// MFMA 4x4x4 kernels.  v_mfma_f32_4x4x4_16B_f16 multiplies 16 independent 4x4x4 blocks; here
+// MFMA 4x4x4 kernel.  v_mfma_f32_4x4x4_16B_f16 multiplies 16 independent 4x4x4 blocks; here
 // block b = lane/4 owns the 8 k positions 128*chunk + 8b..8b+7 (two MFMAs of 4 k each) and its
 // four lanes j = lane%4 own four neighbouring weight rows.  One 16-byte load instruction of a
 // wave therefore reads 4 weight rows x 256 contiguous bytes -- the same row-friendly pattern as
@@ -197,8 +197,9 @@ typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ half4_t lo4(u32x4 v) { return __builtin_bit_cast(half4_t, u32x2{v.x, v.y}); }
 __device__ __forceinline__ half4_t hi4(u32x4 v) { return __builtin_bit_cast(half4_t, u32x2{v.z, v.w}); }
 
-// Interleaved variant: the waves of a workgroup interleave over K, every wave covers all
-// 4*R4 columns of the tile and re-reads its slice of A from L2.  Best for M <= 8.
+// The waves of a workgroup interleave over K, every wave covers all 4*R4 columns of the tile
+// and re-reads its slice of A from L2 (4 rows x 256 B per instruction, which is what makes it
+// lose to the row-load kernel below once M exceeds 4).
 template <int MG, int R4, int U, bool STREAM>
 __global__ __launch_bounds__(256) void nk_mfma4_kernel(const half_t* __restrict__ A,
                                                        const half_t* __restrict__ W,
@@ -288,112 +289,6 @@ __global__ __launch_bounds__(256) void nk_mfma4_kernel(const half_t* __restrict_
     }
   }
   finish_splitk<4 * MG, 4 * R4>(ws, counters, C, M, N, m0, n0, accumulate);
-}
-
-// Sliced variant for M = 8..16.  Re-reading A per 4*R4 columns costs as much L1 traffic as the
-// weights themselves once M reaches 16, so here a workgroup owns a K slice of CW*128 positions
-// (blockIdx.z selects it), stages the 4*MG x slice panel of A in LDS once, and its waves split
-// the TN columns of the tile: wave w walks RG = TN/16 groups of 4 rows, each group CW loads of
-// 4 rows x 256 B (4 rows x CW*256 B contiguous), with the next group's loads issued before
-// the current group's MFMAs.  A operands come from LDS (ds_read_b128).  gridDim.z = number of
-// K slices; the slices meet through the split-K workspace.
-template <int MG, int CW, int RG, bool STREAM>
-__global__ __launch_bounds__(256) void nk_mfma4s_kernel(const half_t* __restrict__ A,
-                                                        const half_t* __restrict__ W,
-                                                        half_t* __restrict__ C,
-                                                        float* __restrict__ ws, int* counters, int M,
-                                                        int N, int K, int flags) {
-  const int accumulate = flags & 1;  // bit 1 of flags selects the start stagger
-  constexpr int TN = 16 * RG;     // columns per workgroup (4 waves x RG x 4)
-  constexpr int AROWB = CW * 256;  // bytes per LDS row of A
-  // LDS: A panel [4*MG][CW*256 B], then red[4 waves][4 dpp rows][MG*16] floats.  The 16-byte
-  // pieces of A row r are stored at piece ^ ((r&3) << 2): the four rows j a ds_read_b128 touches
-  // then fall on different banks without padding.
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  unsigned char* a_lds = smem;
-  float(*red)[4][MG * 16] = reinterpret_cast<float(*)[4][MG * 16]>(smem + 4 * MG * AROWB);
-  const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
-  const int j = lane & 3, b = lane >> 2;
-  const int n0 = blockIdx.x * TN;
-  const int m0 = blockIdx.y * (4 * MG);
-  const int nchunks = K >> 7;
-  const int c_lo = blockIdx.z * CW;  // first 128-wide K chunk of this slice
-  const u32x4 zero = {0u, 0u, 0u, 0u};
-
-  // Stage A[m0 .. m0+4MG)[c_lo*128 .. +CW*128) in LDS, zero where the row or chunk is absent.
-  for (int e = threadIdx.x; e < 4 * MG * CW * 16; e += 256) {
-    const int row = e / (CW * 16), q = e % (CW * 16);  // q: 16-byte piece within the slice row
-    const int chunk = c_lo + (q >> 4);
-    const bool ok = (m0 + row) < M && chunk < nchunks;
-    const u32x4 v =
-        ok ? load16<false>(A + (size_t)(m0 + row) * K + (size_t)c_lo * 128 + q * 8) : zero;
-    *reinterpret_cast<u32x4*>(a_lds + row * AROWB + ((q ^ ((row & 3) << 2)) << 4)) = v;
-  }
-
-  // Weight loads of the first row group are in flight while A lands in LDS.
-  const half_t* Wp = W + (size_t)(n0 + wave * (4 * RG) + j) * K + (size_t)c_lo * 128 + b * 8;
-  u32x4 wcur[CW], wnxt[CW];
-#pragma unroll
-  for (int c = 0; c < CW; ++c)
-    wcur[c] = (c_lo + c) < nchunks ? load16<STREAM>(Wp + (size_t)c * 128) : zero;
-  __syncthreads();
-
-#pragma unroll
-  for (int rg = 0; rg < RG; ++rg) {
-    if (rg + 1 < RG) {
-#pragma unroll
-      for (int c = 0; c < CW; ++c)
-        wnxt[c] = (c_lo + c) < nchunks
-                      ? load16<STREAM>(Wp + (size_t)(4 * (rg + 1)) * K + (size_t)c * 128)
-                      : zero;
-    }
-    float4_t acc[MG];
-#pragma unroll
-    for (int g = 0; g < MG; ++g) acc[g] = float4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int c = 0; c < CW; ++c) {
-#pragma unroll
-      for (int g = 0; g < MG; ++g) {
-        const u32x4 a = *reinterpret_cast<const u32x4*>(a_lds + (4 * g + j) * AROWB +
-                                                        (((c * 16 + b) ^ (j << 2)) << 4));
-        acc[g] = __builtin_amdgcn_mfma_f32_4x4x4f16(lo4(a), lo4(wcur[c]), acc[g], 0, 0, 0);
-        acc[g] = __builtin_amdgcn_mfma_f32_4x4x4f16(hi4(a), hi4(wcur[c]), acc[g], 0, 0, 0);
-      }
-    }
-    // 16 blocks -> one value: row_ror within the DPP row, the 4 rows through wave-private LDS.
-#pragma unroll
-    for (int g = 0; g < MG; ++g)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        float v = acc[g][i];
-        v += dpp_f32<0x124>(v);
-        v += dpp_f32<0x128>(v);
-        if ((lane & 12) == 0) red[wave][lane >> 4][(g * 4 + i) * 4 + j] = v;
-      }
-    wave_lds_sync();  // red[wave] is private to this wave: ordering only, no s_barrier
-    if (lane < MG * 16) {
-      const float sum =
-          red[wave][0][lane] + red[wave][1][lane] + red[wave][2][lane] + red[wave][3][lane];
-      const int mg = m0 + (lane >> 2), n = n0 + wave * (4 * RG) + 4 * rg + (lane & 3);
-      if (mg < M) {
-        if (gridDim.z == 1) {
-          half_t* c = C + (size_t)mg * N + n;
-          float out = sum;
-          if (accumulate) out += static_cast<float>(*c);
-          *c = static_cast<half_t>(out);
-        } else {
-          store_partial(ws + ((size_t)blockIdx.z * M + mg) * N + n, sum, counters != nullptr);
-        }
-      }
-    }
-    wave_lds_sync();
-    if (rg + 1 < RG) {
-#pragma unroll
-      for (int c = 0; c < CW; ++c) wcur[c] = wnxt[c];
-    }
-  }
-  finish_splitk<4 * MG, TN>(ws, counters, C, M, N, m0, n0, accumulate);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -774,53 +669,6 @@ bool launch_nk_mfma4(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
   }
 }
 
-// Sliced variant: unroll = chunks of 128 K positions per slice (8 or 16), tile_n = 16*RG.
-bool nk_mfma4s_supported(int m_block, int tile_n, int cw) {
-  const bool mg_ok = m_block == 8 || m_block == 12 || m_block == 16;
-  const bool tn_ok = tile_n == 16 || tile_n == 32 || tile_n == 64;
-  return mg_ok && tn_ok && (cw == 8 || cw == 16);
-}
-
-template <int MG, int CW, int RG, bool STREAM>
-static void nk_mfma4s_launch(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
-  constexpr unsigned lds = 4 * MG * CW * 256 + 4 * 4 * MG * 16 * sizeof(float);
-  static bool raised = false;  // more than 64 KB of LDS per workgroup has to be asked for once
-  if (!raised) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&nk_mfma4s_kernel<MG, CW, RG, STREAM>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-    raised = true;
-  }
-  hipLaunchKernelGGL((nk_mfma4s_kernel<MG, CW, RG, STREAM>), dim3(p.grid_x, p.grid_y, p.grid_z),
-                     dim3(256), lds, s, static_cast<const half_t*>(a.A),
-                     static_cast<const half_t*>(a.W), static_cast<half_t*>(a.C), a.ws, a.counters,
-                     a.M, a.N, a.K, a.accumulate);
-}
-
-template <int MG, int CW, int RG>
-static void nk_mfma4s_go(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
-  if (p.stream_w) nk_mfma4s_launch<MG, CW, RG, true>(p, a, s);
-  else nk_mfma4s_launch<MG, CW, RG, false>(p, a, s);
-}
-
-template <int MG, int CW>
-static bool nk_mfma4s_rg(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
-  switch (p.tile_n) {
-    case 16: nk_mfma4s_go<MG, CW, 1>(p, a, s); return true;
-    case 32: nk_mfma4s_go<MG, CW, 2>(p, a, s); return true;
-    case 64: nk_mfma4s_go<MG, CW, 4>(p, a, s); return true;
-    default: return false;
-  }
-}
-
-template <int MG>
-static bool nk_mfma4s_cw(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
-  switch (p.unroll) {
-    case 8: return nk_mfma4s_rg<MG, 8>(p, a, s);
-    case 16: return nk_mfma4s_rg<MG, 16>(p, a, s);
-    default: return false;
-  }
-}
-
 // Transposing variant: unroll = rows per tile (8 or 16), tile_n = rows * T with T in {2,4,8}.
 bool nk_mfma_t_supported(int rows, int tile_n) {
   if (rows != 8 && rows != 16) return false;
@@ -875,16 +723,6 @@ bool launch_nk_mfma_t(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
   switch (p.unroll) {
     case 8: return nk_mfma_t_t<8>(p, a, s);
     case 16: return nk_mfma_t_t<16>(p, a, s);
-    default: return false;
-  }
-}
-
-bool launch_nk_mfma4s(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
-  if (p.block != 256) return false;
-  switch (p.m_block) {
-    case 8: return nk_mfma4s_cw<2>(p, a, s);
-    case 12: return nk_mfma4s_cw<3>(p, a, s);
-    case 16: return nk_mfma4s_cw<4>(p, a, s);
     default: return false;
   }
 }

@@ -51,8 +51,6 @@ enum {
   FG_KERNEL_KN_DOT2 = 3, /* [K,N] weights, 8x8 register transpose + v_dot2_f32_f16       */
   FG_KERNEL_KN_MFMA = 4, /* [K,N] weights, 8x8 register transpose + MFMA                 */
   FG_KERNEL_NK_MFMA4 = 5, /* [N,K] weights, v_mfma_f32_4x4x4_16B_f16: 4 rows x 256 B a load */
-  FG_KERNEL_NK_MFMA4S = 6, /* same instruction; a workgroup owns a K slice of unroll*128, keeps
-                              that slice of A in LDS, its waves split tile_n (16/32/64) columns */
   FG_KERNEL_NK_MFMA_T = 7, /* [N,K] weights, 16x16x32 MFMA fed through a wave-private LDS
                               transpose: loads are `unroll` (8/16) rows x 1 KB, every wave keeps
                               the A operands of its fixed K range in registers               */

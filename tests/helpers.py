@@ -63,7 +63,7 @@ def capi_gemm(A, W, C, w_layout, accumulate=False, splitk=0, plan=None):
         wsb = p.workspace_bytes
     else:
         p = plan
-        # the sliced kernel derives its split from K; leave room for any split up to K/128
+        # the transposing kernel derives its split from K; leave room for any split up to K/128
         wsb = hdr + max(p.splitk, K // 128) * M * N * 4
     ws = None
     if wsb:

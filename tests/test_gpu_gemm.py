@@ -71,27 +71,6 @@ def test_every_instantiation(device, name, layout, kw):
             assert_close_f16(got, ref, "%s M=%d waves=%d S=%d" % (name, M, waves, splitk))
 
 
-@pytest.mark.parametrize("m_block", [8, 12, 16])
-@pytest.mark.parametrize("tile_n", [16, 32, 64])
-@pytest.mark.parametrize("chunks", [8, 16])
-def test_sliced_mfma4_kernel(device, m_block, tile_n, chunks):
-    # K = 2176 = 17 chunks of 128: two or three K slices, the last one ragged
-    N = 384
-    for K in (640, 2176):
-        for M in sorted({1, m_block - 3, m_block, 2 * m_block + 1}):
-            A, W = _case(M, N, K, NK, 40 + M + K)
-            ref, _ = oracle.gemm_f16(A.numpy(), W.numpy(), NK)
-            C0 = normal((M, N), gen(41), 2.0)
-            refa, _ = oracle.gemm_f16(A.numpy(), W.numpy(), NK, C=C0.numpy(), accumulate=True)
-            for fused in (1, 0):
-                kw = dict(kernel=capi.FG_KERNEL_NK_MFMA4S, tile_n=tile_n, m_block=m_block, unroll=chunks, fused=fused)
-                got, p = _run(A, W, NK, device, plan=make_plan(**kw))
-                assert p.splitk == -(-(K // 128) // chunks)
-                assert_close_f16(got, ref, "mfma4s M=%d K=%d fused=%d" % (M, K, fused))
-                got, _ = _run(A, W, NK, device, accumulate=True, C0=C0, plan=make_plan(**kw))
-                assert_close_f16(got, refa, "mfma4s accumulate M=%d K=%d fused=%d" % (M, K, fused))
-
-
 @pytest.mark.parametrize("rows", [8, 16])
 @pytest.mark.parametrize("tiles", [2, 4, 8])
 def test_transposing_mfma_kernel(device, rows, tiles):
