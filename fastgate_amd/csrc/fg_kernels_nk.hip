@@ -413,7 +413,7 @@ __global__ __launch_bounds__(256) void nk_mfma_t_kernel(const half_t* __restrict
 // over the bands of K and meet in LDS once at the end.  MH = instructions per step for A:
 // 4 covers M <= 8, 8 covers M <= 16.
 // ---------------------------------------------------------------------------------------
-template <int AROWS, int BAND, bool FULL, int NW>
+template <int AROWS, int BAND, bool FULL, int NW, int CB>
 __global__ __launch_bounds__(64 * NW) void nk_mfma_r_kernel(const half_t* __restrict__ A,
                                                         const half_t* __restrict__ W,
                                                         half_t* __restrict__ C,
@@ -425,22 +425,22 @@ __global__ __launch_bounds__(64 * NW) void nk_mfma_r_kernel(const half_t* __rest
   const int accumulate = flags & 1;  // bit 1 of flags selects the start stagger
   constexpr int LPR = BAND / 16;       // lanes per row piece
   constexpr int RPI = 64 / LPR;        // rows per load instruction
-  constexpr int WI = 16 / RPI;         // load instructions per step for the weights
+  constexpr int WI = 16 * CB / RPI;    // load instructions per step for the weights (CB blocks of 16 rows)
   constexpr int AI = AROWS / RPI;      // ... for the activations
   constexpr int UNITS = BAND / 64;     // 32-wide MFMA K units per band
   constexpr int BK = BAND / 2;         // K positions per band
   constexpr int RS = BAND + 16;        // LDS bytes per staged row
-  constexpr int WSTRIP = 16 * RS;      // weights of one wave
+  constexpr int WSTRIP = 16 * CB * RS;  // weights of one wave
   constexpr int ASTRIP = AROWS * RS;   // activations of one wave (rows beyond AROWS re-read row j%8)
   constexpr int WAVE_LDS = WSTRIP + ASTRIP;
-  static_assert(WAVE_LDS >= 256 * (int)sizeof(float), "reduction scratch fits");
+  static_assert(WAVE_LDS >= CB * 256 * (int)sizeof(float), "reduction scratch fits");
   __shared__ __attribute__((aligned(16))) unsigned char smem[NW * WAVE_LDS];  // NW = most waves
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int nw = blockDim.x >> 6;
   const int j = lane & 15, g = lane >> 4;       // operand order: row j, 8 k at 8g within a unit
   const int h = lane / LPR, c = lane % LPR;     // load order: row RPI*i + h, 16-byte piece c
-  const int n0 = blockIdx.x * 16;
+  const int n0 = blockIdx.x * (16 * CB);
   const int m0 = blockIdx.y * 16;
   const int slots = nw * gridDim.z;
   const int slot = blockIdx.z * nw + wave;
@@ -469,7 +469,9 @@ __global__ __launch_bounds__(64 * NW) void nk_mfma_r_kernel(const half_t* __rest
     for (int i = 0; i < AI; ++i)
       a[i] = (ok && arow[i]) ? load16<false>(Ap + (size_t)(RPI * i) * K + (size_t)band * BK) : zero;
   };
-  float4_t acc = {0.f, 0.f, 0.f, 0.f};
+  float4_t acc[CB];
+#pragma unroll
+  for (int b = 0; b < CB; ++b) acc[b] = float4_t{0.f, 0.f, 0.f, 0.f};
   auto multiply = [&](const u32x4(&w)[WI], const u32x4(&a)[AI]) {
 #pragma unroll
     for (int i = 0; i < WI; ++i) *reinterpret_cast<u32x4*>(wstrip + st_off + RPI * i * RS) = w[i];
@@ -479,8 +481,11 @@ __global__ __launch_bounds__(64 * NW) void nk_mfma_r_kernel(const half_t* __rest
 #pragma unroll
     for (int u = 0; u < UNITS; ++u) {
       const u32x4 av = *reinterpret_cast<const u32x4*>(astrip + lda_off + u * 64);
-      const u32x4 bv = *reinterpret_cast<const u32x4*>(wstrip + ldw_off + u * 64);
-      acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(av), as_half8(bv), acc, 0, 0, 0);
+#pragma unroll
+      for (int b = 0; b < CB; ++b) {
+        const u32x4 bv = *reinterpret_cast<const u32x4*>(wstrip + b * 16 * RS + ldw_off + u * 64);
+        acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(av), as_half8(bv), acc[b], 0, 0, 0);
+      }
     }
     wave_lds_sync();
   };
@@ -503,17 +508,20 @@ __global__ __launch_bounds__(64 * NW) void nk_mfma_r_kernel(const half_t* __rest
     multiply(w1, a1);
   }
 
-  // acc[r] = D[m = 4g + r][column j]; the waves' partials meet in LDS
+  // acc[b][r] = D[m = 4g + r][column 16b + j]; the waves' partials meet in LDS
+  constexpr int TN = 16 * CB;
   __syncthreads();
-  float(*red)[256] = reinterpret_cast<float(*)[256]>(smem);
+  float(*red)[16 * TN] = reinterpret_cast<float(*)[16 * TN]>(smem);
 #pragma unroll
-  for (int r = 0; r < 4; ++r) red[wave][(4 * g + r) * 16 + j] = acc[r];
+  for (int b = 0; b < CB; ++b)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) red[wave][(4 * g + r) * TN + 16 * b + j] = acc[b][r];
   __syncthreads();
-  for (int e = threadIdx.x; e < 256; e += blockDim.x) {
+  for (int e = threadIdx.x; e < 16 * TN; e += blockDim.x) {
     float sum = 0.f;
     for (int wv = 0; wv < nw; ++wv) sum += red[wv][e];
-    const int mg = m0 + (e >> 4), n = n0 + (e & 15);
-    if ((e >> 4) < AROWS && mg < M) {
+    const int mg = m0 + e / TN, n = n0 + e % TN;
+    if (e / TN < AROWS && mg < M) {
       if (gridDim.z == 1) {
         half_t* cp = C + (size_t)mg * N + n;
         if (accumulate) sum += static_cast<float>(*cp);
@@ -523,7 +531,7 @@ __global__ __launch_bounds__(64 * NW) void nk_mfma_r_kernel(const half_t* __rest
       }
     }
   }
-  finish_splitk<16, 16>(ws, counters, C, M, N, m0, n0, accumulate);
+  finish_splitk<16, TN>(ws, counters, C, M, N, m0, n0, accumulate);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -727,37 +735,45 @@ bool launch_nk_mfma_t(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
   }
 }
 
-template <int AROWS, int BAND>
+template <int AROWS, int BAND, int CB>
 static void nk_mfma_r_go(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
   const int slots = p.waves * p.grid_z;
   const int bk = BAND / 2;
   const bool full = a.K % bk == 0 && (a.K / bk) % slots == 0;
   if constexpr (BAND == 256) {
     if (p.waves == 8) {
-      if (full) FG_LAUNCH((nk_mfma_r_kernel<AROWS, BAND, true, 8>), p, a, s);
-      else FG_LAUNCH((nk_mfma_r_kernel<AROWS, BAND, false, 8>), p, a, s);
+      if (full) FG_LAUNCH((nk_mfma_r_kernel<AROWS, BAND, true, 8, CB>), p, a, s);
+      else FG_LAUNCH((nk_mfma_r_kernel<AROWS, BAND, false, 8, CB>), p, a, s);
       return;
     }
   }
-  if (full) FG_LAUNCH((nk_mfma_r_kernel<AROWS, BAND, true, 4>), p, a, s);
-  else FG_LAUNCH((nk_mfma_r_kernel<AROWS, BAND, false, 4>), p, a, s);
+  if (full) FG_LAUNCH((nk_mfma_r_kernel<AROWS, BAND, true, 4, CB>), p, a, s);
+  else FG_LAUNCH((nk_mfma_r_kernel<AROWS, BAND, false, 4, CB>), p, a, s);
 }
 
-// unroll = 2: 512-byte bands (two rows per load instruction); unroll = 1: 256-byte bands.
-bool launch_nk_mfma_r(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
-  if (p.tile_n != 16 || p.m_block != 16) return false;
-  if (p.waves > 4 && !(p.waves == 8 && p.unroll == 1)) return false;
+template <int CB>
+static bool nk_mfma_r_cb(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
   const bool half_m = a.M <= 8;  // one block row whose A strip needs only 8 rows
   if (p.unroll == 2) {
-    if (half_m) nk_mfma_r_go<8, 512>(p, a, s);
-    else nk_mfma_r_go<16, 512>(p, a, s);
+    if (half_m) nk_mfma_r_go<8, 512, CB>(p, a, s);
+    else nk_mfma_r_go<16, 512, CB>(p, a, s);
   } else if (p.unroll == 1) {
-    if (half_m) nk_mfma_r_go<8, 256>(p, a, s);
-    else nk_mfma_r_go<16, 256>(p, a, s);
+    if (half_m) nk_mfma_r_go<8, 256, CB>(p, a, s);
+    else nk_mfma_r_go<16, 256, CB>(p, a, s);
   } else {
     return false;
   }
   return true;
+}
+
+// unroll = 2: 512-byte bands (two rows per load instruction); unroll = 1: 256-byte bands.
+// tile_n = 16 or 32 (two 16-column blocks sharing the staged activations).
+bool launch_nk_mfma_r(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
+  if (p.m_block != 16) return false;
+  if (p.waves > 4 && !(p.waves == 8 && p.unroll == 1)) return false;
+  if (p.tile_n == 16) return nk_mfma_r_cb<1>(p, a, s);
+  if (p.tile_n == 32) return nk_mfma_r_cb<2>(p, a, s);
+  return false;
 }
 
 }  // namespace fg
