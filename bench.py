@@ -51,9 +51,10 @@ def _traffic(fetch_kib: float, write_kib: float) -> int:
 
 TRAFFIC_BYTES = {
     "nk_dot2_M1": _traffic(65621.2, 64.0),
-    "nk_mfma4_M8": _traffic(66096.5, 128.0),
-    "nk_mfma_t_M16": _traffic(66629.0, 2048.0),   # main kernel only; the 2 MiB written are split-K partials
-    "kn_dot2_M1": _traffic(65635.6, 128.0),
+    "nk_mfma_r_M8": _traffic(66077.0, 128.0),
+    "nk_mfma_r_M16": _traffic(66596.5, 256.0),
+    "kn_dot2_M1": _traffic(65699.1, 154.0),     # 128 KiB of the written bytes are split-K partials
+    "kn_mfma_M8": _traffic(66591.0, 1152.0),    # 1 MiB of split-K partials
 }
 
 
