@@ -144,6 +144,19 @@ def run_sweep(torch, sg, capi, dev, steps, warmup):
                  "weights_per_ns": round(Kk * Nn / us_i8 / 1e3, 3),
                  "fp16_M1_weights_per_ns": round(Kk * Nn / us_f16 / 1e3, 3),
                  "weight_throughput_vs_fp16": round(us_f16 / us_i8, 3)})
+    # beyond the benchmark's configurations: the same GEMV with 4-bit weights (two per byte)
+    del wq
+    wq4 = [torch.randint(0, 256, (Nn, Kk // 2), device=dev, generator=g, dtype=torch.uint8) for _ in range(20)]
+    us_i4 = time_us(lambda i: sg.fastgemv_int4(wq4[i % 20], x, y, scale=scale, zero_point=8.0))
+    by = Kk * Nn // 2 + 2 * Kk + 2 * Nn + 2 * Nn
+    rows.append({"config": "extra: int4 fastgemv", "op": "fastgemv_int4", "M": 1, "K": Kk, "N": Nn,
+                 "w_layout": "[N,K/2] uint4x2", "seed": 1004, "kernel": "w4a16", "splitk": 1, "bytes": by,
+                 "us_per_call": round(us_i4, 2), "GBps": round(by / us_i4 / 1e3, 1),
+                 "frac_hbm_peak": round(by / us_i4 / 1e3 / HBM_PEAK_GBPS, 4),
+                 "frac_read_ceiling": round(by / us_i4 / 1e3 / ceiling, 4),
+                 "weights_per_ns": round(Kk * Nn / us_i4 / 1e3, 3),
+                 "fp16_M1_weights_per_ns": round(Kk * Nn / us_f16 / 1e3, 3),
+                 "weight_throughput_vs_fp16": round(us_f16 / us_i4, 3)})
     return {"sweep": rows, "read_ceiling_GBps": round(ceiling, 1), "hbm_peak_GBps": HBM_PEAK_GBPS,
             "steps": steps, "warmup": warmup, "data": "synthetic", "dtype": "f16",
             "device": torch.cuda.get_device_name(0)}

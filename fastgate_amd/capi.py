@@ -42,6 +42,7 @@ EXPORTS = (
     "fg_workspace_header_bytes",
     "fg_workspace_init",
     "fg_gemv_w8a16",
+    "fg_gemv_w4a16",
     "fg_gemv_i8i8_i32",
     "fg_dequant_i32_f16",
     "fg_stream_read",
@@ -110,6 +111,8 @@ def lib() -> ctypes.CDLL:
         L.fg_workspace_init.argtypes = [vp, sz, vp]
         L.fg_gemv_w8a16.restype = ci
         L.fg_gemv_w8a16.argtypes = [vp, vp, vp, cf, cf, vp, ci, ci, ci, vp]
+        L.fg_gemv_w4a16.restype = ci
+        L.fg_gemv_w4a16.argtypes = [vp, vp, vp, cf, cf, vp, ci, ci, ci, vp]
         L.fg_gemv_i8i8_i32.restype = ci
         L.fg_gemv_i8i8_i32.argtypes = [vp, vp, vp, ci, ci, ci, vp]
         L.fg_dequant_i32_f16.restype = ci

@@ -337,6 +337,20 @@ int fg_gemv_w8a16(const void* Wq, const void* x, const void* scale, float scalar
   return fg::check_launch();
 }
 
+int fg_gemv_w4a16(const void* Wq4, const void* x, const void* scale, float scalar_scale,
+                  float zero_point, void* y, int M, int N, int K, void* stream) {
+  if (Wq4 == nullptr || x == nullptr || y == nullptr) return FG_ERR_INVALID_ARG;
+  if (M <= 0 || M > 4 || N <= 0 || K <= 0) return FG_ERR_INVALID_ARG;
+  if (N % 128 != 0 || K % 128 != 0) return FG_ERR_ALIGN128;
+  if ((reinterpret_cast<uintptr_t>(Wq4) | reinterpret_cast<uintptr_t>(x)) & 15) {
+    return FG_ERR_INVALID_ARG;
+  }
+  fg::W8A16Args a{Wq4, x, scale, scalar_scale, zero_point, y, M, N, K};
+  (void)hipGetLastError();
+  if (!fg::launch_w4a16(a, static_cast<hipStream_t>(stream))) return FG_ERR_UNSUPPORTED;
+  return fg::check_launch();
+}
+
 int fg_gemv_i8i8_i32(const void* Wq, const void* xq, int32_t* acc, int M, int N, int K,
                      void* stream) {
   if (Wq == nullptr || xq == nullptr || acc == nullptr) return FG_ERR_INVALID_ARG;

@@ -51,6 +51,7 @@ struct W8A16Args {
   int M, N, K;
 };
 bool launch_w8a16(const W8A16Args& a, hipStream_t s);
+bool launch_w4a16(const W8A16Args& a, hipStream_t s);  // Wq: two unsigned nibbles per byte, [N,K/2]
 bool launch_i8i8_i32(const void* Wq, const void* xq, int32_t* acc, int M, int N, int K,
                      hipStream_t s);
 void launch_dequant_i32_f16(const int32_t* acc, const void* scale, float x_scale, void* y, int M,

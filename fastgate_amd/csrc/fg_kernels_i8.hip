@@ -340,6 +340,131 @@ __global__ __launch_bounds__(256) void dequant_i32_f16_kernel(const int32_t* __r
 }
 
 // ---------------------------------------------------------------------------------------
+// w4a16: unsigned 4-bit weights, two per byte, the low nibble first (element 2i in bits 0-3 of
+// byte i, element 2i+1 in bits 4-7: uint4_2 of backend/cuda/hk/utility.cuh:13-36), fp16
+// activations.  A register w of 8 nibbles n0..n7 becomes four half2 with four v_and_or and one
+// shift, by letting the exponent absorb the nibble's position:
+//   (w      & 0x000F000F) | 0x64006400 = (1024 + n0, 1024 + n4)     (w >> 8 likewise: n2, n6)
+//   (w      & 0x00F000F0) | 0x54005400 = (  64 + n1,   64 + n5)     (w >> 8 likewise: n3, n7)
+// The 1024 is subtracted in fp16 (exact); the 64 stays in and is removed once per output as
+// 64·Σ x over the odd positions, which costs two v_dot2 per 8 activations shared by all rows
+// (products of at most 79·|x| instead of 15·|x| in the fp32 sum: two bits of headroom, not ten).
+// The activations are paired the same way, (x_j, x_{j+4}), once per chunk.
+// Replaces gemv_quantized_int4 (backend/cuda/hk/fastgemv.cuh:394-495), which the reference
+// defines but never launches.  Lanes along K: one 16-byte load = 32 weights of one row.
+// ---------------------------------------------------------------------------------------
+template <int MB, int RN>
+__global__ __launch_bounds__(256) void w4a16_kernel(const uint8_t* __restrict__ Wq,
+                                                    const half_t* __restrict__ X,
+                                                    const half_t* __restrict__ scale,
+                                                    float scalar_scale, float zero_point,
+                                                    half_t* __restrict__ Y, int M, int N, int K) {
+  __shared__ float red[16][RN * MB];
+  __shared__ float redx[16][MB];
+  __shared__ float redo[16][MB];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int nw = blockDim.x >> 6;
+  const int n0 = blockIdx.x * RN;
+  const int nq = K >> 5;        // 32-weight chunks per row
+  const size_t rowb = (size_t)K >> 1;  // bytes per weight row
+  const bool use_zp = zero_point != 0.f;
+
+  float acc[RN][MB];
+  float xsum[MB], xodd[MB];
+#pragma unroll
+  for (int m = 0; m < MB; ++m) {
+    xsum[m] = 0.f;
+    xodd[m] = 0.f;
+#pragma unroll
+    for (int r = 0; r < RN; ++r) acc[r][m] = 0.f;
+  }
+  const uint8_t* Wt = Wq + (size_t)n0 * rowb;
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+  const half2_t ones = {static_cast<half_t>(1.f), static_cast<half_t>(1.f)};
+  const half2_t bias = {static_cast<half_t>(1024.f), static_cast<half_t>(1024.f)};
+
+  const int nsteps = (nq + nw * 64 - 1) / (nw * 64);
+  int step = stagger_start(nsteps, 0);
+  for (int it = 0; it < nsteps; ++it) {
+    const int q = (step * nw + wave) * 64 + lane;
+    step = step + 1 == nsteps ? 0 : step + 1;
+    const bool ok = q < nq;
+    u32x4 wr[RN];
+#pragma unroll
+    for (int r = 0; r < RN; ++r) wr[r] = ok ? load16<true>(Wt + (size_t)r * rowb + (size_t)q * 16) : zero;
+    // xp[m][d][j] = (x[8d + j], x[8d + j + 4]) for the 8 activations under weight register d
+    uint32_t xp[MB][4][4];
+#pragma unroll
+    for (int m = 0; m < MB; ++m) {
+      const bool okm = ok && m < M;
+      const half_t* xptr = X + (size_t)m * K + (size_t)q * 32;
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        const u32x4 xv = okm ? load16<false>(xptr + 8 * d) : zero;  // x[8d .. 8d+7]
+        xp[m][d][0] = __builtin_amdgcn_perm(xv.z, xv.x, 0x05040100u);  // (x0, x4)
+        xp[m][d][1] = __builtin_amdgcn_perm(xv.z, xv.x, 0x07060302u);  // (x1, x5)
+        xp[m][d][2] = __builtin_amdgcn_perm(xv.w, xv.y, 0x05040100u);  // (x2, x6)
+        xp[m][d][3] = __builtin_amdgcn_perm(xv.w, xv.y, 0x07060302u);  // (x3, x7)
+        xodd[m] = __builtin_amdgcn_fdot2(as_half2(xp[m][d][1]), ones, xodd[m], false);
+        xodd[m] = __builtin_amdgcn_fdot2(as_half2(xp[m][d][3]), ones, xodd[m], false);
+        if (use_zp) {
+          xsum[m] = __builtin_amdgcn_fdot2(as_half2(xp[m][d][0]), ones, xsum[m], false);
+          xsum[m] = __builtin_amdgcn_fdot2(as_half2(xp[m][d][2]), ones, xsum[m], false);
+        }
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < RN; ++r)
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        const uint32_t w = wr[r][d], w8 = w >> 8;
+        const half2_t wv[4] = {as_half2((w & 0x000F000Fu) | 0x64006400u) - bias,
+                               as_half2((w & 0x00F000F0u) | 0x54005400u),
+                               as_half2((w8 & 0x000F000Fu) | 0x64006400u) - bias,
+                               as_half2((w8 & 0x00F000F0u) | 0x54005400u)};
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+          for (int m = 0; m < MB; ++m)
+            acc[r][m] = __builtin_amdgcn_fdot2(wv[j], as_half2(xp[m][d][j]), acc[r][m], false);
+      }
+  }
+
+  // xsum holds Σ x over the even positions (only when a zero point needs it), xodd over the odd
+#pragma unroll
+  for (int m = 0; m < MB; ++m) {
+#pragma unroll
+    for (int r = 0; r < RN; ++r) {
+      const float v = row16_allreduce(acc[r][m]);
+      if ((lane & 15) == 0) red[wave * 4 + (lane >> 4)][r * MB + m] = v;
+    }
+    const float xe = row16_allreduce(xsum[m]);
+    const float xo = row16_allreduce(xodd[m]);
+    if ((lane & 15) == 0) {
+      redx[wave * 4 + (lane >> 4)][m] = xe;
+      redo[wave * 4 + (lane >> 4)][m] = xo;
+    }
+  }
+  __syncthreads();
+  for (int t = threadIdx.x; t < RN * MB; t += blockDim.x) {
+    const int m = t / RN, r = t % RN;
+    float sum = 0.f, xe = 0.f, xo = 0.f;
+    for (int p = 0; p < nw * 4; ++p) {
+      sum += red[p][r * MB + m];
+      xe += redx[p][m];
+      xo += redo[p][m];
+    }
+    const int n = n0 + r;
+    if (m < M) {
+      float s = scalar_scale;
+      if (scale != nullptr) s *= static_cast<float>(scale[n]);
+      Y[(size_t)m * N + n] = static_cast<half_t>((sum - 64.f * xo - zero_point * (xe + xo)) * s);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
 // Host launchers.  Rows per workgroup: 8 when that still yields >= 512 workgroups, else 4.
 // Waves per workgroup: as many (<= 4) as the row has 1 KB pieces.
 // ---------------------------------------------------------------------------------------
@@ -367,6 +492,24 @@ bool launch_w8a16(const W8A16Args& a, hipStream_t s) {
   } else {
     return false;
   }
+  return true;
+}
+
+bool launch_w4a16(const W8A16Args& a, hipStream_t s) {
+  auto* Wq = static_cast<const uint8_t*>(a.Wq);
+  auto* X = static_cast<const half_t*>(a.x);
+  auto* sc = static_cast<const half_t*>(a.scale);
+  auto* Y = static_cast<half_t*>(a.y);
+  const int pieces = (a.K / 32 + 63) / 64;  // 1 KB pieces per weight row
+  const dim3 block(64 * (pieces >= 4 ? 4 : (pieces >= 2 ? 2 : 1)));
+#define W4(MB) \
+  hipLaunchKernelGGL((w4a16_kernel<MB, 4>), dim3(a.N / 4), block, 0, s, Wq, X, sc, a.scalar_scale, \
+                     a.zero_point, Y, a.M, a.N, a.K)
+  if (a.M == 1) W4(1);
+  else if (a.M == 2) W4(2);
+  else if (a.M <= 4) W4(4);
+  else return false;
+#undef W4
   return true;
 }
 

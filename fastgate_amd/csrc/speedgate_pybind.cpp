@@ -239,6 +239,39 @@ void fastgemv_int8(at::Tensor mat, at::Tensor vec, at::Tensor res, c10::optional
                op);
 }
 
+// fastgemv_int4(mat_u8[N,K/2], vec_f16, res_f16): the formula of gemv_quantized_int4
+// (hk/fastgemv.cuh:394-495), which the reference defines without a host function or binding.
+// Two unsigned 4-bit weights per byte, even element in the low nibble (hk/utility.cuh:13-36).
+void fastgemv_int4(at::Tensor mat, at::Tensor vec, at::Tensor res, c10::optional<at::Tensor> scale,
+                   double scalar_scale, double zero_point) {
+  const char* op = "fastgemv_int4";
+  TORCH_CHECK(mat.dim() == 2, op, ": mat must be 2-D [N,K/2]");
+  const int64_t N = mat.size(0), K = mat.size(1) * 2;
+  if (N % 128 || K % 128) throw std::invalid_argument(kMsgNK);
+  check_tensor(mat, "mat", at::kByte, op);
+  check_tensor(vec, "vec", at::kHalf, op);
+  check_tensor(res, "res", at::kHalf, op);
+  TORCH_CHECK(vec.numel() > 0 && vec.numel() % K == 0, op, ": vec must hold a multiple of K = ", K,
+              " elements");
+  const int64_t M = vec.numel() / K;
+  TORCH_CHECK(M <= 4, op, ": at most 4 activation rows");
+  TORCH_CHECK(res.numel() == M * N, op, ": res must hold M*N = ", M * N, " elements");
+  const void* sp = nullptr;
+  if (scale.has_value() && scale->defined()) {
+    check_tensor(*scale, "scale", at::kHalf, op);
+    TORCH_CHECK(scale->numel() == N, op, ": scale must hold N = ", N, " elements");
+    TORCH_CHECK(scale->device() == mat.device(), op, ": scale is on a different device");
+    sp = scale->data_ptr();
+  }
+  TORCH_CHECK(mat.device() == vec.device() && mat.device() == res.device(), op,
+              ": tensors are on different devices");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(mat.device());
+  raise_status(fg_gemv_w4a16(mat.data_ptr(), vec.data_ptr(), sp, (float)scalar_scale,
+                             (float)zero_point, res.data_ptr(), (int)M, (int)N, (int)K,
+                             current_stream(mat)),
+               op);
+}
+
 // Integer stage: acc_i32[M,N] = xq_i8[M,K] · mat_i8[N,K]^T (exact).
 void gemv_i8i8_i32(at::Tensor mat, at::Tensor xq, at::Tensor acc) {
   const char* op = "gemv_i8i8_i32";
@@ -339,6 +372,10 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         py::arg("scale") = py::none(), py::arg("scalar_scale") = 1.0, py::arg("zero_point") = 0.0,
         "res = (vec @ (mat_i8[N,K] - zero_point).T) * scalar_scale * scale[N] "
         "(hk/fastgemv.cu:35-61; per-channel scale is an extension)");
+  m.def("fastgemv_int4", &fastgemv_int4, py::arg("mat"), py::arg("vec"), py::arg("res"),
+        py::arg("scale") = py::none(), py::arg("scalar_scale") = 1.0, py::arg("zero_point") = 0.0,
+        "res = (vec @ (mat_u4[N,K] - zero_point).T) * scalar_scale * scale[N]; mat is uint8 [N,K/2], "
+        "even element in the low nibble (formula of hk/fastgemv.cuh:394-495)");
   m.def("gemv_i8i8_i32", &gemv_i8i8_i32, py::arg("mat"), py::arg("xq"), py::arg("acc"),
         "acc_i32[M,N] = xq_i8[M,K] @ mat_i8[N,K].T, exact");
   m.def("dequant_i32_f16", &dequant_i32_f16, py::arg("acc"), py::arg("scale"), py::arg("x_scale"),

@@ -140,6 +140,17 @@ int fg_gemv_w8a16(const void* Wq, const void* x, const void* scale, float scalar
                   float zero_point, void* y, int M, int N, int K, void* stream);
 
 /*
+ * W4A16 GEMV: y[m,n] = s_n · ( Σ_k x[m,k]·float(u4[n,k]) − zero_point·Σ_k x[m,k] ), u4 the unsigned
+ * 4-bit weights packed two per byte, element 2i in the low nibble of byte i (uint4_2,
+ * backend/cuda/hk/utility.cuh:13-36).  Wq4 uint8 [N,K/2] row-major, x fp16 [M,K], scale fp16 [N]
+ * or NULL, y fp16 [M,N].  fp32 accumulation, nibble→fp16 conversion exact.  1 <= M <= 4.
+ * Services the formula of gemv_quantized_int4 (backend/cuda/hk/fastgemv.cuh:394-495), a kernel
+ * the reference defines without a host entry point.
+ */
+int fg_gemv_w4a16(const void* Wq4, const void* x, const void* scale, float scalar_scale,
+                  float zero_point, void* y, int M, int N, int K, void* stream);
+
+/*
  * Integer dot stage: acc[m,n] = Σ_k int32(xq[m,k])·int32(Wq[n,k]) with v_dot4_i32_i8.
  * Wq int8 [N,K], xq int8 [M,K], acc int32 [M,N].  Exact for K <= 2^17.  1 <= M <= 8.
  * No counterpart in the reference (its int8 GEMV multiplies fp16 activations); this is the

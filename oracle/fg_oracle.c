@@ -16,6 +16,7 @@
  *                                 hk/edgemm_tr.cu:19-139; hk/fastgemv.cu:12-33,86-111
  *                                 (res[m*N+n] = Σ_k mat[n,k]·vec[m,k], hk/fastgemv.cuh:244-311)
  *   fg_oracle_gemv_w8a16          hk/fastgemv.cuh:316-389: sum += x·(float(w) − zp); sum *= scale
+ *   fg_oracle_gemv_w4a16          hk/fastgemv.cuh:394-495, nibble order hk/utility.cuh:13-36
  *   fg_oracle_gemv_i8i8_i32       none (integer stage added by this library); exact integer sum
  *
  * Pinning (tests/test_oracle.py): exact rational arithmetic on small cases, closed forms
@@ -204,6 +205,33 @@ void fg_oracle_gemv_w8a16(const int8_t* Wq, const uint16_t* X, const uint16_t* s
       const int8_t* w = Wq + (size_t)n * K;
       float sum = 0.f;
       for (int k = 0; k < K; ++k) sum += g_h2f[x[k]] * ((float)w[k] - zero_point);
+      sum *= scalar_scale;
+      if (scale) sum *= g_h2f[scale[n]];
+      if (Y32) Y32[(size_t)m * N + n] = sum;
+      Y[(size_t)m * N + n] = fg_oracle_f2h(sum);
+    }
+  }
+}
+
+/*
+ * W4A16 GEMV, hk/fastgemv.cuh:394-495 with the nibble order of hk/utility.cuh:13-36 (getX = low
+ * nibble = even element, getY = high nibble = odd element): sum += x·(float(u4) − zp) in
+ * ascending k, scale last.  Wq4 is [N][K/2] bytes.
+ */
+void fg_oracle_gemv_w4a16(const uint8_t* Wq4, const uint16_t* X, const uint16_t* scale,
+                          float scalar_scale, float zero_point, uint16_t* Y, float* Y32, int M, int N,
+                          int K) {
+  ensure_table();
+  for (int m = 0; m < M; ++m) {
+    const uint16_t* x = X + (size_t)m * K;
+    for (int n = 0; n < N; ++n) {
+      const uint8_t* w = Wq4 + (size_t)n * (K / 2);
+      float sum = 0.f;
+      for (int k = 0; k < K; ++k) {
+        const uint8_t b = w[k >> 1];
+        const float u = (float)((k & 1) ? (b >> 4) : (b & 0x0f));
+        sum += g_h2f[x[k]] * (u - zero_point);
+      }
       sum *= scalar_scale;
       if (scale) sum *= g_h2f[scale[n]];
       if (Y32) Y32[(size_t)m * N + n] = sum;

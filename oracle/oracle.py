@@ -51,6 +51,8 @@ def lib() -> ctypes.CDLL:
         L.fg_oracle_gemm_f16_f64.argtypes = [vp, vp, vp, vp, vp, ci, ci, ci, ci, ci]
         L.fg_oracle_gemv_w8a16.restype = None
         L.fg_oracle_gemv_w8a16.argtypes = [vp, vp, vp, cf, cf, vp, vp, ci, ci, ci]
+        L.fg_oracle_gemv_w4a16.restype = None
+        L.fg_oracle_gemv_w4a16.argtypes = [vp, vp, vp, cf, cf, vp, vp, ci, ci, ci]
         L.fg_oracle_gemv_i8i8_i32.restype = ci
         L.fg_oracle_gemv_i8i8_i32.argtypes = [vp, vp, vp, ci, ci, ci]
         L.fg_oracle_dequant_i32_f16.restype = None
@@ -130,6 +132,24 @@ def gemv_w8a16(Wq, x, scale=None, scalar_scale: float = 1.0, zero_point: float =
     y = np.zeros((M, N), np.float16)
     y32 = np.zeros((M, N), np.float32)
     lib().fg_oracle_gemv_w8a16(_ptr(Wq), _ptr(x), _ptr(sc), float(scalar_scale), float(zero_point),
+                               _ptr(y), _ptr(y32), M, N, K)
+    return y, y32
+
+
+def gemv_w4a16(Wq4, x, scale=None, scalar_scale: float = 1.0, zero_point: float = 0.0):
+    """Wq4 uint8 [N,K/2], two unsigned nibbles per byte (even element in the low nibble):
+    y[m,n] = fp16((Σ_k x[m,k]·(float(u4[n,k]) − zp))·scalar_scale·scale[n]); returns
+    (float16 [M,N], float32 unrounded)."""
+    Wq4 = np.ascontiguousarray(Wq4)
+    if Wq4.dtype != np.uint8:
+        raise TypeError("Wq4 must be uint8")
+    N, K = Wq4.shape[0], Wq4.shape[1] * 2
+    x = _f16(x).reshape(-1, K)
+    M = x.shape[0]
+    sc = None if scale is None else _f16(scale).reshape(N)
+    y = np.zeros((M, N), np.float16)
+    y32 = np.zeros((M, N), np.float32)
+    lib().fg_oracle_gemv_w4a16(_ptr(Wq4), _ptr(x), _ptr(sc), float(scalar_scale), float(zero_point),
                                _ptr(y), _ptr(y32), M, N, K)
     return y, y32
 

@@ -127,3 +127,88 @@ def test_int8_error_codes(device):
     assert L.fg_gemv_w8a16(ptr(W), ptr(x), None, 1.0, 0.0, ptr(y), 9, 128, 128, stream_ptr()) == capi.FG_ERR_INVALID_ARG
     assert L.fg_gemv_w8a16(ptr(W), ptr(x), None, 1.0, 0.0, ptr(y), 1, 100, 128, stream_ptr()) == capi.FG_ERR_ALIGN128
     assert L.fg_gemv_w8a16(None, ptr(x), None, 1.0, 0.0, ptr(y), 1, 128, 128, stream_ptr()) == capi.FG_ERR_INVALID_ARG
+
+
+# ---------------------------------------------------------------------------------------
+# int4 weights (two unsigned nibbles per byte, even element in the low nibble)
+# ---------------------------------------------------------------------------------------
+def _w4a16(Wq4, x, scale, scalar_scale, zp, device):
+    L = capi.lib()
+    M = x.shape[0]
+    N, K = Wq4.shape[0], Wq4.shape[1] * 2
+    y = torch.full((M, N), float("nan"), dtype=torch.half, device=device)
+    Wd, xd = Wq4.to(device), x.to(device)
+    sd = None if scale is None else scale.to(device)
+    capi.check(L.fg_gemv_w4a16(ptr(Wd), ptr(xd), ptr(sd), scalar_scale, zp, ptr(y), M, N, K,
+                               stream_ptr()), "fg_gemv_w4a16")
+    torch.cuda.synchronize()
+    return y.cpu().numpy()
+
+
+@pytest.mark.parametrize("M", [1, 2, 3, 4])
+@pytest.mark.parametrize("N,K", [(128, 128), (256, 1152), (1024, 4096), (512, 8192 + 384)])
+def test_w4a16_matches_oracle(device, M, N, K):
+    g = gen(900 + M + N + K)
+    x = normal((M, K), g, 1.0)
+    Wq4 = torch.randint(0, 256, (N, K // 2), generator=g, dtype=torch.uint8)
+    scale = (torch.rand(N, generator=g) * 0.009 + 0.001).half()
+    ref, _ = oracle.gemv_w4a16(Wq4.numpy(), x.numpy(), scale.numpy(), 1.0, 8.0)
+    assert_close_f16(_w4a16(Wq4, x, scale, 1.0, 8.0, device), ref, "per-channel scale, zero point 8")
+    ref, _ = oracle.gemv_w4a16(Wq4.numpy(), (x * 0.01).half().numpy(), None, 1.0, 0.0)
+    assert_close_f16(_w4a16(Wq4, (x * 0.01).half(), None, 1.0, 0.0, device), ref, "no scale, no zero point")
+    ref, _ = oracle.gemv_w4a16(Wq4.numpy(), x.numpy(), scale.numpy(), 0.5, 7.5)
+    assert_close_f16(_w4a16(Wq4, x, scale, 0.5, 7.5, device), ref, "scale 0.5 zp 7.5")
+
+
+def test_w4a16_every_nibble_in_every_position_is_exact(device):
+    # x = e_k picks single weights: the result must be the nibble itself, for all 32 positions of
+    # a 16-byte load and all 16 values
+    N, K = 128, 128
+    Wq4 = torch.zeros((N, K // 2), dtype=torch.uint8)
+    for n in range(N):
+        for b in range(K // 2):
+            lo, hi = (n + b) % 16, (n + 3 * b + 5) % 16
+            Wq4[n, b] = lo | (hi << 4)
+    want = np.empty((N, K), np.float32)
+    want[:, 0::2] = (Wq4 & 0x0F).numpy()
+    want[:, 1::2] = (Wq4 >> 4).numpy()
+    for k in range(0, K, 4):
+        x = torch.zeros((4, K), dtype=torch.half)
+        for m in range(4):
+            x[m, k + m] = 1.0
+        got = _w4a16(Wq4, x, None, 1.0, 0.0, device)
+        for m in range(4):
+            assert (got[m] == want[:, k + m]).all(), (k, m)
+
+
+def test_w4a16_small_integers_are_exact(device):
+    g = gen(950)
+    N, K = 256, 2048
+    Wq4 = torch.randint(0, 256, (N, K // 2), generator=g, dtype=torch.uint8)
+    x = torch.randint(-4, 5, (3, K), generator=g).half()
+    ref, ref32 = oracle.gemv_w4a16(Wq4.numpy(), x.numpy(), None, 1.0, 8.0)
+    got = _w4a16(Wq4, x, None, 1.0, 8.0, device)
+    assert (got == ref).all()
+
+
+def test_w4a16_pybind_and_errors(device):
+    import fastgate_amd
+    sg = fastgate_amd.speedgate
+    g = gen(960)
+    N, K = 256, 512
+    Wq4 = torch.randint(0, 256, (N, K // 2), generator=g, dtype=torch.uint8)
+    x = normal((2, K), g, 1.0)
+    scale = (torch.rand(N, generator=g) * 0.009 + 0.001).half()
+    y = torch.empty((2, N), dtype=torch.half, device=device)
+    sg.fastgemv_int4(Wq4.to(device), x.to(device), y, scale=scale.to(device), zero_point=8.0)
+    ref, _ = oracle.gemv_w4a16(Wq4.numpy(), x.numpy(), scale.numpy(), 1.0, 8.0)
+    assert_close_f16(y.cpu().numpy(), ref, "fastgemv_int4")
+    with pytest.raises(ValueError):
+        sg.fastgemv_int4(Wq4[:100].contiguous().to(device), x.to(device), y)
+    with pytest.raises(RuntimeError):
+        sg.fastgemv_int4(Wq4.to(device).to(torch.int8), x.to(device), y)
+    L = capi.lib()
+    W = Wq4.to(device)
+    xd = x.to(device)
+    assert L.fg_gemv_w4a16(ptr(W), ptr(xd), None, 1.0, 0.0, ptr(y), 5, N, K, stream_ptr()) == capi.FG_ERR_INVALID_ARG
+    assert L.fg_gemv_w4a16(ptr(W), ptr(xd), None, 1.0, 0.0, ptr(y), 1, 100, K, stream_ptr()) == capi.FG_ERR_ALIGN128

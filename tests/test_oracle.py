@@ -255,3 +255,63 @@ def test_operator_table_rejects_unaligned():
         oracle.gemm_op("edgemm_m8n128k64x4", A, np.zeros((200, 128), np.float16), None)
     with pytest.raises(ValueError, match="multiple of 128"):
         oracle.gemm_op("edgemm_m8n128k64x4_bt", np.zeros((8, 128), np.float16), np.zeros((100, 128), np.float16), None)
+
+
+# ---------------------------------------------------------------------------------------
+# int4: two unsigned nibbles per byte, even element in the low nibble (hk/utility.cuh:13-36)
+# ---------------------------------------------------------------------------------------
+def _unpack_u4(Wq4):
+    lo = (Wq4 & 0x0F).astype(np.int64)
+    hi = (Wq4 >> 4).astype(np.int64)
+    out = np.empty((Wq4.shape[0], Wq4.shape[1] * 2), np.int64)
+    out[:, 0::2] = lo   # getX: low nibble = first element
+    out[:, 1::2] = hi   # getY: high nibble = second element
+    return out
+
+
+def test_w4a16_nibble_order_and_every_value():
+    # x = e_k picks single weights: the result is the nibble itself; byte 0xA3 holds 3 then 10
+    N, K = 16, 32
+    Wq4 = np.zeros((N, K // 2), np.uint8)
+    Wq4[:, 0] = 0xA3
+    for n in range(N):
+        Wq4[n, 5] = n | ((15 - n) << 4)
+    for k, want in ((0, 3.0), (1, 10.0)):
+        x = np.zeros((1, K), np.float16)
+        x[0, k] = 1.0
+        y, _ = oracle.gemv_w4a16(Wq4, x)
+        assert (y == want).all()
+    x = np.zeros((2, K), np.float16)
+    x[0, 10] = 1.0
+    x[1, 11] = 1.0
+    y, _ = oracle.gemv_w4a16(Wq4, x)
+    assert (y[0] == np.arange(N)).all() and (y[1] == 15 - np.arange(N)).all()
+
+
+def test_w4a16_matches_exact_integer_arithmetic():
+    # integer x, integer zero point: every product and sum is an exact integer below 2^24
+    rng = np.random.default_rng(404)
+    N, K = 64, 512
+    Wq4 = rng.integers(0, 256, (N, K // 2), dtype=np.uint8)
+    xi = rng.integers(-8, 9, (3, K))
+    for zp in (0, 8, 3):
+        want = xi @ (_unpack_u4(Wq4) - zp).T          # int64, exact
+        y, y32 = oracle.gemv_w4a16(Wq4, xi.astype(np.float16), None, 1.0, float(zp))
+        assert (y32.astype(np.int64) == want).all()
+        assert (y.astype(np.float64) == np.float16(want).astype(np.float64)).all()
+    # power-of-two scales are exact as well
+    sc = np.float16(2.0) ** rng.integers(-6, 1, N)
+    y, _ = oracle.gemv_w4a16(Wq4, xi.astype(np.float16), sc.astype(np.float16), 0.5, 8.0)
+    want = (xi @ (_unpack_u4(Wq4) - 8).T) * 0.5 * sc.astype(np.float64)[None, :]
+    assert (y.astype(np.float64) == np.float16(want).astype(np.float64)).all()
+
+
+def test_w4a16_against_float64_on_random_inputs():
+    rng = np.random.default_rng(405)
+    N, K = 128, 1024
+    Wq4 = rng.integers(0, 256, (N, K // 2), dtype=np.uint8)
+    x = rng.standard_normal((2, K)).astype(np.float16)
+    sc = (rng.random(N) * 0.009 + 0.001).astype(np.float16)
+    _, y32 = oracle.gemv_w4a16(Wq4, x, sc, 1.0, 7.5)
+    want = (x.astype(np.float64) @ (_unpack_u4(Wq4) - 7.5).T) * sc.astype(np.float64)[None, :]
+    assert np.abs(y32 - want).max() <= 2e-4 * np.abs(want).max()
