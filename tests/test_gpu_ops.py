@@ -155,3 +155,23 @@ def test_runs_on_the_current_stream(device, sg):
             sg.edgemm_m8n128k64x4(A, B, C)
     s.synchronize()
     assert_close_f16(C.cpu().numpy(), ref, "side stream")
+
+
+def test_reference_harness_flow(device):
+    # the reference's table row (script/standard-test.py): torch, vendor, then each operator with
+    # its time, share of outputs within 100 and the allclose verdict
+    import eed.backend as backend
+    from fastgate_amd import harness
+    funcs = [backend.edgemm_m8n128k64x4, backend.edgemm_m8n128k64x4_bt, backend.gemm_m8n64k128x8_bt_exp,
+             backend.flat_gemm_m8n256k64x8, backend.edgemm_m8n64k128x8_bt_tuning]
+    row = harness.run_config(funcs, 8, 1024, 2048, warmup=2, iters=3, bz=2)
+    assert set(row["ops"]) == {"edgemm_m8n128k64x4", "edgemm_m8n128k64x4_bt", "gemm_m8n64k128x8_bt_exp",
+                                "flat_gemm_m8n256k64x8"}   # the alias shares its target's name
+    for name, e in row["ops"].items():
+        assert e["share_within_100"] == 1.0 and e["allclose"], (name, e)
+        assert e["ms"] > 0
+    assert row["vendor_share_within_100"] == 1.0
+    assert len(harness.format_row(row).split()) == 3 + 2 + len(row["ops"]) + 1 + len(row["ops"])
+    # the GEMV family: weight first
+    row = harness.run_config([backend.fastgemv, backend.fastgemv_tuned], 1, 2048, 1024, warmup=1, iters=2)
+    assert all(e["allclose"] for e in row["ops"].values())

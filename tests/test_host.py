@@ -198,3 +198,63 @@ def test_product_never_touches_the_oracle():
         if re.search(r"\boracle\b", path.read_text()):
             offenders.append(str(path.relative_to(ROOT)))
     assert not offenders, offenders
+
+
+# ---------------------------------------------------------------------------------------
+# harness conventions (script/standard-test.py:89-118): which operands each family receives
+# ---------------------------------------------------------------------------------------
+def _stub(name, log):
+    def f(*args):
+        log.append((name, args))
+    f.__name__ = name
+    return f
+
+
+def test_harness_dispatch_conventions():
+    from fastgate_amd import harness
+    log = []
+    A, B, C, A_T, B_T, C_T = "A", "B", "C", "A_T", "B_T", "C_T"
+    harness.dispatch_func(_stub("fastgemv", log), A, B, C, A_T, B_T, C_T)
+    harness.dispatch_func(_stub("edgemm_m8n128k64x4_bt", log), A, B, C, A_T, B_T, C_T)
+    harness.dispatch_func(_stub("edgemm_m8n128k64x4", log), A, B, C, A_T, B_T, C_T)
+    assert log == [("fastgemv", (B_T, A_T, C_T)), ("edgemm_m8n128k64x4_bt", (A, B_T, C)),
+                   ("edgemm_m8n128k64x4", (A, B, C))]
+
+    class T:  # stands in for a tensor: transpose().contiguous() yields the [K,N] weight
+        def transpose(self, a, b):
+            return self
+        def contiguous(self):
+            return "B"
+    log.clear()
+    harness.dispatch_func_btrans(_stub("fastgemv_tuned", log), A, B_T, C, 2)
+    harness.dispatch_func_btrans(_stub("gemm_m8n32k256x8_bt", log), A, B_T, C, 2)
+    harness.dispatch_func_btrans(_stub("gemm_m8n64k128x8_bt_exp", log), A, B_T, C, 2)
+    harness.dispatch_func_btrans(_stub("flat_gemm_m8n256k64x8", log), A, T(), C, 4)
+    harness.dispatch_func_btrans(_stub("edgemm_m8n256k32x8", log), A, T(), C, 4)
+    assert log == [("fastgemv_tuned", (B_T, A, C)), ("gemm_m8n32k256x8_bt", (A, B_T, C)),
+                   ("gemm_m8n64k128x8_bt_exp", (A, B_T, C, 2)), ("flat_gemm_m8n256k64x8", (A, "B", C, 4)),
+                   ("edgemm_m8n256k32x8", (A, "B", C))]
+
+
+def test_harness_tables_match_the_bound_operators(sg):
+    from fastgate_amd import harness
+    bound = set(n for n in dir(sg) if not n.startswith("_"))
+    aliases = {"edgemm_m8n32k128x8_bt", "edgemm_m8n32k256x8_bt", "edgemm_m8n64k128x8_bt_tuning",
+               "edgemm_m8n32k256x8_bt_tuning"}
+    for name in harness.ALL_TRANSPOSED + harness.B_TRANSPOSED + harness.TAKES_BZ:
+        assert name in bound or name in aliases, name
+    # every [N,K]-layout GEMM name of the semantics table is routed as "B transposed"
+    from oracle import oracle
+    for name, (layout, _protocol, has_bz) in oracle.GEMM_OPS.items():
+        assert (name in harness.B_TRANSPOSED) == (layout == NK), name
+        assert (name in harness.TAKES_BZ) == has_bz, name
+
+
+def test_eed_backend_reexports_every_operator(sg):
+    import eed.backend as backend
+    for name in dir(sg):
+        if not name.startswith("_"):
+            assert getattr(backend, name) is getattr(sg, name), name
+    assert backend.edgemm_m8n64k128x8_bt_tuning is sg.gemm_m8n64k128x8_bt_exp
+    with pytest.raises(ImportError):
+        from eed.backend import hgemm_warp2  # noqa: F401  (no surviving definition in the reference)
