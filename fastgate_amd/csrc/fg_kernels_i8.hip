@@ -465,6 +465,127 @@ __global__ __launch_bounds__(256) void w4a16_kernel(const uint8_t* __restrict__ 
 }
 
 // ---------------------------------------------------------------------------------------
+// w8a16 with both operands staged through wave-private LDS (the int8 sibling of the fp16
+// row-load kernel).  Per step a wave loads a 256-byte band (256 k) of the tile's 16 weight rows
+// -- 4 rows x 256 B per instruction -- and the matching 512-byte band of the activation rows,
+// parks them in LDS strips and reads them back in v_mfma_f32_16x16x32_f16 operand order: 8 bytes
+// of one weight row per lane, converted to 8 fp16 there, against 16 bytes of one activation row.
+// The activations are fetched once per 16 weight rows instead of once per 4, the dot products run
+// on the matrix pipe, and the VALU only converts.  16-column tiles, 8 waves interleaving over K.
+// XROWS = activation rows staged (2 covers M <= 2, 8 covers M <= 8).
+// ---------------------------------------------------------------------------------------
+template <int XROWS, int NW>
+__global__ __launch_bounds__(64 * NW) void w8a16_r_kernel(const int8_t* __restrict__ Wq,
+                                                          const half_t* __restrict__ X,
+                                                          const half_t* __restrict__ scale,
+                                                          float scalar_scale, float zero_point,
+                                                          half_t* __restrict__ Y, int M, int N, int K) {
+  constexpr int RSW = 256 + 16;      // LDS bytes per staged weight row
+  constexpr int RSX = 512 + 16;      // ... per staged activation row
+  constexpr int WSTRIP = 16 * RSW;
+  constexpr int XSTRIP = XROWS * RSX;
+  constexpr int WAVE_LDS = WSTRIP + XSTRIP;
+  constexpr int XI = XROWS / 2;      // activation load instructions per step (2 rows each)
+  static_assert(WAVE_LDS >= 2 * 256 * (int)sizeof(float), "reduction scratch fits");
+  __shared__ __attribute__((aligned(16))) unsigned char smem[NW * WAVE_LDS];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int nw = blockDim.x >> 6;
+  const int j = lane & 15, g = lane >> 4;        // operand order
+  const int hw = lane >> 4, cw = lane & 15;      // weight load order: row 4i + hw, piece cw
+  const int hx = lane >> 5, cx = lane & 31;      // activation load order: row 2i + hx, piece cx
+  const int n0 = blockIdx.x * 16;
+  const int nbands = (K + 255) >> 8;             // K % 128 == 0: the last band may be half
+  const bool use_zp = zero_point != 0.f;
+  unsigned char* wstrip = smem + wave * WAVE_LDS;
+  unsigned char* xstrip = wstrip + WSTRIP;
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+
+  const int8_t* Wp = Wq + (size_t)(n0 + hw) * K + cw * 16;
+  const half_t* Xp = X + (size_t)hx * K + cx * 8;
+  bool xrow[XI];
+#pragma unroll
+  for (int i = 0; i < XI; ++i) xrow[i] = (2 * i + hx) < M;
+  const int stw_off = hw * RSW + cw * 16;
+  const int stx_off = hx * RSX + cx * 16;
+  const int ldw_off = j * RSW + g * 8;
+  const int ldx_off = (j % XROWS) * RSX + g * 16;  // MFMA rows beyond XROWS re-read staged rows; unused
+
+  auto load_band = [&](int band, u32x4(&w)[4], u32x4(&x)[XI]) {
+    const bool okw = band < nbands && (band * 256 + cw * 16) < K;
+    const bool okx = band < nbands && (band * 256 + cx * 8) < K;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) w[i] = okw ? load16<true>(Wp + (size_t)(4 * i) * K + (size_t)band * 256) : zero;
+#pragma unroll
+    for (int i = 0; i < XI; ++i)
+      x[i] = (okx && xrow[i]) ? load16<false>(Xp + (size_t)(2 * i) * K + (size_t)band * 256) : zero;
+  };
+  float4_t acc = {0.f, 0.f, 0.f, 0.f}, xacc = {0.f, 0.f, 0.f, 0.f};
+  const half8_t ones8 = {static_cast<half_t>(1.f), static_cast<half_t>(1.f), static_cast<half_t>(1.f),
+                         static_cast<half_t>(1.f), static_cast<half_t>(1.f), static_cast<half_t>(1.f),
+                         static_cast<half_t>(1.f), static_cast<half_t>(1.f)};
+  auto multiply = [&](const u32x4(&w)[4], const u32x4(&x)[XI]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(wstrip + stw_off + 4 * i * RSW) = w[i];
+#pragma unroll
+    for (int i = 0; i < XI; ++i) *reinterpret_cast<u32x4*>(xstrip + stx_off + 2 * i * RSX) = x[i];
+    wave_lds_sync();
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const u32x4 xv = *reinterpret_cast<const u32x4*>(xstrip + ldx_off + u * 64);
+      const u32x2 wv = *reinterpret_cast<const u32x2*>(wstrip + ldw_off + u * 32);
+      half2_t h0, h1, h2, h3;
+      i8x4_to_half2x2(wv.x, h0, h1);
+      i8x4_to_half2x2(wv.y, h2, h3);
+      const half8_t wb = {h0[0], h0[1], h1[0], h1[1], h2[0], h2[1], h3[0], h3[1]};
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(xv), wb, acc, 0, 0, 0);
+      if (use_zp) xacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(xv), ones8, xacc, 0, 0, 0);
+    }
+    wave_lds_sync();
+  };
+
+  u32x4 w0[4], w1[4], x0[XI], x1[XI];
+  const int nsteps = (nbands + nw - 1) / nw;
+  int step = stagger_start(nsteps, 0);
+  auto next_band = [&]() {
+    const int band = step * nw + wave;
+    step = step + 1 == nsteps ? 0 : step + 1;
+    return band;
+  };
+  load_band(next_band(), w0, x0);
+  for (int it = 0; it < nsteps; it += 2) {
+    if (it + 1 < nsteps) load_band(next_band(), w1, x1);
+    multiply(w0, x0);
+    if (it + 1 >= nsteps) break;
+    if (it + 2 < nsteps) load_band(next_band(), w0, x0);
+    multiply(w1, x1);
+  }
+
+  // acc[r] = D[m = 4g + r][column j] (xacc: Σ x of row m in every column); waves meet in LDS
+  __syncthreads();
+  float(*red)[2][256] = reinterpret_cast<float(*)[2][256]>(smem);
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    red[wave][0][(4 * g + r) * 16 + j] = acc[r];
+    red[wave][1][(4 * g + r) * 16 + j] = xacc[r];
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < 256; e += blockDim.x) {
+    const int m = e >> 4, n = n0 + (e & 15);
+    if (m < M) {
+      float sum = 0.f, xs = 0.f;
+      for (int wv = 0; wv < nw; ++wv) {
+        sum += red[wv][0][e];
+        xs += red[wv][1][e];
+      }
+      float sc = scalar_scale;
+      if (scale != nullptr) sc *= static_cast<float>(scale[n]);
+      Y[(size_t)m * N + n] = static_cast<half_t>((sum - zero_point * xs) * sc);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
 // Host launchers.  Rows per workgroup: 8 when that still yields >= 512 workgroups, else 4.
 // Waves per workgroup: as many (<= 4) as the row has 1 KB pieces.
 // ---------------------------------------------------------------------------------------
@@ -473,8 +594,10 @@ static int i8_waves(int K) {
   return pieces >= 4 ? 4 : (pieces >= 2 ? 2 : 1);
 }
 
-// Measured at K = N = 8192 (us per call, lanes-along-K kernel / MFMA kernel): M=1 12.6 / 13.5,
-// M=2 15.1 / 13.9, M=4 21.1 / 15.4, M=5 33.5 / 18.2, M=8 32.9 / 20.7.
+// Measured (us per call; lanes-along-K kernel / 4x4x4 MFMA kernel / row-load kernel):
+//   K = N = 8192   M=1 12.6 / 13.5 / 14.3   M=2 15.1 / 13.9 / 14.2   M=4 21.1 / 15.4 / 14.9   M=8 32.9 / 20.7 / 17.2
+//   K = N = 16384  M=1 41.2 /  -   / 44.8   M=2  -   / 50.2 / 45.8   M=4  -   / 52.7 / 47.8   M=8  -   / 66.9 / 49.7
+// The row-load kernel exists with 8 waves only.
 bool launch_w8a16(const W8A16Args& a, hipStream_t s) {
   auto* Wq = static_cast<const int8_t*>(a.Wq);
   auto* X = static_cast<const half_t*>(a.x);
@@ -483,11 +606,14 @@ bool launch_w8a16(const W8A16Args& a, hipStream_t s) {
   if (a.M == 1) {  // 4 rows per workgroup, one load group in flight
     hipLaunchKernelGGL((w8a16_kernel<1, 4, 1>), dim3(a.N / 4), dim3(64 * i8_waves(a.K)), 0, s, Wq, X,
                        sc, a.scalar_scale, a.zero_point, Y, a.M, a.N, a.K);
-  } else if (a.M <= 4) {
+  } else if (a.M <= 3 && (size_t)a.N * a.K <= ((size_t)1 << 27)) {
     hipLaunchKernelGGL((w8a16_mfma_kernel<1, 4, 2>), dim3(a.N / 16), dim3(256), 0, s, Wq, X, sc,
                        a.scalar_scale, a.zero_point, Y, a.M, a.N, a.K);
+  } else if (a.M <= 2) {
+    hipLaunchKernelGGL((w8a16_r_kernel<2, 8>), dim3(a.N / 16), dim3(512), 0, s, Wq, X, sc,
+                       a.scalar_scale, a.zero_point, Y, a.M, a.N, a.K);
   } else if (a.M <= 8) {
-    hipLaunchKernelGGL((w8a16_mfma_kernel<2, 4, 1>), dim3(a.N / 16), dim3(256), 0, s, Wq, X, sc,
+    hipLaunchKernelGGL((w8a16_r_kernel<8, 8>), dim3(a.N / 16), dim3(512), 0, s, Wq, X, sc,
                        a.scalar_scale, a.zero_point, Y, a.M, a.N, a.K);
   } else {
     return false;

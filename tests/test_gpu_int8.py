@@ -43,6 +43,21 @@ def test_w8a16_matches_oracle(device, M, N, K):
     assert_close_f16(_w8a16(Wq, x, scale, 0.5, 3.0, device), ref, "scale 0.5 zp 3")
 
 
+@pytest.mark.parametrize("M", [2, 3])
+def test_w8a16_large_weights_take_the_row_load_kernel(device, M):
+    # above 2^27 weights M = 2..3 switches to the LDS-staged kernel (2-row and 8-row activation
+    # strips); the oracle checks a band of output channels
+    N, K = 16384, 8192 + 128
+    g = gen(880 + M)
+    x = normal((M, K), g, 1.0)
+    Wq = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8)
+    scale = (torch.rand(N, generator=g) * 0.009 + 0.001).half()
+    got = _w8a16(Wq, x, scale, 1.0, 2.0, device)
+    for lo in (0, 8000, N - 144):
+        ref, _ = oracle.gemv_w8a16(Wq[lo:lo + 144].numpy(), x.numpy(), scale[lo:lo + 144].numpy(), 1.0, 2.0)
+        assert_close_f16(got[:, lo:lo + 144], ref, "rows %d.." % lo)
+
+
 def test_w8a16_every_int8_value_is_exact(device):
     # x = e_k picks single weights: the result must be the int8 value itself, all 256 of them.
     N, K = 256, 128
