@@ -259,6 +259,16 @@ def main() -> int:
     e1.record()
     barrier()
     ceiling_gbps = (1 << 30) * 10 / (e0.elapsed_time(e1) * 1e-3) / 1e9
+    # device-to-device copy of 1 GiB, counted as read + write bytes (the other usual "copy bandwidth")
+    for i in range(2):
+        probe[1].copy_(probe[0])
+    barrier()
+    e0.record()
+    for i in range(5):
+        probe[1].copy_(probe[0])
+    e1.record()
+    barrier()
+    copy_gbps = 2 * (1 << 30) * 5 / (e0.elapsed_time(e1) * 1e-3) / 1e9
     del probe
 
     # ---- warm-up, then exactly `steps` timed steps ------------------------------------------------
@@ -299,11 +309,20 @@ def main() -> int:
         it += args.steps
         us = e0.elapsed_time(e1) * 1e3 / args.steps
         gbps = algorithmic_bytes(M) / (us * 1e-6) / 1e9
+        # the same call on one weight buffer: 128 MiB stays in the 256 MB Infinity Cache
+        barrier()
+        e0.record()
+        for s in range(args.steps):
+            fn(0)
+        e1.record()
+        barrier()
+        us_hot = e0.elapsed_time(e1) * 1e3 / args.steps
         per_call.append({
             "op": label, "M": M, "w_layout": "[N,K]" if layout == capi.FG_W_NK else "[K,N]",
             "kernel": p["kernel_name"], "splitk": p["splitk"], "tile_n": p["tile_n"], "waves": p["waves"],
             "unroll": p["unroll"], "launches": 1 + (p["splitk"] > 1 and not p["fused"]),
             "bytes": algorithmic_bytes(M), "us_per_call": round(us, 2), "GBps": round(gbps, 1),
+            "us_per_call_single_buffer": round(us_hot, 2),
             "TFLOPs": round(2.0 * M * N * K / (us * 1e-6) / 1e12, 2),
             "frac_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4),
             "frac_read_ceiling": round(gbps / ceiling_gbps, 4)})
@@ -372,6 +391,7 @@ def main() -> int:
         "gpu_ms_per_step": round(gpu_ms / args.steps, 4),
         "frac_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
         "read_ceiling_GBps": round(ceiling_gbps, 1), "frac_read_ceiling": round(value / ceiling_gbps, 4),
+        "copy_ceiling_GBps": round(copy_gbps, 1),
         "per_call": per_call,
     }
     print(json.dumps(out))
