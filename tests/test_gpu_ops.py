@@ -175,3 +175,50 @@ def test_reference_harness_flow(device):
     # the GEMV family: weight first
     row = harness.run_config([backend.fastgemv, backend.fastgemv_tuned], 1, 2048, 1024, warmup=1, iters=2)
     assert all(e["allclose"] for e in row["ops"].values())
+
+
+def test_operators_replay_correctly_from_a_hip_graph(device):
+    # serving loops capture the calls once and replay them: every launch (split-K second pass and
+    # in-launch completion included) must be capturable and give the eager result on each replay
+    import fastgate_amd
+    sg = fastgate_amd.speedgate
+    g = gen(4242)
+    K, N = 2048, 1024
+    Wkn = normal((K, N), g, 0.05).to(device)
+    Wnk = Wkn.t().contiguous()
+    Wq = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8).to(device)
+    acts = {M: normal((M, K), g, 1.0).to(device) for M in (1, 8, 16)}
+    outs = {k: torch.zeros((M, N), dtype=torch.half, device=device)
+            for k, M in (("kn1", 1), ("kn8", 8), ("kn16", 16), ("nk8", 8), ("nk16", 16), ("gemv", 1), ("i8", 1))}
+
+    def step():
+        sg.edgemm_m8n128k64x4(acts[1], Wkn, outs["kn1"])
+        sg.edgemm_m8n128k64x4(acts[8], Wkn, outs["kn8"])
+        sg.edgemm_m8n128k64x4(acts[16], Wkn, outs["kn16"])
+        sg.edgemm_m8n128k64x4_bt(acts[8], Wnk, outs["nk8"])
+        sg.edgemm_m8n128k64x4_bt(acts[16], Wnk, outs["nk16"])
+        sg.fastgemv(Wnk, acts[1], outs["gemv"])
+        sg.fastgemv_int8(Wq, acts[1], outs["i8"])
+
+    step()                      # eager: also sizes the cached workspace outside the capture
+    torch.cuda.synchronize()
+    want = {k: v.clone() for k, v in outs.items()}
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()                  # the capture stream gets its own workspace first
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            step()
+    torch.cuda.synchronize()
+    for replay in range(3):
+        for v in outs.values():
+            v.fill_(float("nan"))
+        # eager work of the program between replays
+        sg.edgemm_m8n128k64x4(acts[8], Wkn, torch.empty((8, N), dtype=torch.half, device=device))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for k in outs:
+            assert torch.equal(outs[k], want[k]), (replay, k)
