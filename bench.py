@@ -41,7 +41,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E peak
 # KiB per dispatch), keyed by kernel family and M.  Each counter is scaled by what it reads for
 # kernels of known traffic (--calibrate-traffic: a 1 GiB read and a 256 MiB copy): FETCH_SIZE
 # reports half the bytes on this part (factor 2.0), WRITE_SIZE all of them (factor 1.0).
-# The summaries are under profiles/.  A kernel/M not listed reports null.
+# A kernel/M not listed reports null.
 FETCH_SCALE, WRITE_SCALE = 2.0, 1.0
 
 

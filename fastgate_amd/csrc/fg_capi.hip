@@ -122,19 +122,19 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
   bool wide_tiles = false;  // ... in its 32-column form
   if (w_layout == FG_W_NK) {
     // Measured on MI355X at K = N = 8192 (us per call): M=1 dot2 tile 4: 21.6-22.4; M=4 dot2
-    // 24.3 / mfma4 22.1; M=8 dot2 27.8 / mfma4 26.2 / mfma16 29.2; M=16 mfma4 36 / mfma16 31.7.
-    // The shape sweep (K = N in 1024..16384 and the LLaMA / DiT shapes) behind these choices is
-    // summarised in profiles/; every rule below is the measured winner for its range.
-    if (M <= 2 || (M <= 4 && N <= 4096 && K >= 8192)) {
-      // (few, long rows at M = 3..4: v_dot2 16.3 us against 19.8 for N = 3072, K = 12288)
+    // 24.3 / mfma4 22.3; M=8 dot2 27.8 / mfma4 25.6 / row-load 23.3; M=16 mfma4 36 / direct
+    // 16x16x32 31.7 / transposing 27.3 / row-load 24.6.  Every rule below is the measured winner of
+    // a sweep over K = N in 1024..16384 and the LLaMA / DiT projection shapes for its range.
+    if (M <= 2 || (M <= 4 && N <= 2048 && K >= 8192)) {
+      // (few, long rows at M = 3..4: v_dot2 8.8-9.3 us against 9.4-9.5 for N = 2048, K = 8192)
       p->kernel = FG_KERNEL_NK_DOT2;
       p->m_block = M <= 2 ? M : 4;
       p->tile_n = 4;
       p->unroll = (K >= 16384 || M > 2) ? 2 : 1;
       items = ceil_div(K / 8, 64 * p->unroll);
       p->stagger = items <= 16;  // at most 4 steps for 4 waves
-    } else if (M <= 4 || (M <= 8 && K >= 16384)) {
-      // (K = N = 16384, M = 8: 77.5 us against 78.9 for the row-load kernel)
+    } else if (M <= 8 && K >= 16384) {
+      // (K = N = 16384: M = 4 78.7 us against 79.9 for the row-load kernel, M = 8 77.5 / 78.9)
       p->kernel = FG_KERNEL_NK_MFMA4;
       p->m_block = M <= 4 ? 4 : 8;
       if (K >= 16384) {
@@ -147,11 +147,13 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
       }
       items = ceil_div(K / 128, p->unroll);
     } else {
-      // M >= 5: 16-column tiles, weights and activations as contiguous row pieces through LDS,
+      // M >= 3: 16-column tiles, weights and activations as contiguous row pieces through LDS,
       // 8 waves on 256-byte bands.  Measured against the best of the other [N,K] kernels (us):
       // K = N = 8192 M=8 23.2 / 25.6, M=16 24.6 / 27.3; K=3072 N=12288 M=16 15.6 / 21.0;
       // K=12288 N=3072 M=16 19.1 / 20.3; K = N = 4096 M=8 7.8 / 9.5; K=4096 N=11008 M=8 16.5 / 20.1.
       // At K = 16384 four waves on 512-byte bands are level or slightly ahead (M=16 84.3 / 85.8).
+      // M = 3..4 against the 4x4x4 kernel: K = N = 4096 8.7-8.9 / 9.2-9.5, K = N = 8192 22.9 / 22.3-24.0,
+      // K=12288 N=3072 14.6 / 15.2-16.0, K=4096 N=11008 15.8 / 16.6-16.9.
       p->kernel = FG_KERNEL_NK_MFMA_R;
       p->m_block = 16;
       p->tile_n = 16;
