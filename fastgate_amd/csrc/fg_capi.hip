@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <cmath>
 #include <cstring>
 
 #include "fg_internal.h"
@@ -53,7 +54,11 @@ int validate_shape(int M, int N, int K, int w_layout) {
 
 // Fills grid/block/workspace from the tile fields; rejects tiles that were not built.
 int finish_plan(int M, int N, int K, fg_plan_t* p) {
-  const int max_waves = (p->kernel == FG_KERNEL_NK_MFMA_R && p->unroll == 1) ? 8 : 4;
+  const int max_waves =
+      ((p->kernel == FG_KERNEL_NK_MFMA_R && p->unroll == 1) || p->kernel == FG_KERNEL_KN_MFMA ||
+       (p->kernel == FG_KERNEL_KN_DOT2 && p->m_block <= 2))
+          ? 8
+          : 4;
   if (p->splitk < 1 || p->waves < 1 || p->waves > max_waves || (p->waves & (p->waves - 1))) {
     return FG_ERR_INVALID_ARG;
   }
@@ -190,7 +195,22 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
       // [K,N] tiles are 128 columns wide, so the grid needs split-K to cover the chip: the
       // factor that brings tiles*S closest to one workgroup per CU.
       int best = 1;
-      if ((size_t)N * K >= ((size_t)1 << 18)) {  // 1024 x 1024: 7.7 us with S = 8 against 9.0 without
+      if ((size_t)N * K < ((size_t)1 << 26) && items >= 16 && M <= 16) {
+        // Below 8192 x 8192 the call is latency-bound: 8 waves per workgroup and half the split
+        // (about 192 workgroups) shorten every wave's chain of dependent loads.  Measured (us,
+        // 4 waves / 8 waves, M = 4): K=N=4096 12.3 / 11.2, K=4096 N=11008 20.1 / 18.1,
+        // K=3072 N=12288 17.2 / 15.9, K=12288 N=3072 20.5 / 17.8, K=N=2048 12.3 / 8.8.
+        p->waves = 8;
+        double best_dist = 1e30;
+        for (int S = 1; S <= 16; S *= 2) {
+          if (items / (p->waves * S) < 1) break;
+          const double dist = std::fabs(std::log2((double)tiles * S / 192.0));
+          if (dist < best_dist - 1e-9) {
+            best_dist = dist;
+            best = S;
+          }
+        }
+      } else if ((size_t)N * K >= ((size_t)1 << 18)) {  // 1024 x 1024: 7.7 us with S = 8 against 9.0 without
         double best_ratio = 1e30;
         for (int S = 1; S <= 16; S *= 2) {
           if (items / (p->waves * S) < 1) break;

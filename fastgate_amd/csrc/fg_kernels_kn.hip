@@ -37,14 +37,14 @@ __device__ __forceinline__ void transpose8x8(const u32x4 (&rows)[8], u32x4 (&bt)
 // column index), so acc[i][r] = D[m = 4g + r][n = n0 + 8j + i]: a lane ends up with 8
 // consecutive columns per row, which makes the epilogue 16-byte stores.
 // ---------------------------------------------------------------------------------------
-template <int U, bool STREAM>
-__global__ __launch_bounds__(256) void kn_mfma_kernel(const half_t* __restrict__ A,
+template <int U, bool STREAM, int NW>
+__global__ __launch_bounds__(64 * NW) void kn_mfma_kernel(const half_t* __restrict__ A,
                                                       const half_t* __restrict__ W,
                                                       half_t* __restrict__ C,
                                                       float* __restrict__ ws, int* counters, int M, int N,
                                                       int K, int accumulate) {
   accumulate &= 1;  // the flag word also carries the stagger mode of the [N,K] kernels
-  __shared__ float red[4][16][128];
+  __shared__ float red[NW][16][128];  // NW = most waves per workgroup
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int nw = blockDim.x >> 6;
@@ -129,14 +129,14 @@ __global__ __launch_bounds__(256) void kn_mfma_kernel(const half_t* __restrict__
 // positions are one 16-byte load per row m (identical for the 16 lanes of a DPP row).
 // The four k-groups g of a wave are summed in LDS together with the waves.
 // ---------------------------------------------------------------------------------------
-template <int MB, int U, bool STREAM>
-__global__ __launch_bounds__(256) void kn_dot2_kernel(const half_t* __restrict__ A,
+template <int MB, int U, bool STREAM, int NW>
+__global__ __launch_bounds__(64 * NW) void kn_dot2_kernel(const half_t* __restrict__ A,
                                                       const half_t* __restrict__ W,
                                                       half_t* __restrict__ C,
                                                       float* __restrict__ ws, int* counters, int M, int N,
                                                       int K, int accumulate) {
   accumulate &= 1;  // the flag word also carries the stagger mode of the [N,K] kernels
-  __shared__ float red[16][MB][128];
+  __shared__ float red[4 * NW][MB][128];  // NW = most waves per workgroup
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int nw = blockDim.x >> 6;
@@ -221,11 +221,18 @@ static void kn_dot2_go(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
   auto* A = static_cast<const half_t*>(a.A);
   auto* W = static_cast<const half_t*>(a.W);
   auto* C = static_cast<half_t*>(a.C);
+  if constexpr (MB <= 2) {
+    if (p.waves == 8) {
+      hipLaunchKernelGGL((kn_dot2_kernel<MB, U, true, 8>), grid, block, 0, s, A, W, C, a.ws, a.counters, a.M,
+                         a.N, a.K, a.accumulate);
+      return;
+    }
+  }
   if (p.stream_w)
-    hipLaunchKernelGGL((kn_dot2_kernel<MB, U, true>), grid, block, 0, s, A, W, C, a.ws, a.counters, a.M, a.N,
+    hipLaunchKernelGGL((kn_dot2_kernel<MB, U, true, 4>), grid, block, 0, s, A, W, C, a.ws, a.counters, a.M, a.N,
                        a.K, a.accumulate);
   else
-    hipLaunchKernelGGL((kn_dot2_kernel<MB, U, false>), grid, block, 0, s, A, W, C, a.ws, a.counters, a.M, a.N,
+    hipLaunchKernelGGL((kn_dot2_kernel<MB, U, false, 4>), grid, block, 0, s, A, W, C, a.ws, a.counters, a.M, a.N,
                        a.K, a.accumulate);
 }
 
@@ -242,6 +249,7 @@ static bool kn_dot2_u(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
 }
 
 bool launch_kn_dot2(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
+  if (p.waves > 4 && p.m_block > 2) return false;  // 8 waves are built for one or two rows only
   switch (p.m_block) {
     case 1: return kn_dot2_u<1>(p, a, s);
     case 2: return kn_dot2_u<2>(p, a, s);
@@ -257,12 +265,16 @@ static void kn_mfma_go(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
   auto* A = static_cast<const half_t*>(a.A);
   auto* W = static_cast<const half_t*>(a.W);
   auto* C = static_cast<half_t*>(a.C);
-  if (p.stream_w)
-    hipLaunchKernelGGL((kn_mfma_kernel<U, true>), grid, block, 0, s, A, W, C, a.ws, a.counters, a.M, a.N, a.K,
+  if (p.waves == 8) {
+    hipLaunchKernelGGL((kn_mfma_kernel<U, true, 8>), grid, block, 0, s, A, W, C, a.ws, a.counters, a.M, a.N, a.K,
                        a.accumulate);
-  else
-    hipLaunchKernelGGL((kn_mfma_kernel<U, false>), grid, block, 0, s, A, W, C, a.ws, a.counters, a.M, a.N, a.K,
+  } else if (p.stream_w) {
+    hipLaunchKernelGGL((kn_mfma_kernel<U, true, 4>), grid, block, 0, s, A, W, C, a.ws, a.counters, a.M, a.N, a.K,
                        a.accumulate);
+  } else {
+    hipLaunchKernelGGL((kn_mfma_kernel<U, false, 4>), grid, block, 0, s, A, W, C, a.ws, a.counters, a.M, a.N, a.K,
+                       a.accumulate);
+  }
 }
 
 bool launch_kn_mfma(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
