@@ -138,7 +138,7 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
       p->unroll = (K >= 16384 || M > 2) ? 2 : 1;
       items = ceil_div(K / 8, 64 * p->unroll);
       p->stagger = items <= 16;  // at most 4 steps for 4 waves
-    } else if (M <= 8 && K >= 16384) {
+    } else if (M <= 8 && K >= 16384 && N >= 8192) {
       // (K = N = 16384: M = 4 78.7 us against 79.9 for the row-load kernel, M = 8 77.5 / 78.9)
       p->kernel = FG_KERNEL_NK_MFMA4;
       p->m_block = M <= 4 ? 4 : 8;
@@ -162,7 +162,7 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
       p->kernel = FG_KERNEL_NK_MFMA_R;
       p->m_block = 16;
       p->tile_n = 16;
-      p->unroll = K >= 16384 ? 2 : 1;
+      p->unroll = (K >= 16384 && N >= 8192) ? 2 : 1;
       if (M > 8 && K >= 8192 && N / 32 >= 2 * kCUs) {
         // plenty of tiles: two 16-column blocks share the staged activations, four waves
         // (K = N = 16384, M=16: 79.0 us against 84.8)
@@ -224,10 +224,14 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
       }
       p->splitk = best;
     } else if (row_tiles) {
-      // (K=12288 N=3072, 192 tiles, M=8: 16.0 us unsplit against 19.3 with S = 3)
-      int S = tiles >= kCUs / 2 ? 1 : ceil_div(kCUs, tiles);
+      // 192 tiles still run best unsplit (K=12288 N=3072 M=8: 16.0 us against 17.4 with S = 4);
+      // 128 tiles or fewer want two workgroups per CU once K is long (N=2048: K=8192 M=16
+      // 10.5 us with S = 2 against 12.4, K=16384 15.7 against 21.7).  The partials of a 16-column
+      // tile are small, so the split always completes inside the launch.
+      int S = (tiles > kCUs / 2 || K < 8192) ? 1 : ceil_div(kCUs, tiles);
       while (S > 1 && items / (p->waves * S) < 2) --S;  // keep two bands per wave
       p->splitk = S;
+      p->fused = 1;
     } else {
       p->splitk = pick_splitk(tiles, p->waves, items, M, N, K, kCUs);
     }
