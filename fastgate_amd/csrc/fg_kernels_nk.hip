@@ -405,13 +405,15 @@ __global__ __launch_bounds__(256) void nk_mfma_t_kernel(const half_t* __restrict
 // 16 rows x 64 B (operand order) or 4 rows x 256 B, a 16-row A costs as much as the weights;
 // read as whole contiguous row pieces it costs under 10 % (a load-only probe with 16 weight rows
 // and 16 activation rows per step: 24.5 us against 22.7 us without the activation rows, at
-// K = N = 8192).  So here a wave loads, per step, a 512-byte band (256 k) of the tile's 16 weight
-// rows and of the A rows -- two rows per instruction, 32 lanes x 16 B each -- parks both in
-// wave-private LDS strips (rows padded to 528 B: conflict-free in both directions) and reads them
-// back in operand order for 8 MFMAs.  The tile is only 16 columns wide, so N/16 workgroups fill
-// the chip without split-K and there is no second pass; the 4 waves of a workgroup interleave
-// over the bands of K and meet in LDS once at the end.  MH = instructions per step for A:
-// 4 covers M <= 8, 8 covers M <= 16.
+// K = N = 8192).  So here a wave loads, per step, a BAND-byte band (BAND/2 k) of the tile's weight
+// rows and of the A rows -- 64 lanes x 16 B cover 1024/BAND rows per instruction -- parks both in
+// wave-private LDS strips (rows padded by 16 B: conflict-free in both directions) and reads them
+// back in operand order for BAND/64 MFMAs per 16-column block.  The tile is only 16 (or, with
+// CB = 2, 32) columns wide, so N/16 workgroups fill the chip without split-K and there is no second
+// pass; the waves of a workgroup interleave over the bands of K and meet in LDS once at the end.
+// Occupancy decides the rest: 256-byte bands need 35 KB of LDS and about 100 VGPRs per four
+// waves, so two 8-wave workgroups fit a CU (16 waves per CU; M = 16 at K = N = 8192: 24.6 us
+// against 26.0 us with four waves on 512-byte bands).
 // ---------------------------------------------------------------------------------------
 template <int AROWS, int BAND, bool FULL, int NW, int CB>
 __global__ __launch_bounds__(64 * NW) void nk_mfma_r_kernel(const half_t* __restrict__ A,
