@@ -352,6 +352,7 @@ __global__ __launch_bounds__(256) void dequant_i32_f16_kernel(const int32_t* __r
 // The activations are paired the same way, (x_j, x_{j+4}), once per chunk.
 // Replaces gemv_quantized_int4 (backend/cuda/hk/fastgemv.cuh:394-495), which the reference
 // defines but never launches.  Lanes along K: one 16-byte load = 32 weights of one row.
+// Launched for one activation row; two to four rows take w4a16_r_kernel below.
 // ---------------------------------------------------------------------------------------
 template <int MB, int RN>
 __global__ __launch_bounds__(256) void w4a16_kernel(const uint8_t* __restrict__ Wq,
@@ -586,6 +587,131 @@ __global__ __launch_bounds__(64 * NW) void w8a16_r_kernel(const int8_t* __restri
 }
 
 // ---------------------------------------------------------------------------------------
+// w4a16 with both operands staged through wave-private LDS (4-bit sibling of w8a16_r_kernel).
+// A band is 512 k: 256 bytes of each of the tile's 16 weight rows (4 rows x 256 B per load
+// instruction) and 1 KB of each activation row (one row per instruction).  The activations are
+// parked already paired the way the nibble conversion produces its halves -- (x0,x4),(x1,x5),
+// (x2,x6),(x3,x7) per 8 k -- so the 4 bytes a lane reads per MFMA unit turn into the B operand with
+// one shift, four v_and_or and four exact fp16 subtractions, and the dot products run on the
+// matrix pipe.  XROWS = activation rows staged (2 or 4).
+// ---------------------------------------------------------------------------------------
+template <int XROWS>
+__global__ __launch_bounds__(512) void w4a16_r_kernel(const uint8_t* __restrict__ Wq,
+                                                      const half_t* __restrict__ X,
+                                                      const half_t* __restrict__ scale,
+                                                      float scalar_scale, float zero_point,
+                                                      half_t* __restrict__ Y, int M, int N, int K) {
+  constexpr int NW = 8;
+  constexpr int RSW = 256 + 16;      // LDS bytes per staged weight row (512 k)
+  constexpr int RSX = 1024 + 16;     // ... per staged activation row
+  constexpr int WSTRIP = 16 * RSW;
+  constexpr int XSTRIP = XROWS * RSX;
+  constexpr int WAVE_LDS = WSTRIP + XSTRIP;
+  static_assert(WAVE_LDS >= 2 * 256 * (int)sizeof(float), "reduction scratch fits");
+  __shared__ __attribute__((aligned(16))) unsigned char smem[NW * WAVE_LDS];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int nw = blockDim.x >> 6;
+  const int j = lane & 15, g = lane >> 4;        // operand order
+  const int hw = lane >> 4, cw = lane & 15;      // weight load order: row 4i + hw, piece cw (32 k)
+  const int n0 = blockIdx.x * 16;
+  const int nbands = (K + 511) >> 9;             // K % 128 == 0: the last band may be partial
+  const size_t rowb = (size_t)K >> 1;            // bytes per weight row
+  const bool use_zp = zero_point != 0.f;
+  unsigned char* wstrip = smem + wave * WAVE_LDS;
+  unsigned char* xstrip = wstrip + WSTRIP;
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+
+  const uint8_t* Wp = Wq + (size_t)(n0 + hw) * rowb + cw * 16;
+  const half_t* Xp = X + lane * 8;
+  const int stw_off = hw * RSW + cw * 16;
+  const int stx_off = lane * 16;
+  const int ldw_off = j * RSW + g * 4;
+  const int ldx_off = (j % XROWS) * RSX + g * 16;  // MFMA rows beyond XROWS re-read staged rows; unused
+
+  auto load_band = [&](int band, u32x4(&w)[4], u32x4(&x)[XROWS]) {
+    const bool okw = band < nbands && (band * 512 + cw * 32) < K;
+    const bool okx = band < nbands && (band * 512 + lane * 8) < K;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) w[i] = okw ? load16<true>(Wp + (size_t)(4 * i) * rowb + (size_t)band * 256) : zero;
+#pragma unroll
+    for (int i = 0; i < XROWS; ++i)
+      x[i] = (okx && i < M) ? load16<false>(Xp + (size_t)i * K + (size_t)band * 512) : zero;
+  };
+  float4_t acc = {0.f, 0.f, 0.f, 0.f}, xacc = {0.f, 0.f, 0.f, 0.f};
+  const half8_t ones8 = {static_cast<half_t>(1.f), static_cast<half_t>(1.f), static_cast<half_t>(1.f),
+                         static_cast<half_t>(1.f), static_cast<half_t>(1.f), static_cast<half_t>(1.f),
+                         static_cast<half_t>(1.f), static_cast<half_t>(1.f)};
+  const half2_t b1024 = {static_cast<half_t>(1024.f), static_cast<half_t>(1024.f)};
+  const half2_t b64 = {static_cast<half_t>(64.f), static_cast<half_t>(64.f)};
+  auto multiply = [&](const u32x4(&w)[4], const u32x4(&x)[XROWS]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(wstrip + stw_off + 4 * i * RSW) = w[i];
+#pragma unroll
+    for (int i = 0; i < XROWS; ++i) {
+      const u32x4 xv = x[i];  // x0..x7 -> (x0,x4) (x1,x5) (x2,x6) (x3,x7)
+      const u32x4 xp = {__builtin_amdgcn_perm(xv.z, xv.x, 0x05040100u), __builtin_amdgcn_perm(xv.z, xv.x, 0x07060302u),
+                        __builtin_amdgcn_perm(xv.w, xv.y, 0x05040100u), __builtin_amdgcn_perm(xv.w, xv.y, 0x07060302u)};
+      *reinterpret_cast<u32x4*>(xstrip + stx_off + i * RSX) = xp;
+    }
+    wave_lds_sync();
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+      const u32x4 xa = *reinterpret_cast<const u32x4*>(xstrip + ldx_off + u * 64);
+      const uint32_t wd = *reinterpret_cast<const uint32_t*>(wstrip + ldw_off + u * 16), w8 = wd >> 8;
+      const half2_t p0 = as_half2((wd & 0x000F000Fu) | 0x64006400u) - b1024;   // (n0, n4)
+      const half2_t p1 = as_half2((wd & 0x00F000F0u) | 0x54005400u) - b64;     // (n1, n5)
+      const half2_t p2 = as_half2((w8 & 0x000F000Fu) | 0x64006400u) - b1024;   // (n2, n6)
+      const half2_t p3 = as_half2((w8 & 0x00F000F0u) | 0x54005400u) - b64;     // (n3, n7)
+      const half8_t wb = {p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(xa), wb, acc, 0, 0, 0);
+      if (use_zp) xacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(xa), ones8, xacc, 0, 0, 0);
+    }
+    wave_lds_sync();
+  };
+
+  u32x4 w0[4], w1[4], x0[XROWS], x1[XROWS];
+  const int nsteps = (nbands + nw - 1) / nw;
+  int step = stagger_start(nsteps, 0);
+  auto next_band = [&]() {
+    const int band = step * nw + wave;
+    step = step + 1 == nsteps ? 0 : step + 1;
+    return band;
+  };
+  load_band(next_band(), w0, x0);
+  for (int it = 0; it < nsteps; it += 2) {
+    if (it + 1 < nsteps) load_band(next_band(), w1, x1);
+    multiply(w0, x0);
+    if (it + 1 >= nsteps) break;
+    if (it + 2 < nsteps) load_band(next_band(), w0, x0);
+    multiply(w1, x1);
+  }
+
+  // acc[r] = D[m = 4g + r][column j] (xacc: sum of x of row m in every column); waves meet in LDS
+  __syncthreads();
+  float(*red)[2][256] = reinterpret_cast<float(*)[2][256]>(smem);
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    red[wave][0][(4 * g + r) * 16 + j] = acc[r];
+    red[wave][1][(4 * g + r) * 16 + j] = xacc[r];
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < 256; e += blockDim.x) {
+    const int m = e >> 4, n = n0 + (e & 15);
+    if (m < M) {
+      float sum = 0.f, xs = 0.f;
+      for (int wv = 0; wv < nw; ++wv) {
+        sum += red[wv][0][e];
+        xs += red[wv][1][e];
+      }
+      float sc = scalar_scale;
+      if (scale != nullptr) sc *= static_cast<float>(scale[n]);
+      Y[(size_t)m * N + n] = static_cast<half_t>((sum - zero_point * xs) * sc);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
 // Host launchers.  Rows per workgroup: 8 when that still yields >= 512 workgroups, else 4.
 // Waves per workgroup: as many (<= 4) as the row has 1 KB pieces.
 // ---------------------------------------------------------------------------------------
@@ -626,16 +752,20 @@ bool launch_w4a16(const W8A16Args& a, hipStream_t s) {
   auto* X = static_cast<const half_t*>(a.x);
   auto* sc = static_cast<const half_t*>(a.scale);
   auto* Y = static_cast<half_t*>(a.y);
-  const int pieces = (a.K / 32 + 63) / 64;  // 1 KB pieces per weight row
-  const dim3 block(64 * (pieces >= 4 ? 4 : (pieces >= 2 ? 2 : 1)));
-#define W4(MB) \
-  hipLaunchKernelGGL((w4a16_kernel<MB, 4>), dim3(a.N / 4), block, 0, s, Wq, X, sc, a.scalar_scale, \
-                     a.zero_point, Y, a.M, a.N, a.K)
-  if (a.M == 1) W4(1);
-  else if (a.M == 2) W4(2);
-  else if (a.M <= 4) W4(4);
-  else return false;
-#undef W4
+  if (a.M < 1 || a.M > 4) return false;
+  if (a.M == 1) {
+    // one activation row: the dot2 kernel's straight 1 KB row pieces are the shorter path
+    const int pieces = (a.K / 32 + 63) / 64;  // 1 KB pieces per weight row
+    const dim3 block(64 * (pieces >= 4 ? 4 : (pieces >= 2 ? 2 : 1)));
+    hipLaunchKernelGGL((w4a16_kernel<1, 4>), dim3(a.N / 4), block, 0, s, Wq, X, sc, a.scalar_scale,
+                       a.zero_point, Y, a.M, a.N, a.K);
+  } else if (a.M == 2) {
+    hipLaunchKernelGGL((w4a16_r_kernel<2>), dim3(a.N / 16), dim3(512), 0, s, Wq, X, sc, a.scalar_scale,
+                       a.zero_point, Y, a.M, a.N, a.K);
+  } else {
+    hipLaunchKernelGGL((w4a16_r_kernel<4>), dim3(a.N / 16), dim3(512), 0, s, Wq, X, sc, a.scalar_scale,
+                       a.zero_point, Y, a.M, a.N, a.K);
+  }
   return true;
 }
 

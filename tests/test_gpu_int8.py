@@ -175,9 +175,10 @@ def test_w4a16_matches_oracle(device, M, N, K):
     assert_close_f16(_w4a16(Wq4, x, scale, 0.5, 7.5, device), ref, "scale 0.5 zp 7.5")
 
 
-def test_w4a16_every_nibble_in_every_position_is_exact(device):
+@pytest.mark.parametrize("M", [1, 2, 4])
+def test_w4a16_every_nibble_in_every_position_is_exact(device, M):
     # x = e_k picks single weights: the result must be the nibble itself, for all 32 positions of
-    # a 16-byte load and all 16 values
+    # a 16-byte load and all 16 values (M = 1 runs the dot2 kernel, M >= 2 the row-load kernels)
     N, K = 128, 128
     Wq4 = torch.zeros((N, K // 2), dtype=torch.uint8)
     for n in range(N):
@@ -187,13 +188,31 @@ def test_w4a16_every_nibble_in_every_position_is_exact(device):
     want = np.empty((N, K), np.float32)
     want[:, 0::2] = (Wq4 & 0x0F).numpy()
     want[:, 1::2] = (Wq4 >> 4).numpy()
-    for k in range(0, K, 4):
-        x = torch.zeros((4, K), dtype=torch.half)
-        for m in range(4):
+    for k in range(0, K, M):
+        x = torch.zeros((M, K), dtype=torch.half)
+        for m in range(M):
             x[m, k + m] = 1.0
         got = _w4a16(Wq4, x, None, 1.0, 0.0, device)
-        for m in range(4):
+        for m in range(M):
             assert (got[m] == want[:, k + m]).all(), (k, m)
+
+
+def test_w4a16_row_load_band_positions_are_exact(device):
+    # a 512-element band and its partial successor: single weights picked out at positions spread
+    # over both, with a zero point, must come back exactly
+    g = gen(955)
+    N, K = 128, 512 + 256
+    Wq4 = torch.randint(0, 256, (N, K // 2), generator=g, dtype=torch.uint8)
+    want = np.empty((N, K), np.float32)
+    want[:, 0::2] = (Wq4 & 0x0F).numpy()
+    want[:, 1::2] = (Wq4 >> 4).numpy()
+    for k in range(0, K - 3, 37):
+        x = torch.zeros((3, K), dtype=torch.half)
+        for m in range(3):
+            x[m, k + m] = 1.0
+        got = _w4a16(Wq4, x, None, 1.0, 8.0, device)
+        for m in range(3):
+            assert (got[m] == want[:, k + m] - 8.0).all(), (k, m)
 
 
 def test_w4a16_small_integers_are_exact(device):
