@@ -157,6 +157,35 @@ def run_sweep(torch, sg, capi, dev, steps, warmup):
                  "weights_per_ns": round(Kk * Nn / us_i4 / 1e3, 3),
                  "fp16_M1_weights_per_ns": round(Kk * Nn / us_f16 / 1e3, 3),
                  "weight_throughput_vs_fp16": round(us_f16 / us_i4, 3)})
+    # beyond the benchmark's configurations: the feed-forward pair of C3 (16 x 3072 x 12288, then
+    # 16 x 12288 x 3072) with bias and GELU, fused into the two GEMM launches against the same two
+    # GEMMs followed by separate elementwise launches
+    del wq4
+    g = torch.Generator(device=dev).manual_seed(1003)
+    Mf, Kf, Nf, nb = 16, 3072, 12288, 5
+    w1 = [(torch.randn((Nf, Kf), device=dev, generator=g) * 0.02).half() for _ in range(nb)]
+    w2 = [(torch.randn((Kf, Nf), device=dev, generator=g) * 0.02).half() for _ in range(nb)]
+    b1 = torch.randn(Nf, device=dev, generator=g).half()
+    b2 = torch.randn(Kf, device=dev, generator=g).half()
+    af = torch.randn((Mf, Kf), device=dev, generator=g).half()
+    hf = torch.empty((Mf, Nf), dtype=torch.half, device=dev)
+    cf = torch.empty((Mf, Kf), dtype=torch.half, device=dev)
+    us_fused = time_us(lambda i: sg.ffn_bt(af, w1[i % nb], b1, w2[i % nb], b2, hf, cf, "gelu"))
+
+    def unfused(i):
+        sg.gemm_m8n128k64x4_bt(af, w1[i % nb], hf)
+        h = torch.nn.functional.gelu(hf + b1)
+        sg.gemm_m8n128k64x4_bt(h, w2[i % nb], cf)
+        cf.add_(b2)
+
+    us_unfused = time_us(unfused)
+    by = 2 * (2 * Kf * Nf) + 2 * Mf * Kf * 2 + 2 * Mf * Nf * 2 + 2 * Nf + 2 * Kf
+    rows.append({"config": "extra: FFN pair, bias + GELU fused", "op": "ffn_bt", "M": Mf, "K": Kf, "N": Nf,
+                 "w_layout": "[N,K] twice", "seed": 1003, "kernel": "nk_mfma_r x2", "splitk": "-", "bytes": by,
+                 "us_per_call": round(us_fused, 2), "GBps": round(by / us_fused / 1e3, 1),
+                 "frac_hbm_peak": round(by / us_fused / 1e3 / HBM_PEAK_GBPS, 4),
+                 "frac_read_ceiling": round(by / us_fused / 1e3 / ceiling, 4),
+                 "us_unfused_with_torch_elementwise": round(us_unfused, 2)})
     return {"sweep": rows, "read_ceiling_GBps": round(ceiling, 1), "hbm_peak_GBps": HBM_PEAK_GBPS,
             "steps": steps, "warmup": warmup, "data": "synthetic", "dtype": "f16",
             "device": torch.cuda.get_device_name(0)}

@@ -31,12 +31,15 @@ FG_KERNEL_KN_MFMA = 4
 FG_KERNEL_NK_MFMA4 = 5
 FG_KERNEL_NK_MFMA_T = 7
 FG_KERNEL_NK_MFMA_R = 8
+FG_ACT_NONE, FG_ACT_RELU, FG_ACT_GELU, FG_ACT_GELU_TANH, FG_ACT_SILU = range(5)
+ACT_IDS = {"none": 0, "relu": 1, "gelu": 2, "gelu_tanh": 3, "silu": 4}
 KERNEL_NAMES = {1: "nk_dot2", 2: "nk_mfma", 3: "kn_dot2", 4: "kn_mfma", 5: "nk_mfma4", 7: "nk_mfma_t", 8: "nk_mfma_r"}
 
 # Every symbol include/fastgate.h declares.
 EXPORTS = (
     "fg_gemm_f16",
     "fg_gemm_f16_planned",
+    "fg_gemm_f16_bias_act",
     "fg_plan",
     "fg_workspace_bytes",
     "fg_workspace_header_bytes",
@@ -101,6 +104,8 @@ def lib() -> ctypes.CDLL:
         L.fg_gemm_f16.argtypes = [vp, vp, vp, ci, ci, ci, ci, ci, ci, vp, sz, vp]
         L.fg_gemm_f16_planned.restype = ci
         L.fg_gemm_f16_planned.argtypes = [vp, vp, vp, ci, ci, ci, ci, ci, pp, vp, sz, vp]
+        L.fg_gemm_f16_bias_act.restype = ci
+        L.fg_gemm_f16_bias_act.argtypes = [vp, vp, vp, ci, vp, ci, ci, ci, ci, ci, pp, vp, sz, vp]
         L.fg_plan.restype = ci
         L.fg_plan.argtypes = [ci, ci, ci, ci, ci, pp]
         L.fg_workspace_bytes.restype = sz

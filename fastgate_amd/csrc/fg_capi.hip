@@ -241,14 +241,17 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
 
 int check_launch() { return hipGetLastError() == hipSuccess ? FG_OK : FG_ERR_LAUNCH; }
 
+// `tail`: bias and activation bits of the kernels' flag word (0 for a plain product).
 int run_gemm(const void* A, const void* W, void* C, int M, int N, int K, int accumulate,
-             const fg_plan_t& p, void* ws, size_t ws_bytes, hipStream_t s) {
+             const fg_plan_t& p, void* ws, size_t ws_bytes, hipStream_t s, int tail = 0,
+             const void* bias = nullptr) {
   if (p.splitk > 1 && (ws == nullptr || ws_bytes < p.workspace_bytes)) return FG_ERR_WORKSPACE;
   if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(W) |
        reinterpret_cast<uintptr_t>(C) | reinterpret_cast<uintptr_t>(ws)) & 15) {
     return FG_ERR_INVALID_ARG;  // 16-byte loads and stores
   }
-  GemmArgs a{A, W, C, nullptr, nullptr, M, N, K, (accumulate ? 1 : 0) | (p.stagger ? 2 : 0)};
+  GemmArgs a{A, W, C, nullptr, nullptr, M, N, K,
+             (accumulate ? kFlagAccumulate : 0) | (p.stagger ? kFlagStagger : 0) | tail, bias};
   if (p.splitk > 1) {
     a.ws = reinterpret_cast<float*>(static_cast<unsigned char*>(ws) + kWsHeaderBytes);
     a.counters = p.fused ? static_cast<int*>(ws) : nullptr;
@@ -268,7 +271,7 @@ int run_gemm(const void* A, const void* W, void* C, int M, int N, int K, int acc
   if (!ok) return FG_ERR_UNSUPPORTED;
   if (check_launch() != FG_OK) return FG_ERR_LAUNCH;
   if (p.splitk > 1 && !p.fused) {
-    launch_splitk_reduce(a.ws, C, p.splitk, M, N, a.accumulate & 1, s);
+    launch_splitk_reduce(a.ws, C, p.splitk, M, N, a.accumulate, a.bias, s);
     if (check_launch() != FG_OK) return FG_ERR_LAUNCH;
   }
   return FG_OK;
@@ -347,6 +350,33 @@ int fg_gemm_f16_planned(const void* A, const void* W, void* C, int M, int N, int
   if (st != FG_OK) return st;
   return fg::run_gemm(A, W, C, M, N, K, accumulate, *plan, ws, ws_bytes,
                       static_cast<hipStream_t>(stream));
+}
+
+int fg_gemm_f16_bias_act(const void* A, const void* W, const void* bias, int act, void* C, int M,
+                         int N, int K, int w_layout, int splitk, fg_plan_t* plan, void* ws,
+                         size_t ws_bytes, void* stream) {
+  if (A == nullptr || W == nullptr || C == nullptr) return FG_ERR_INVALID_ARG;
+  if (act < FG_ACT_NONE || act > FG_ACT_SILU) return FG_ERR_INVALID_ARG;
+  if (reinterpret_cast<uintptr_t>(bias) & 1) return FG_ERR_INVALID_ARG;
+  const int tail = (bias != nullptr ? fg::kFlagBias : 0) | (act << fg::kFlagActShift);
+  fg_plan_t p;
+  int st;
+  if (plan == nullptr) {
+    st = fg_plan(M, N, K, w_layout, splitk, &p);
+    if (st != FG_OK) return st;
+    plan = &p;
+  } else {
+    st = fg::validate_shape(M, N, K, w_layout);
+    if (st != FG_OK) return st;
+    if ((w_layout == FG_W_NK && !fg::is_nk(plan->kernel)) ||
+        (w_layout == FG_W_KN && !fg::is_kn(plan->kernel))) {
+      return FG_ERR_UNSUPPORTED;
+    }
+    st = fg::finish_plan(M, N, K, plan);
+    if (st != FG_OK) return st;
+  }
+  return fg::run_gemm(A, W, C, M, N, K, 0, *plan, ws, ws_bytes, static_cast<hipStream_t>(stream),
+                      tail, bias);
 }
 
 int fg_gemv_w8a16(const void* Wq, const void* x, const void* scale, float scalar_scale,

@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "fg_flags.h"
+
 namespace fg {
 
 typedef _Float16 half_t;
@@ -136,6 +138,37 @@ __device__ __forceinline__ float4_t load_partial4(const float* base, size_t idx)
                                           partials_rsrc(base), (int)(idx * 4), 0, kCachePolicyAgent));
 }
 
+// ---------------------------------------------------------------------------------------
+// Value written to C.  The flag word of a launch: bit 0 C += (accumulate), bit 1 start stagger
+// of the [N,K] kernels, bit 4 add bias[n] (fp16, one per output column), bits 5-7 activation
+// (FG_ACT_*).  Bias and activation are applied in fp32 to the finished sum, before the single
+// rounding to fp16.
+// ---------------------------------------------------------------------------------------
+__device__ __forceinline__ float activate(float v, int act) {
+  switch (act) {
+    case FG_ACT_RELU: return v > 0.f ? v : 0.f;
+    case FG_ACT_GELU: return 0.5f * v * (1.f + erff(v * 0.70710678118654752f));
+    case FG_ACT_GELU_TANH: {
+      const float u = 0.79788456080286536f * (v + 0.044715f * v * v * v);
+      return 0.5f * v * (1.f + tanhf(u));
+    }
+    case FG_ACT_SILU: return v / (1.f + __expf(-v));
+    default: return v;
+  }
+}
+__device__ __forceinline__ float apply_tail(float v, int n, const void* bias, int flags) {
+  if (flags & kFlagTailMask) {
+    if (flags & kFlagBias) v += static_cast<float>(static_cast<const half_t*>(bias)[n]);
+    v = activate(v, (flags >> kFlagActShift) & 7);
+  }
+  return v;
+}
+__device__ __forceinline__ half_t finish_value(float sum, const half_t* c, int n, const void* bias,
+                                               int flags) {
+  if (flags & kFlagAccumulate) sum += static_cast<float>(*c);
+  return static_cast<half_t>(apply_tail(sum, n, bias, flags));
+}
+
 __device__ __forceinline__ bool splitk_last_arriver(int* counter, int S) {
   __shared__ int s_last;
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // partial stores have completed
@@ -154,7 +187,7 @@ __device__ __forceinline__ bool splitk_last_arriver(int* counter, int S) {
 // C[m0..m0+mcnt)[n0..n0+ncnt) = fp16( Σ_z part[z] (+ C) ); ncnt and n0 are multiples of 4.
 __device__ __forceinline__ void splitk_reduce_tile(const float* part, half_t* C, int S, int M, int N,
                                                    int m0, int mcnt, int n0, int ncnt,
-                                                   int accumulate) {
+                                                   int flags, const void* bias) {
   typedef half_t half4v __attribute__((ext_vector_type(4)));
   const int nq = ncnt >> 2;
   const size_t MN = (size_t)M * N;
@@ -165,14 +198,14 @@ __device__ __forceinline__ void splitk_reduce_tile(const float* part, half_t* C,
     float4_t sum = {0.f, 0.f, 0.f, 0.f};
     for (int z = 0; z < S; ++z) sum += load_partial4(part, (size_t)z * MN + off);
     half4v* c = reinterpret_cast<half4v*>(C + off);
-    if (accumulate) {
+    if (flags & kFlagAccumulate) {
       const half4v old = *c;
 #pragma unroll
       for (int k = 0; k < 4; ++k) sum[k] += static_cast<float>(old[k]);
     }
     half4v out;
 #pragma unroll
-    for (int k = 0; k < 4; ++k) out[k] = static_cast<half_t>(sum[k]);
+    for (int k = 0; k < 4; ++k) out[k] = static_cast<half_t>(apply_tail(sum[k], n + k, bias, flags));
     *c = out;
   }
 }
@@ -182,10 +215,10 @@ __device__ __forceinline__ void splitk_reduce_tile(const float* part, half_t* C,
 // without counters a second kernel does.
 template <int MROWS, int NCOLS>
 __device__ __forceinline__ void finish_splitk(float* ws, int* counters, half_t* C, int M, int N,
-                                              int m0, int n0, int accumulate) {
+                                              int m0, int n0, int flags, const void* bias) {
   if (gridDim.z > 1 && counters != nullptr) {
     if (splitk_last_arriver(counters + blockIdx.y * gridDim.x + blockIdx.x, gridDim.z))
-      splitk_reduce_tile(ws, C, gridDim.z, M, N, m0, MROWS, n0, NCOLS, accumulate);
+      splitk_reduce_tile(ws, C, gridDim.z, M, N, m0, MROWS, n0, NCOLS, flags, bias);
   }
 }
 

@@ -7,7 +7,7 @@
 #include <stddef.h>
 #include <stdint.h>
 
-#include "../../include/fastgate.h"
+#include "fg_flags.h"
 
 namespace fg {
 
@@ -18,7 +18,9 @@ struct GemmArgs {
   float* ws;      // fp32 [S,M,N] partials when plan.splitk > 1
   int* counters;  // per-tile arrival counters (fused split-K) or null (second-pass kernel)
   int M, N, K;
-  int accumulate;  // bit 0: C += A*W; bit 1: plan.stagger (start step = workgroup id % steps)
+  int accumulate;  // flag word: bit 0 C += A*W; bit 1 plan.stagger (start step = workgroup id %
+                   // steps); bit 4 add bias; bits 5-7 activation (FG_ACT_*)
+  const void* bias;  // fp16 [N] when bit 4 is set
 };
 
 // Tile sets that exist as instantiations (the planner and the validators share these).
@@ -38,9 +40,10 @@ bool launch_nk_mfma_r(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
 bool launch_kn_dot2(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
 bool launch_kn_mfma(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
 
-// Second pass of split-K: C[m,n] = fp16( Σ_s ws[s,m,n] (+ C[m,n]) ), fixed summation order.
-void launch_splitk_reduce(const float* ws, void* C, int S, int M, int N, int accumulate,
-                          hipStream_t s);
+// Second pass of split-K: C[m,n] = fp16( tail( Σ_s ws[s,m,n] (+ C[m,n]) ) ), fixed summation
+// order; `flags` and `bias` as in GemmArgs.
+void launch_splitk_reduce(const float* ws, void* C, int S, int M, int N, int flags,
+                          const void* bias, hipStream_t s);
 
 struct W8A16Args {
   const void* Wq;     // int8 [N,K]

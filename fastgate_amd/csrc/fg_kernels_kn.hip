@@ -42,8 +42,7 @@ __global__ __launch_bounds__(64 * NW) void kn_mfma_kernel(const half_t* __restri
                                                       const half_t* __restrict__ W,
                                                       half_t* __restrict__ C,
                                                       float* __restrict__ ws, int* counters, int M, int N,
-                                                      int K, int accumulate) {
-  accumulate &= 1;  // the flag word also carries the stagger mode of the [N,K] kernels
+                                                      int K, int flags, const void* bias) {
   __shared__ float red[NW][16][128];  // NW = most waves per workgroup
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -106,13 +105,13 @@ __global__ __launch_bounds__(64 * NW) void kn_mfma_kernel(const half_t* __restri
       if (gridDim.z == 1) {
         half_t* c = C + (size_t)mg * N + n0 + c0;
         half8_t out;
-        if (accumulate) {
+        if (flags & kFlagAccumulate) {
           const half8_t old = *reinterpret_cast<const half8_t*>(c);
 #pragma unroll
           for (int i = 0; i < 8; ++i) sum[i] += static_cast<float>(old[i]);
         }
 #pragma unroll
-        for (int i = 0; i < 8; ++i) out[i] = static_cast<half_t>(sum[i]);
+        for (int i = 0; i < 8; ++i) out[i] = static_cast<half_t>(apply_tail(sum[i], n0 + c0 + i, bias, flags));
         *reinterpret_cast<half8_t*>(c) = out;
       } else {
         const size_t o = ((size_t)blockIdx.z * M + mg) * N + n0 + c0;
@@ -121,7 +120,7 @@ __global__ __launch_bounds__(64 * NW) void kn_mfma_kernel(const half_t* __restri
       }
     }
   }
-  finish_splitk<16, 128>(ws, counters, C, M, N, m0, n0, accumulate);
+  finish_splitk<16, 128>(ws, counters, C, M, N, m0, n0, flags, bias);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -134,8 +133,7 @@ __global__ __launch_bounds__(64 * NW) void kn_dot2_kernel(const half_t* __restri
                                                       const half_t* __restrict__ W,
                                                       half_t* __restrict__ C,
                                                       float* __restrict__ ws, int* counters, int M, int N,
-                                                      int K, int accumulate) {
-  accumulate &= 1;  // the flag word also carries the stagger mode of the [N,K] kernels
+                                                      int K, int flags, const void* bias) {
   __shared__ float red[4 * NW][MB][128];  // NW = most waves per workgroup
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -196,14 +194,13 @@ __global__ __launch_bounds__(64 * NW) void kn_dot2_kernel(const half_t* __restri
     if (mg < M) {
       if (gridDim.z == 1) {
         half_t* c = C + (size_t)mg * N + n;
-        if (accumulate) sum += static_cast<float>(*c);
-        *c = static_cast<half_t>(sum);
+        *c = finish_value(sum, c, n, bias, flags);
       } else {
         store_partial(ws + ((size_t)blockIdx.z * M + mg) * N + n, sum, counters != nullptr);
       }
     }
   }
-  finish_splitk<MB, 128>(ws, counters, C, M, N, m0, n0, accumulate);
+  finish_splitk<MB, 128>(ws, counters, C, M, N, m0, n0, flags, bias);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -224,16 +221,16 @@ static void kn_dot2_go(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
   if constexpr (MB <= 2) {
     if (p.waves == 8) {
       hipLaunchKernelGGL((kn_dot2_kernel<MB, U, true, 8>), grid, block, 0, s, A, W, C, a.ws, a.counters, a.M,
-                         a.N, a.K, a.accumulate);
+                         a.N, a.K, a.accumulate, a.bias);
       return;
     }
   }
   if (p.stream_w)
     hipLaunchKernelGGL((kn_dot2_kernel<MB, U, true, 4>), grid, block, 0, s, A, W, C, a.ws, a.counters, a.M, a.N,
-                       a.K, a.accumulate);
+                       a.K, a.accumulate, a.bias);
   else
     hipLaunchKernelGGL((kn_dot2_kernel<MB, U, false, 4>), grid, block, 0, s, A, W, C, a.ws, a.counters, a.M, a.N,
-                       a.K, a.accumulate);
+                       a.K, a.accumulate, a.bias);
 }
 
 template <int MB>
@@ -267,13 +264,13 @@ static void kn_mfma_go(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
   auto* C = static_cast<half_t*>(a.C);
   if (p.waves == 8) {
     hipLaunchKernelGGL((kn_mfma_kernel<U, true, 8>), grid, block, 0, s, A, W, C, a.ws, a.counters, a.M, a.N, a.K,
-                       a.accumulate);
+                       a.accumulate, a.bias);
   } else if (p.stream_w) {
     hipLaunchKernelGGL((kn_mfma_kernel<U, true, 4>), grid, block, 0, s, A, W, C, a.ws, a.counters, a.M, a.N, a.K,
-                       a.accumulate);
+                       a.accumulate, a.bias);
   } else {
     hipLaunchKernelGGL((kn_mfma_kernel<U, false, 4>), grid, block, 0, s, A, W, C, a.ws, a.counters, a.M, a.N, a.K,
-                       a.accumulate);
+                       a.accumulate, a.bias);
   }
 }
 

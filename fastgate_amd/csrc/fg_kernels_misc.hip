@@ -5,34 +5,36 @@
 
 namespace fg {
 
-// C[m,n] = fp16( Σ_{s<S} ws[s,m,n] (+ C[m,n]) ), s ascending: the result does not depend on
+// C[m,n] = fp16( tail( Σ_{s<S} ws[s,m,n] (+ C[m,n]) ) ), s ascending: the result does not depend on
 // the order in which the first-pass workgroups finished.  Four columns per thread.
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ ws,
                                                             half_t* __restrict__ C, int S,
-                                                            size_t MN, int accumulate) {
+                                                            size_t MN, int N, int flags,
+                                                            const void* bias) {
   const size_t i = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
   if (i >= MN) return;
   float4_t sum = *reinterpret_cast<const float4_t*>(ws + i);
   for (int s = 1; s < S; ++s) sum += *reinterpret_cast<const float4_t*>(ws + (size_t)s * MN + i);
   typedef half_t half4_t __attribute__((ext_vector_type(4)));
   half4_t* c = reinterpret_cast<half4_t*>(C + i);
-  if (accumulate) {
+  if (flags & kFlagAccumulate) {
     const half4_t old = *c;
 #pragma unroll
     for (int k = 0; k < 4; ++k) sum[k] += static_cast<float>(old[k]);
   }
+  const int n = (int)(i % (size_t)N);  // N % 4 == 0: the four columns share a row
   half4_t out;
 #pragma unroll
-  for (int k = 0; k < 4; ++k) out[k] = static_cast<half_t>(sum[k]);
+  for (int k = 0; k < 4; ++k) out[k] = static_cast<half_t>(apply_tail(sum[k], n + k, bias, flags));
   *c = out;
 }
 
-void launch_splitk_reduce(const float* ws, void* C, int S, int M, int N, int accumulate,
-                          hipStream_t s) {
+void launch_splitk_reduce(const float* ws, void* C, int S, int M, int N, int flags,
+                          const void* bias, hipStream_t s) {
   const size_t MN = (size_t)M * N;  // N % 128 == 0, so MN % 4 == 0
   const unsigned blocks = (unsigned)((MN / 4 + 255) / 256);
   hipLaunchKernelGGL(splitk_reduce_kernel, dim3(blocks), dim3(256), 0, s, ws,
-                     static_cast<half_t*>(C), S, MN, accumulate);
+                     static_cast<half_t*>(C), S, MN, N, flags, bias);
 }
 
 // Read-only streaming probe.  Each workgroup owns 64 KB of contiguous input and walks it in

@@ -25,8 +25,7 @@ __global__ __launch_bounds__(256) void nk_dot2_kernel(const half_t* __restrict__
                                                       const half_t* __restrict__ W,
                                                       half_t* __restrict__ C,
                                                       float* __restrict__ ws, int* counters, int M,
-                                                      int N, int K, int flags) {
-  const int accumulate = flags & 1;  // bit 1 of flags selects the start stagger
+                                                      int N, int K, int flags, const void* bias) {
   __shared__ float red[16][RN * MB];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -90,14 +89,13 @@ __global__ __launch_bounds__(256) void nk_dot2_kernel(const half_t* __restrict__
     if (mg < M) {
       if (gridDim.z == 1) {
         half_t* c = C + (size_t)mg * N + n;
-        if (accumulate) sum += static_cast<float>(*c);
-        *c = static_cast<half_t>(sum);
+        *c = finish_value(sum, c, n, bias, flags);
       } else {
         store_partial(ws + ((size_t)blockIdx.z * M + mg) * N + n, sum, counters != nullptr);
       }
     }
   }
-  finish_splitk<MB, RN>(ws, counters, C, M, N, m0, n0, accumulate);
+  finish_splitk<MB, RN>(ws, counters, C, M, N, m0, n0, flags, bias);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -112,8 +110,7 @@ __global__ __launch_bounds__(256) void nk_mfma_kernel(const half_t* __restrict__
                                                       const half_t* __restrict__ W,
                                                       half_t* __restrict__ C,
                                                       float* __restrict__ ws, int* counters, int M,
-                                                      int N, int K, int flags) {
-  const int accumulate = flags & 1;  // bit 1 of flags selects the start stagger
+                                                      int N, int K, int flags, const void* bias) {
   __shared__ float red[4][TNW][256];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -172,14 +169,13 @@ __global__ __launch_bounds__(256) void nk_mfma_kernel(const half_t* __restrict__
     if (mg < M) {
       if (gridDim.z == 1) {
         half_t* c = C + (size_t)mg * N + n;
-        if (accumulate) sum += static_cast<float>(*c);
-        *c = static_cast<half_t>(sum);
+        *c = finish_value(sum, c, n, bias, flags);
       } else {
         store_partial(ws + ((size_t)blockIdx.z * M + mg) * N + n, sum, counters != nullptr);
       }
     }
   }
-  finish_splitk<16, 16 * TNW>(ws, counters, C, M, N, m0, n0, accumulate);
+  finish_splitk<16, 16 * TNW>(ws, counters, C, M, N, m0, n0, flags, bias);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -205,8 +201,7 @@ __global__ __launch_bounds__(256) void nk_mfma4_kernel(const half_t* __restrict_
                                                        const half_t* __restrict__ W,
                                                        half_t* __restrict__ C,
                                                        float* __restrict__ ws, int* counters, int M,
-                                                       int N, int K, int flags) {
-  const int accumulate = flags & 1;  // bit 1 of flags selects the start stagger
+                                                       int N, int K, int flags, const void* bias) {
   __shared__ float red[16][R4 * MG * 16];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -281,14 +276,13 @@ __global__ __launch_bounds__(256) void nk_mfma4_kernel(const half_t* __restrict_
     if (mg < M) {
       if (gridDim.z == 1) {
         half_t* c = C + (size_t)mg * N + n;
-        if (accumulate) sum += static_cast<float>(*c);
-        *c = static_cast<half_t>(sum);
+        *c = finish_value(sum, c, n, bias, flags);
       } else {
         store_partial(ws + ((size_t)blockIdx.z * M + mg) * N + n, sum, counters != nullptr);
       }
     }
   }
-  finish_splitk<4 * MG, 4 * R4>(ws, counters, C, M, N, m0, n0, accumulate);
+  finish_splitk<4 * MG, 4 * R4>(ws, counters, C, M, N, m0, n0, flags, bias);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -311,9 +305,8 @@ __global__ __launch_bounds__(256) void nk_mfma_t_kernel(const half_t* __restrict
                                                         const half_t* __restrict__ W,
                                                         half_t* __restrict__ C,
                                                         float* __restrict__ ws, int* counters, int M,
-                                                        int N, int K, int accumulate, int ur) {
+                                                        int N, int K, int flags, int ur, const void* bias) {
   // FULL: every wave range is complete (ur == 16 and K a multiple of 2048), no K masks needed.
-  accumulate &= 1;  // the flag word also carries the stagger mode of the interleaved kernels
   constexpr int RS = 1040;  // LDS bytes per staged row: 1 KB + 16 B
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int lane = threadIdx.x & 63;
@@ -389,14 +382,13 @@ __global__ __launch_bounds__(256) void nk_mfma_t_kernel(const half_t* __restrict
     if (mg < M) {
       if (gridDim.z == 1) {
         half_t* cp = C + (size_t)mg * N + n;
-        if (accumulate) sum += static_cast<float>(*cp);
-        *cp = static_cast<half_t>(sum);
+        *cp = finish_value(sum, cp, n, bias, flags);
       } else {
         store_partial(ws + ((size_t)blockIdx.z * M + mg) * N + n, sum, counters != nullptr);
       }
     }
   }
-  finish_splitk<16, ROWS * T>(ws, counters, C, M, N, m0, n0, accumulate);
+  finish_splitk<16, ROWS * T>(ws, counters, C, M, N, m0, n0, flags, bias);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -420,11 +412,10 @@ __global__ __launch_bounds__(64 * NW) void nk_mfma_r_kernel(const half_t* __rest
                                                         const half_t* __restrict__ W,
                                                         half_t* __restrict__ C,
                                                         float* __restrict__ ws, int* counters, int M,
-                                                        int N, int K, int flags) {
+                                                        int N, int K, int flags, const void* bias) {
   // AROWS: rows of A staged per step (8 covers M <= 8, 16 covers M <= 16).  BAND: bytes of K per
   // row and step (512 or 256).  FULL: K is a multiple of the band and the bands divide evenly
   // over the waves -- no masks needed.
-  const int accumulate = flags & 1;  // bit 1 of flags selects the start stagger
   constexpr int LPR = BAND / 16;       // lanes per row piece
   constexpr int RPI = 64 / LPR;        // rows per load instruction
   constexpr int WI = 16 * CB / RPI;    // load instructions per step for the weights (CB blocks of 16 rows)
@@ -526,14 +517,13 @@ __global__ __launch_bounds__(64 * NW) void nk_mfma_r_kernel(const half_t* __rest
     if (e / TN < AROWS && mg < M) {
       if (gridDim.z == 1) {
         half_t* cp = C + (size_t)mg * N + n;
-        if (accumulate) sum += static_cast<float>(*cp);
-        *cp = static_cast<half_t>(sum);
+        *cp = finish_value(sum, cp, n, bias, flags);
       } else {
         store_partial(ws + ((size_t)blockIdx.z * M + mg) * N + n, sum, counters != nullptr);
       }
     }
   }
-  finish_splitk<16, TN>(ws, counters, C, M, N, m0, n0, accumulate);
+  finish_splitk<16, TN>(ws, counters, C, M, N, m0, n0, flags, bias);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -543,7 +533,7 @@ __global__ __launch_bounds__(64 * NW) void nk_mfma_r_kernel(const half_t* __rest
   hipLaunchKernelGGL(KERNEL, dim3((p).grid_x, (p).grid_y, (p).grid_z), dim3((p).block), 0, s, \
                      static_cast<const half_t*>((a).A), static_cast<const half_t*>((a).W),    \
                      static_cast<half_t*>((a).C), (a).ws, (a).counters, (a).M, (a).N, (a).K,  \
-                     (a).accumulate)
+                     (a).accumulate, (a).bias)
 
 bool nk_dot2_supported(int mb, int rn, int u) {
   const bool mb_ok = mb == 1 || mb == 2 || mb == 4 || mb == 8;
@@ -701,7 +691,7 @@ static void nk_mfma_t_launch(const fg_plan_t& p, const GemmArgs& a, hipStream_t 
   hipLaunchKernelGGL((nk_mfma_t_kernel<ROWS, T, FULL, STREAM>),
                      dim3(p.grid_x, p.grid_y, p.grid_z), dim3(256), lds, s,
                      static_cast<const half_t*>(a.A), static_cast<const half_t*>(a.W),
-                     static_cast<half_t*>(a.C), a.ws, a.counters, a.M, a.N, a.K, a.accumulate, ur);
+                     static_cast<half_t*>(a.C), a.ws, a.counters, a.M, a.N, a.K, a.accumulate, ur, a.bias);
 }
 
 template <int ROWS, int T>

@@ -69,8 +69,10 @@ at::Tensor workspace(const at::Tensor& like, size_t bytes) {
 enum Protocol { kOverwrite = 0, kAccumulate = 1 };
 
 // C = A·W or C += A·W for fp16 tensors; `msg128` is the reference's exception text.
+// With `tail` set: C = act(A·W + bias) (bias may be undefined), always overwriting C.
 void gemm(const char* op, const at::Tensor& A, const at::Tensor& W, at::Tensor& C, int w_layout,
-          Protocol protocol, int bz, const char* msg128) {
+          Protocol protocol, int bz, const char* msg128, bool tail = false,
+          const at::Tensor& bias = at::Tensor(), int act = FG_ACT_NONE) {
   TORCH_CHECK(A.dim() == 2 && W.dim() == 2, op, ": A and B must be 2-D");
   const int64_t M = A.size(0), K = A.size(1);
   const int64_t N = w_layout == FG_W_KN ? W.size(1) : W.size(0);
@@ -96,10 +98,36 @@ void gemm(const char* op, const at::Tensor& A, const at::Tensor& W, at::Tensor& 
     ws = workspace(A, ws_bytes);
     ws_ptr = ws.data_ptr();
   }
-  const int st = fg_gemm_f16(A.data_ptr(), W.data_ptr(), C.data_ptr(), (int)M, (int)N, (int)K,
-                             w_layout, protocol == kAccumulate, bz, ws_ptr, ws_bytes,
-                             current_stream(A));
+  int st;
+  if (tail) {
+    const void* bias_ptr = nullptr;
+    if (bias.defined()) {
+      check_tensor(bias, "bias", at::kHalf, op);
+      TORCH_CHECK(bias.numel() == N && bias.device() == A.device(), op,
+                  ": bias must hold N = ", N, " elements on the device of A");
+      bias_ptr = bias.data_ptr();
+    }
+    st = fg_gemm_f16_bias_act(A.data_ptr(), W.data_ptr(), bias_ptr, act, C.data_ptr(), (int)M,
+                              (int)N, (int)K, w_layout, bz, nullptr, ws_ptr, ws_bytes,
+                              current_stream(A));
+  } else {
+    st = fg_gemm_f16(A.data_ptr(), W.data_ptr(), C.data_ptr(), (int)M, (int)N, (int)K, w_layout,
+                     protocol == kAccumulate, bz, ws_ptr, ws_bytes, current_stream(A));
+  }
   raise_status(st, op);
+}
+
+int act_id(const std::string& act, const char* op) {
+  if (act == "none") return FG_ACT_NONE;
+  if (act == "relu") return FG_ACT_RELU;
+  if (act == "gelu") return FG_ACT_GELU;
+  if (act == "gelu_tanh") return FG_ACT_GELU_TANH;
+  if (act == "silu") return FG_ACT_SILU;
+  throw std::invalid_argument(std::string(op) + ": act must be none, relu, gelu, gelu_tanh or silu");
+}
+
+at::Tensor optional_tensor(const py::object& o) {
+  return o.is_none() ? at::Tensor() : o.cast<at::Tensor>();
 }
 
 const char* kMsgKN = "K(input column) & N(output column) must be multiple of 128!";
@@ -376,6 +404,37 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         py::arg("scale") = py::none(), py::arg("scalar_scale") = 1.0, py::arg("zero_point") = 0.0,
         "res = (vec @ (mat_u4[N,K] - zero_point).T) * scalar_scale * scale[N]; mat is uint8 [N,K/2], "
         "even element in the low nibble (formula of hk/fastgemv.cuh:394-495)");
+  m.def(
+      "gemm_bias_act",
+      [](at::Tensor A, at::Tensor B, at::Tensor C, py::object bias, const std::string& act) {
+        gemm("gemm_bias_act", A, B, C, FG_W_KN, kOverwrite, 0, kMsgKN, true, optional_tensor(bias),
+             act_id(act, "gemm_bias_act"));
+      },
+      py::arg("A"), py::arg("B"), py::arg("C"), py::arg("bias") = py::none(),
+      py::arg("act") = "none",
+      "C = act(A @ B + bias), B[K,N]; bias fp16 [N] or None; act in none, relu, gelu, gelu_tanh, "
+      "silu (no counterpart in the reference: the tail of an FFN up-projection, fused)");
+  m.def(
+      "gemm_bias_act_bt",
+      [](at::Tensor A, at::Tensor B_t, at::Tensor C, py::object bias, const std::string& act) {
+        gemm("gemm_bias_act_bt", A, B_t, C, FG_W_NK, kOverwrite, 0, kMsgNK, true,
+             optional_tensor(bias), act_id(act, "gemm_bias_act_bt"));
+      },
+      py::arg("A"), py::arg("B_t"), py::arg("C"), py::arg("bias") = py::none(),
+      py::arg("act") = "none", "C = act(A @ B_t.T + bias), B_t[N,K]");
+  m.def(
+      "ffn_bt",
+      [](at::Tensor A, at::Tensor W1_t, py::object b1, at::Tensor W2_t, py::object b2, at::Tensor H,
+         at::Tensor C, const std::string& act) {
+        const int a = act_id(act, "ffn_bt");
+        gemm("ffn_bt (up)", A, W1_t, H, FG_W_NK, kOverwrite, 0, kMsgNK, true, optional_tensor(b1), a);
+        gemm("ffn_bt (down)", H, W2_t, C, FG_W_NK, kOverwrite, 0, kMsgNK, true, optional_tensor(b2),
+             FG_ACT_NONE);
+      },
+      py::arg("A"), py::arg("W1_t"), py::arg("b1"), py::arg("W2_t"), py::arg("b2"), py::arg("H"),
+      py::arg("C"), py::arg("act") = "gelu",
+      "feed-forward pair in two launches: H = act(A @ W1_t.T + b1), C = H @ W2_t.T + b2; "
+      "W1_t[N1,K], W2_t[N2,N1], H[M,N1] and C[M,N2] caller allocated");
   m.def("gemv_i8i8_i32", &gemv_i8i8_i32, py::arg("mat"), py::arg("xq"), py::arg("acc"),
         "acc_i32[M,N] = xq_i8[M,K] @ mat_i8[N,K].T, exact");
   m.def("dequant_i32_f16", &dequant_i32_f16, py::arg("acc"), py::arg("scale"), py::arg("x_scale"),

@@ -113,6 +113,28 @@ int fg_gemm_f16_planned(const void* A, const void* W, void* C, int M, int N, int
                         int w_layout, int accumulate, fg_plan_t* plan, void* ws,
                         size_t ws_bytes, void* stream);
 
+/*
+ * C = act(A·W + bias): the same kernels with the bias add and the activation applied in fp32 to
+ * the finished sum (after the split-K reduction when there is one), before the single rounding
+ * to fp16.  bias: fp16 [N], one value per output column, or NULL.  act: FG_ACT_*.  plan: NULL for
+ * the library's choice (then `splitk` is honoured as in fg_gemm_f16), or a caller-edited plan as
+ * in fg_gemm_f16_planned.  Always overwrites C.
+ *
+ * No counterpart in the reference, whose operators stop at the product: the up-projection of
+ * its DiT feed-forward pair (16 x 3072 x 12288, then 16 x 12288 x 3072) would be followed by a
+ * separate elementwise launch over C; here the up-projection writes act(A·W1 + b1) directly.
+ */
+enum {
+  FG_ACT_NONE = 0,
+  FG_ACT_RELU = 1,      /* max(x, 0)                                               */
+  FG_ACT_GELU = 2,      /* 0.5 x (1 + erf(x / sqrt 2))                             */
+  FG_ACT_GELU_TANH = 3, /* 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3)))         */
+  FG_ACT_SILU = 4       /* x / (1 + exp(-x))                                       */
+};
+int fg_gemm_f16_bias_act(const void* A, const void* W, const void* bias, int act, void* C, int M,
+                         int N, int K, int w_layout, int splitk, fg_plan_t* plan, void* ws,
+                         size_t ws_bytes, void* stream);
+
 /* The plan fg_gemm_f16 would use for this shape (splitk as above).  Host only. */
 int fg_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* out);
 

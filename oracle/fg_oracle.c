@@ -18,6 +18,8 @@
  *   fg_oracle_gemv_w8a16          hk/fastgemv.cuh:316-389: sum += x·(float(w) − zp); sum *= scale
  *   fg_oracle_gemv_w4a16          hk/fastgemv.cuh:394-495, nibble order hk/utility.cuh:13-36
  *   fg_oracle_gemv_i8i8_i32       none (integer stage added by this library); exact integer sum
+ *   fg_oracle_bias_act            none (bias + activation tail added by this library; the
+ *                                 reference's operators stop at the product): textbook formulas
  *
  * Pinning (tests/test_oracle.py): exact rational arithmetic on small cases, closed forms
  * (ones·ones = K from script/ncu-gemv-test.py:29-30, unit vectors, identity), the committed
@@ -262,6 +264,30 @@ void fg_oracle_dequant_i32_f16(const int32_t* acc, const uint16_t* scale, float 
       float s = x_scale;
       if (scale) s *= fg_oracle_h2f(scale[n]);
       Y[(size_t)m * N + n] = fg_oracle_f2h((float)acc[(size_t)m * N + n] * s);
+    }
+  }
+}
+
+/*
+ * Y[m,n] = fp16( act( C32[m,n] + bias[n] ) ), fp32 arithmetic with libm; act: 0 none, 1 relu,
+ * 2 gelu 0.5 x (1 + erf(x / sqrt 2)), 3 gelu-tanh 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3))),
+ * 4 silu x / (1 + exp(-x)).  bias: fp16 [N] or NULL.  Y32 (optional) receives the unrounded values.
+ */
+void fg_oracle_bias_act(const float* C32, const uint16_t* bias, int act, uint16_t* Y, float* Y32,
+                        int M, int N) {
+  for (int m = 0; m < M; ++m) {
+    for (int n = 0; n < N; ++n) {
+      float v = C32[(size_t)m * N + n];
+      if (bias) v += fg_oracle_h2f(bias[n]);
+      switch (act) {
+        case 1: v = v > 0.f ? v : 0.f; break;
+        case 2: v = 0.5f * v * (1.f + erff(v * 0.70710678118654752f)); break;
+        case 3: v = 0.5f * v * (1.f + tanhf(0.79788456080286536f * (v + 0.044715f * v * v * v))); break;
+        case 4: v = v / (1.f + expf(-v)); break;
+        default: break;
+      }
+      if (Y32) Y32[(size_t)m * N + n] = v;
+      Y[(size_t)m * N + n] = fg_oracle_f2h(v);
     }
   }
 }

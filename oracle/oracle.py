@@ -35,8 +35,7 @@ def build(force: bool = False) -> Path:
 def lib() -> ctypes.CDLL:
     global _lib
     if _lib is None:
-        if not _LIB_PATH.exists():
-            build()
+        build()  # compiles only when the library is missing or older than its source
         L = ctypes.CDLL(str(_LIB_PATH))
         vp, ci, cf = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
         L.fg_oracle_h2f.restype = ctypes.c_float
@@ -57,6 +56,8 @@ def lib() -> ctypes.CDLL:
         L.fg_oracle_gemv_i8i8_i32.argtypes = [vp, vp, vp, ci, ci, ci]
         L.fg_oracle_dequant_i32_f16.restype = None
         L.fg_oracle_dequant_i32_f16.argtypes = [vp, vp, cf, vp, ci, ci]
+        L.fg_oracle_bias_act.restype = None
+        L.fg_oracle_bias_act.argtypes = [vp, vp, ci, vp, vp, ci, ci]
         _lib = L
     return _lib
 
@@ -176,6 +177,26 @@ def dequant_i32_f16(acc, scale, x_scale: float):
     y = np.zeros((M, N), np.float16)
     lib().fg_oracle_dequant_i32_f16(_ptr(acc), _ptr(sc), float(x_scale), _ptr(y), M, N)
     return y
+
+
+ACTS = {"none": 0, "relu": 1, "gelu": 2, "gelu_tanh": 3, "silu": 4}
+
+
+def bias_act(raw32, bias=None, act="none"):
+    """fp16(act(raw32 + bias[n])) on unrounded fp32 sums [M,N]; returns (float16, float32)."""
+    raw = np.ascontiguousarray(raw32, dtype=np.float32)
+    M, N = raw.shape
+    b = None if bias is None else _f16(bias).reshape(N)
+    y = np.zeros((M, N), np.float16)
+    y32 = np.zeros((M, N), np.float32)
+    lib().fg_oracle_bias_act(_ptr(raw), _ptr(b), int(ACTS[act]), _ptr(y), _ptr(y32), M, N)
+    return y, y32
+
+
+def gemm_bias_act(A, W, w_layout: int, bias=None, act="none"):
+    """fp16(act(A·W + bias)): the fp32-accumulate product, then the tail in fp32."""
+    _, raw = gemm_f16(A, W, w_layout)
+    return bias_act(raw, bias, act)[0]
 
 
 # ------------------------------------------------------------------------------------------

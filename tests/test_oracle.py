@@ -315,3 +315,47 @@ def test_w4a16_against_float64_on_random_inputs():
     _, y32 = oracle.gemv_w4a16(Wq4, x, sc, 1.0, 7.5)
     want = (x.astype(np.float64) @ (_unpack_u4(Wq4) - 7.5).T) * sc.astype(np.float64)[None, :]
     assert np.abs(y32 - want).max() <= 2e-4 * np.abs(want).max()
+
+
+# ---------------------------------------------------------------------------------------
+# bias + activation tail: pinned by torch's float64 routines and by closed forms
+# ---------------------------------------------------------------------------------------
+@pytest.mark.parametrize("act", ["none", "relu", "gelu", "gelu_tanh", "silu"])
+def test_bias_act_matches_torch_float64(act):
+    import torch
+    rng = np.random.default_rng(11)
+    raw = (rng.standard_normal((5, 384)) * 3).astype(np.float32)
+    raw[0, :8] = [0.0, -0.0, 1.0, -1.0, 10.0, -10.0, 30.0, -30.0]
+    bias = (rng.standard_normal(384)).astype(np.float16)
+    x = torch.from_numpy(raw).double() + torch.from_numpy(bias).double()[None, :]
+    want = {"none": lambda t: t, "relu": torch.relu, "gelu": torch.nn.functional.gelu,
+            "gelu_tanh": lambda t: torch.nn.functional.gelu(t, approximate="tanh"),
+            "silu": torch.nn.functional.silu}[act](x).numpy()
+    y, y32 = oracle.bias_act(raw, bias, act)
+    assert np.abs(y32.astype(np.float64) - want).max() <= 2e-6 * max(1.0, np.abs(want).max())
+    # the fp16 result is the correctly rounded float64 value except where fp32 noise crosses a tie;
+    # in the far negative tail 1 + erf cancels in fp32, so tiny outputs are held to 1e-6 absolute
+    big = np.abs(want) > 1e-3
+    assert (y[big] == want.astype(np.float16)[big]).mean() > 0.995
+    assert np.abs(y.astype(np.float64) - want)[~big].max(initial=0.0) <= 1e-6 + 6e-8
+    assert (np.abs(y.astype(np.float64) - want) <= np.spacing(np.abs(want).astype(np.float16)) + 1e-6).all()
+
+
+def test_bias_act_closed_forms():
+    raw = np.array([[0.0, -5.0, 5.0, 1.0]], np.float32)
+    for act in ("relu", "gelu", "gelu_tanh", "silu"):
+        assert oracle.bias_act(raw, None, act)[1][0, 0] == 0.0
+    assert (oracle.bias_act(raw, None, "relu")[1] == [[0.0, 0.0, 5.0, 1.0]]).all()
+    # silu(1) = 1/(1+1/e), gelu(1) = Phi(1)
+    assert abs(oracle.bias_act(raw, None, "silu")[1][0, 3] - 0.7310585786300049) < 1e-6
+    assert abs(oracle.bias_act(raw, None, "gelu")[1][0, 3] - 0.8413447460685429) < 1e-6
+    # the bias is indexed by column, not by row
+    raw = np.zeros((3, 128), np.float32)
+    bias = np.arange(128).astype(np.float16)
+    assert (oracle.bias_act(raw, bias, "none")[0] == bias[None, :]).all()
+    # gemm_bias_act = product then tail
+    rng = np.random.default_rng(12)
+    A = rng.standard_normal((2, 128)).astype(np.float16)
+    W = (rng.standard_normal((128, 128)) * 0.1).astype(np.float16)
+    _, raw = oracle.gemm_f16(A, W, oracle.W_KN)
+    assert (oracle.gemm_bias_act(A, W, oracle.W_KN, bias, "relu") == oracle.bias_act(raw, bias, "relu")[0]).all()
