@@ -200,7 +200,11 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
         // (about 192 workgroups) shorten every wave's chain of dependent loads.  Measured (us,
         // 4 waves / 8 waves, M = 4): K=N=4096 12.3 / 11.2, K=4096 N=11008 20.1 / 18.1,
         // K=3072 N=12288 17.2 / 15.9, K=12288 N=3072 20.5 / 17.8, K=N=2048 12.3 / 8.8.
+        // Here the in-launch reduction also wins for 9..16 rows (M = 16: K=3072 N=12288 17.2 us
+        // against 17.9 with the second kernel, K=12288 N=3072 18.9 / 20.0, K=4096 N=11008 19.3 /
+        // 20.3); at 8192 x 8192 the second kernel stays 0.6 us ahead for them.
         p->waves = 8;
+        p->fused = 1;
         double best_dist = 1e30;
         for (int S = 1; S <= 16; S *= 2) {
           if (items / (p->waves * S) < 1) break;
