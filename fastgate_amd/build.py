@@ -3,6 +3,7 @@
   libfastgate.so   HIP kernels + C ABI (include/fastgate.h), hipcc --offload-arch=gfx950
   speedgate*.so    pybind11 / ATen host module that mirrors the reference's operator names
                    and forwards to libfastgate (plain C++, no device code)
+  fg_cbench        standalone C++ caller of the C ABI (csrc/fg_cbench.cpp): self-check + timing
 
 `python -m fastgate_amd.build` compiles everything; nothing is installed outside the tree.
 """
@@ -114,9 +115,22 @@ def build_ext(verbose: bool = True) -> Path:
     return out
 
 
+def build_cbench(verbose: bool = True) -> Path:
+    """Compile the standalone C++ caller of the C ABI (no torch, no Python)."""
+    t0 = time.time()
+    out = PKG / "fg_cbench"
+    _run([_hipcc(), "-O2", "-std=c++17", "-Wall", "-I", str(ROOT / "include"),
+          str(CSRC / "fg_cbench.cpp"), "-o", str(out), "-L", str(PKG), "-l:" + LIB_NAME,
+          "-Wl,-rpath,$ORIGIN"])
+    if verbose:
+        print("built %s in %.1fs" % (out, time.time() - t0), file=sys.stderr)
+    return out
+
+
 def build_all() -> None:
     build_lib()
     build_ext()
+    build_cbench()
 
 
 if __name__ == "__main__":
@@ -125,3 +139,5 @@ if __name__ == "__main__":
         build_lib()
     if "ext" in what or "all" in what:
         build_ext()
+    if "cbench" in what or "all" in what:
+        build_cbench()

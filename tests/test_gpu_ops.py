@@ -222,3 +222,28 @@ def test_operators_replay_correctly_from_a_hip_graph(device):
         torch.cuda.synchronize()
         for k in outs:
             assert torch.equal(outs[k], want[k]), (replay, k)
+
+
+@pytest.mark.parametrize("args", [
+    ["--m", "1", "--n", "4096", "--k", "4096", "--layout", "nk"],
+    ["--m", "8", "--n", "2048", "--k", "4480", "--layout", "kn"],
+    ["--m", "16", "--n", "1024", "--k", "8192", "--layout", "kn"],
+    ["--m", "16", "--n", "3072", "--k", "1152", "--layout", "nk"],
+    ["--m", "3", "--n", "1024", "--k", "2048", "--dtype", "i8"],
+    ["--m", "1", "--n", "1024", "--k", "2048", "--dtype", "i8"],
+    ["--m", "1", "--n", "1024", "--k", "4096", "--dtype", "i4"],
+    ["--m", "4", "--n", "1024", "--k", "1152", "--dtype", "i4"],
+], ids=lambda a: "-".join(x.lstrip("-") for x in a))
+def test_standalone_cpp_caller_of_the_c_abi(device, args):
+    """fg_cbench: hipMalloc + include/fastgate.h only (no torch in that process); it checks a closed
+    form on the device result and reports a timing."""
+    import json
+    import subprocess
+    from pathlib import Path
+
+    exe = Path(__file__).resolve().parent.parent / "fastgate_amd" / "fg_cbench"
+    assert exe.exists(), "fastgate_amd/fg_cbench is not built (python -m fastgate_amd.build)"
+    out = subprocess.run([str(exe), *args, "--iters", "20"], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, out.stdout + out.stderr
+    rec = json.loads(out.stdout.strip().splitlines()[-1])
+    assert rec["ok"] is True and rec["mismatches"] == 0 and rec["us_per_call"] > 0
