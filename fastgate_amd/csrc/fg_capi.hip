@@ -100,6 +100,7 @@ int finish_plan(int M, int N, int K, fg_plan_t* p) {
   if (p->splitk > 65535) return FG_ERR_INVALID_ARG;
   p->grid_x = N / p->tile_n;
   p->grid_y = ceil_div(M, p->m_block);
+  if (p->grid_y > 65535) return FG_ERR_INVALID_ARG;  // HIP's limit on grid.y
   p->grid_z = p->splitk;
   p->block = 64 * p->waves;
   if (p->splitk > 1) {

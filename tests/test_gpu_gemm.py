@@ -262,3 +262,17 @@ def test_error_codes_on_device(device):
     assert L.fg_gemm_f16(None, ptr(W), ptr(C), 8, 256, 256, NK, 0, 0, None, 0, stream_ptr()) == capi.FG_ERR_INVALID_ARG
     assert L.fg_gemm_f16(ptr(A), ptr(W), ptr(C), 8, 256, 256, NK, 0, 4, None, 0, stream_ptr()) == capi.FG_ERR_WORKSPACE
     assert L.fg_gemm_f16(ptr(A), ptr(W), ptr(C), 8, 256, 256, 7, 0, 0, None, 0, stream_ptr()) == capi.FG_ERR_INVALID_ARG
+
+
+@pytest.mark.parametrize("layout", [KN, NK])
+def test_split_deeper_than_k_has_idle_workgroups_that_contribute_zero(device, layout):
+    # K = 128 is a single K unit of every kernel: with S = 16 most workgroups own no part of K and
+    # must still publish an all-zero partial and arrive at the counter
+    for M in (1, 4, 8, 16):
+        A, W = _case(M, 256, 128, layout, 600 + M)
+        ref, _ = oracle.gemm_f16(A.numpy(), W.numpy(), layout)
+        got, p = _run(A, W, layout, device, splitk=16)
+        assert p.splitk == 16 or p.kernel == capi.FG_KERNEL_NK_MFMA_T
+        assert_close_f16(got, ref, "S=16 on K=128, M=%d" % M)
+        got, _ = _run(A, W, layout, device, splitk=3)
+        assert_close_f16(got, ref, "S=3 on K=128, M=%d" % M)

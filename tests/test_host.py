@@ -258,3 +258,10 @@ def test_eed_backend_reexports_every_operator(sg):
     assert backend.edgemm_m8n64k128x8_bt_tuning is sg.gemm_m8n64k128x8_bt_exp
     with pytest.raises(ImportError):
         from eed.backend import hgemm_warp2  # noqa: F401  (no surviving definition in the reference)
+
+
+def test_row_count_beyond_the_grid_limit_is_rejected():
+    import ctypes
+    p = capi.Plan()
+    assert capi.lib().fg_plan(16 * 65535 + 1, 128, 128, capi.FG_W_NK, 0, ctypes.byref(p)) == capi.FG_ERR_INVALID_ARG
+    assert capi.lib().fg_plan(16 * 65535, 128, 128, capi.FG_W_NK, 0, ctypes.byref(p)) == capi.FG_OK
