@@ -207,6 +207,7 @@ void gemv_f16(const char* op, const at::Tensor& mat, const at::Tensor& vec, at::
   TORCH_CHECK(vec.numel() > 0 && vec.numel() % K == 0, op, ": vec must hold a multiple of K = ", K,
               " elements (got ", vec.numel(), ")");
   const int64_t M = vec.numel() / K;
+  TORCH_CHECK(M <= INT32_MAX && N <= INT32_MAX && K <= INT32_MAX, op, ": size overflow");
   TORCH_CHECK(M == 1 || (vec.dim() == 2 && vec.size(1) == K), op, ": batched vec must be [M,K]");
   TORCH_CHECK(res.numel() == M * N, op, ": res must hold M*N = ", M * N, " elements (got ",
               res.numel(), ")");
@@ -249,6 +250,7 @@ void fastgemv_int8(at::Tensor mat, at::Tensor vec, at::Tensor res, c10::optional
   TORCH_CHECK(vec.numel() > 0 && vec.numel() % K == 0, op, ": vec must hold a multiple of K = ", K,
               " elements");
   const int64_t M = vec.numel() / K;
+  TORCH_CHECK(M <= INT32_MAX && N <= INT32_MAX && K <= INT32_MAX, op, ": size overflow");
   TORCH_CHECK(M <= 8, op, ": at most 8 activation rows");
   TORCH_CHECK(res.numel() == M * N, op, ": res must hold M*N = ", M * N, " elements");
   const void* sp = nullptr;
@@ -282,6 +284,7 @@ void fastgemv_int4(at::Tensor mat, at::Tensor vec, at::Tensor res, c10::optional
   TORCH_CHECK(vec.numel() > 0 && vec.numel() % K == 0, op, ": vec must hold a multiple of K = ", K,
               " elements");
   const int64_t M = vec.numel() / K;
+  TORCH_CHECK(M <= INT32_MAX && N <= INT32_MAX && K <= INT32_MAX, op, ": size overflow");
   TORCH_CHECK(M <= 4, op, ": at most 4 activation rows");
   TORCH_CHECK(res.numel() == M * N, op, ": res must hold M*N = ", M * N, " elements");
   const void* sp = nullptr;
