@@ -247,3 +247,27 @@ def test_standalone_cpp_caller_of_the_c_abi(device, args):
     assert out.returncode == 0, out.stdout + out.stderr
     rec = json.loads(out.stdout.strip().splitlines()[-1])
     assert rec["ok"] is True and rec["mismatches"] == 0 and rec["us_per_call"] > 0
+
+
+def test_two_streams_with_split_k_calls_in_flight_do_not_interfere(device, sg):
+    # the binding keeps one split-K workspace per (device, stream): calls that overlap in time on
+    # different streams must each complete their own tiles
+    g = gen(77)
+    K, N = 4096, 1024                        # [K,N] at this size always splits K
+    assert sg.plan(8, N, K, sg.W_KN)["splitk"] > 1
+    W = [normal((K, N), g, 0.03).to(device) for _ in range(2)]
+    A = [normal((8, K), g).to(device) for _ in range(2)]
+    ref = [oracle.gemm_f16(A[i].cpu().numpy(), W[i].cpu().numpy(), oracle.W_KN)[0] for i in range(2)]
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    outs = [[torch.full((8, N), float("nan"), dtype=torch.half, device=device) for _ in range(30)] for _ in range(2)]
+    torch.cuda.synchronize()
+    for it in range(30):
+        for i in range(2):
+            with torch.cuda.stream(streams[i]):
+                sg.edgemm_m8n128k64x4(A[i], W[i], outs[i][it])
+    torch.cuda.synchronize()
+    for i in range(2):
+        first = outs[i][0].cpu().numpy()
+        assert_close_f16(first, ref[i], "stream %d" % i)
+        for it in range(1, 30):
+            assert (outs[i][it].cpu().numpy().view(np.uint16) == first.view(np.uint16)).all(), (i, it)
