@@ -68,6 +68,7 @@ class Plan(ctypes.Structure):
         ("unroll", ctypes.c_int),
         ("stream_w", ctypes.c_int),
         ("stagger", ctypes.c_int),
+        ("band", ctypes.c_int),
         ("grid_x", ctypes.c_int),
         ("grid_y", ctypes.c_int),
         ("grid_z", ctypes.c_int),

@@ -55,7 +55,8 @@ int validate_shape(int M, int N, int K, int w_layout) {
 // Fills grid/block/workspace from the tile fields; rejects tiles that were not built.
 int finish_plan(int M, int N, int K, fg_plan_t* p) {
   const int max_waves =
-      ((p->kernel == FG_KERNEL_NK_MFMA_R && p->unroll == 1) || p->kernel == FG_KERNEL_KN_MFMA ||
+      ((p->kernel == FG_KERNEL_NK_MFMA_R && (p->band ? p->band : 256 * p->unroll) <= 256) ||
+       p->kernel == FG_KERNEL_KN_MFMA ||
        (p->kernel == FG_KERNEL_KN_DOT2 && p->m_block <= 2))
           ? 8
           : 4;
@@ -76,7 +77,12 @@ int finish_plan(int M, int N, int K, fg_plan_t* p) {
     case FG_KERNEL_NK_MFMA_R:
       if (p->tile_n != 32) p->tile_n = 16;
       p->m_block = 16;
-      if (p->unroll != 1 && p->unroll != 2) return FG_ERR_UNSUPPORTED;
+      if (p->band == 0) {
+        if (p->unroll != 1 && p->unroll != 2) return FG_ERR_UNSUPPORTED;
+        p->band = 256 * p->unroll;
+      }
+      if (p->band != 128 && p->band != 256 && p->band != 512) return FG_ERR_UNSUPPORTED;
+      p->unroll = p->band == 512 ? 2 : 1;
       break;
     case FG_KERNEL_NK_MFMA_T:
       if (!nk_mfma_t_supported(p->unroll, p->tile_n)) return FG_ERR_UNSUPPORTED;
@@ -126,6 +132,7 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
   int items = 1;
   bool row_tiles = false;   // the 16-column row-load kernel picks its own split
   bool wide_tiles = false;  // ... in its 32-column form
+  int wide_band_waves = 0, wide_band_split = 0;  // ... on 128-byte bands: waves and split are fixed
   if (w_layout == FG_W_NK) {
     // Measured on MI355X at K = N = 8192 (us per call): M=1 dot2 tile 4: 21.6-22.4; M=4 dot2
     // 24.3 / mfma4 22.3; M=8 dot2 27.8 / mfma4 25.6 / row-load 23.3; M=16 mfma4 36 / direct
@@ -173,6 +180,33 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
       }
       items = ceil_div(K, 128 * p->unroll);
       row_tiles = true;
+      // 32-column tiles on 128-byte bands: two column blocks share the staged activations and a
+      // band carries half the activation bytes, so the L2 traffic for A is a quarter of the
+      // 16-column / 256-byte form -- but the grid is only N/32 workgroups, so it has to land on
+      // (nearly) whole CUs: 192..256 workgroups of 8 waves, or 512 of 4.  Measured (us, this form
+      // / the rule above): K = N = 8192 M=16 22.8 / 24.7, M=8 22.9 / 23.3; K = N = 6144 M=16
+      // 16.6 / 18.9, M=4 14.3 / 15.7; K=2048 N=8192 M=16 7.9 / 9.0; K=4096 N=16384 M=16 22.4 / 24.3;
+      // K=12288 N=3072 with two-way split-K M=16 18.2 / 19.4 (M <= 8: 16.3 / 16.1, so not there).
+      // 384 workgroups (N = 12288) leave half the CUs with one: 46+ us against 45 at K = 12288.
+      const int t32 = N / 32;
+      int s32 = 0;
+      if (N % 32 == 0) {
+        if (t32 >= 192) s32 = 1;
+        else if (2 * t32 >= 192 && K >= 8192 && M >= 9) s32 = 2;
+      }
+      if (s32 && M <= 16 && !wide_tiles && (splitk == 0 || (splitk == 1 && s32 == 1))) {
+        const int wgs = t32 * s32;
+        const bool one_round = wgs <= kCUs && 4 * wgs >= 3 * kCUs;
+        const bool two_rounds = wgs == 2 * kCUs && M >= 5;
+        if ((one_round && (M >= 4 || t32 < kCUs)) || two_rounds) {
+          p->tile_n = 32;
+          p->unroll = 1;
+          p->band = 128;
+          wide_tiles = true;
+          wide_band_waves = one_round ? 8 : 4;
+          wide_band_split = s32;
+        }
+      }
     }
   } else {
     if (M <= 2 && (size_t)N * K < ((size_t)1 << 28)) {
@@ -189,6 +223,10 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
   }
   {
     p->waves = (row_tiles && !wide_tiles && p->unroll == 1 && items >= 16) ? 8 : pick_waves(items);
+    if (wide_band_waves) {
+      p->waves = wide_band_waves;
+      while (p->waves > 1 && p->waves > K / 64) p->waves >>= 1;  // one 128-byte band per wave at least
+    }
     const int tiles = (N / p->tile_n) * ceil_div(M, p->m_block);
     if (splitk > 0) {
       p->splitk = splitk;
@@ -228,6 +266,9 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
         }
       }
       p->splitk = best;
+    } else if (wide_band_split) {
+      p->splitk = wide_band_split;
+      p->fused = 1;
     } else if (row_tiles) {
       // 192 tiles still run best unsplit (K=12288 N=3072 M=8: 16.0 us against 17.4 with S = 4);
       // 128 tiles or fewer want two workgroups per CU once K is long (N=2048: K=8192 M=16

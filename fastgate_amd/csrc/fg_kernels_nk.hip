@@ -414,7 +414,7 @@ __global__ __launch_bounds__(64 * NW) void nk_mfma_r_kernel(const half_t* __rest
                                                         float* __restrict__ ws, int* counters, int M,
                                                         int N, int K, int flags, const void* bias) {
   // AROWS: rows of A staged per step (8 covers M <= 8, 16 covers M <= 16).  BAND: bytes of K per
-  // row and step (512 or 256).  FULL: K is a multiple of the band and the bands divide evenly
+  // row and step (512, 256 or 128).  FULL: K is a multiple of the band and the bands divide evenly
   // over the waves -- no masks needed.
   constexpr int LPR = BAND / 16;       // lanes per row piece
   constexpr int RPI = 64 / LPR;        // rows per load instruction
@@ -732,7 +732,7 @@ static void nk_mfma_r_go(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
   const int slots = p.waves * p.grid_z;
   const int bk = BAND / 2;
   const bool full = a.K % bk == 0 && (a.K / bk) % slots == 0;
-  if constexpr (BAND == 256) {
+  if constexpr (BAND <= 256) {
     if (p.waves == 8) {
       if (full) FG_LAUNCH((nk_mfma_r_kernel<AROWS, BAND, true, 8, CB>), p, a, s);
       else FG_LAUNCH((nk_mfma_r_kernel<AROWS, BAND, false, 8, CB>), p, a, s);
@@ -746,23 +746,30 @@ static void nk_mfma_r_go(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
 template <int CB>
 static bool nk_mfma_r_cb(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
   const bool half_m = a.M <= 8;  // one block row whose A strip needs only 8 rows
-  if (p.unroll == 2) {
-    if (half_m) nk_mfma_r_go<8, 512, CB>(p, a, s);
-    else nk_mfma_r_go<16, 512, CB>(p, a, s);
-  } else if (p.unroll == 1) {
-    if (half_m) nk_mfma_r_go<8, 256, CB>(p, a, s);
-    else nk_mfma_r_go<16, 256, CB>(p, a, s);
-  } else {
-    return false;
+  switch (p.band) {
+    case 128:
+      if (half_m) nk_mfma_r_go<8, 128, CB>(p, a, s);
+      else nk_mfma_r_go<16, 128, CB>(p, a, s);
+      return true;
+    case 256:
+      if (half_m) nk_mfma_r_go<8, 256, CB>(p, a, s);
+      else nk_mfma_r_go<16, 256, CB>(p, a, s);
+      return true;
+    case 512:
+      if (half_m) nk_mfma_r_go<8, 512, CB>(p, a, s);
+      else nk_mfma_r_go<16, 512, CB>(p, a, s);
+      return true;
+    default:
+      return false;
   }
-  return true;
 }
 
-// unroll = 2: 512-byte bands (two rows per load instruction); unroll = 1: 256-byte bands.
-// tile_n = 16 or 32 (two 16-column blocks sharing the staged activations).
+// band = bytes of K per row and step: 512 (two rows per load instruction, four waves at most),
+// 256 or 128 (four or eight rows per instruction, up to eight waves).  tile_n = 16 or 32 (two
+// 16-column blocks sharing the staged activations).
 bool launch_nk_mfma_r(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
   if (p.m_block != 16) return false;
-  if (p.waves > 4 && !(p.waves == 8 && p.unroll == 1)) return false;
+  if (p.waves > 4 && !(p.waves == 8 && p.band <= 256)) return false;
   if (p.tile_n == 16) return nk_mfma_r_cb<1>(p, a, s);
   if (p.tile_n == 32) return nk_mfma_r_cb<2>(p, a, s);
   return false;

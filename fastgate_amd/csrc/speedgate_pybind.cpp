@@ -363,6 +363,7 @@ py::dict plan(int M, int N, int K, int w_layout, int splitk) {
   d["unroll"] = p.unroll;
   d["stream_w"] = p.stream_w;
   d["stagger"] = p.stagger;
+  d["band"] = p.band;
   d["grid"] = py::make_tuple(p.grid_x, p.grid_y, p.grid_z);
   d["block"] = p.block;
   d["workspace_bytes"] = p.workspace_bytes;

@@ -80,6 +80,9 @@ typedef struct fg_plan_t {
   int stagger;  /* K-interleaved [N,K] kernels start each workgroup at its own K step:
                    0 = (workgroup id / 8) % steps, spread within every XCD (default);
                    1 = workgroup id % steps, one K band per XCD (only with 8 steps)  */
+  int band;     /* FG_KERNEL_NK_MFMA_R only: bytes of K per weight row and step, 128, 256 or
+                   512 (0 = 256 * unroll); a narrower band halves the activation bytes a
+                   32-column tile re-reads, a wider one halves the load instructions   */
   int grid_x, grid_y, grid_z, block; /* filled by fg_plan / fg_gemm_f16_planned       */
   size_t workspace_bytes;            /* 0 when splitk == 1                            */
 } fg_plan_t;

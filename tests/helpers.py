@@ -80,8 +80,9 @@ def capi_gemm(A, W, C, w_layout, accumulate=False, splitk=0, plan=None):
     return p
 
 
-def make_plan(kernel, tile_n=0, m_block=0, waves=4, unroll=1, splitk=1, stream_w=1, fused=1, stagger=0):
+def make_plan(kernel, tile_n=0, m_block=0, waves=4, unroll=1, splitk=1, stream_w=1, fused=1, stagger=0, band=0):
     p = capi.Plan()
     p.kernel, p.tile_n, p.m_block, p.waves = kernel, tile_n, m_block, waves
     p.unroll, p.splitk, p.stream_w, p.fused, p.stagger = unroll, splitk, stream_w, fused, stagger
+    p.band = band
     return p

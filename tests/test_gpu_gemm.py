@@ -98,12 +98,16 @@ def test_transposing_mfma_kernel(device, rows, tiles):
     assert (got == ref).all()
 
 
-@pytest.mark.parametrize("unroll", [1, 2])
+@pytest.mark.parametrize("unroll", [1, 2, 128])
 @pytest.mark.parametrize("waves", [1, 2, 4, 8])
 @pytest.mark.parametrize("splitk,fused", [(1, 0), (2, 0), (3, 1)])
 def test_row_load_mfma_kernel(device, waves, splitk, fused, unroll):
+    # unroll 1 / 2: 256- / 512-byte bands through the `unroll` field; 128: the `band` field
+    band = 0
+    if unroll == 128:
+        unroll, band = 1, 128
     if waves == 8 and unroll != 1:
-        pytest.skip("8-wave workgroups exist for 256-byte bands only")
+        pytest.skip("8-wave workgroups exist for 128- and 256-byte bands only")
     # K = 128 (half a band), 384 (one and a half), 2048 (8 bands: the unmasked path when they divide
     # evenly over waves x splits), 4480 (ragged); M <= 8 uses the 8-row A strip, M = 19 two block rows
     N = 384
@@ -114,9 +118,10 @@ def test_row_load_mfma_kernel(device, waves, splitk, fused, unroll):
             C0 = normal((M, N), gen(71), 2.0)
             refa, _ = oracle.gemm_f16(A.numpy(), W.numpy(), NK, C=C0.numpy(), accumulate=True)
             tile = 32 if (M + K // 128) % 2 else 16
-            kw = dict(kernel=capi.FG_KERNEL_NK_MFMA_R, tile_n=tile, waves=waves, splitk=splitk, fused=fused, unroll=unroll)
+            kw = dict(kernel=capi.FG_KERNEL_NK_MFMA_R, tile_n=tile, waves=waves, splitk=splitk, fused=fused, unroll=unroll, band=band)
             got, p = _run(A, W, NK, device, plan=make_plan(**kw))
             assert p.tile_n == tile and p.grid_x == N // tile and p.block == 64 * waves
+            assert p.band == (band or 256 * unroll)
             assert_close_f16(got, ref, "mfma_r M=%d K=%d" % (M, K))
             got, _ = _run(A, W, NK, device, accumulate=True, C0=C0, plan=make_plan(**kw))
             assert_close_f16(got, refa, "mfma_r accumulate M=%d K=%d" % (M, K))
@@ -127,7 +132,7 @@ def test_row_load_mfma_kernel(device, waves, splitk, fused, unroll):
         W = torch.randint(-3, 4, (N, 768), generator=g).half()
         ref, _ = oracle.gemm_f16(A.numpy(), W.numpy(), NK)
         for tile in (16, 32):
-            got, _ = _run(A, W, NK, device, plan=make_plan(kernel=capi.FG_KERNEL_NK_MFMA_R, tile_n=tile, waves=waves, splitk=splitk, fused=fused, unroll=unroll))
+            got, _ = _run(A, W, NK, device, plan=make_plan(kernel=capi.FG_KERNEL_NK_MFMA_R, tile_n=tile, waves=waves, splitk=splitk, fused=fused, unroll=unroll, band=band))
             assert (got == ref).all()
 
 
