@@ -50,11 +50,11 @@ def _traffic(fetch_kib: float, write_kib: float) -> int:
 
 
 TRAFFIC_BYTES = {
-    "nk_dot2_M1": _traffic(65621.2, 64.0),
-    "nk_mfma_r_M8": _traffic(66077.0, 128.0),
-    "nk_mfma_r_M16": _traffic(66596.5, 256.0),
-    "kn_dot2_M1": _traffic(65699.1, 154.0),     # 128 KiB of the written bytes are split-K partials
-    "kn_mfma_M8": _traffic(66597.5, 1152.0),    # 1 MiB of split-K partials
+    "nk_dot2_M1": _traffic(65637.6, 64.0),
+    "nk_mfma_r_M8": _traffic(66091.5, 128.0),
+    "nk_mfma_r_M16": _traffic(66604.5, 256.0),
+    "kn_dot2_M1": _traffic(65729.1, 154.0),     # 128 KiB of the written bytes are split-K partials
+    "kn_mfma_M8": _traffic(66621.3, 1152.0),    # 1 MiB of split-K partials
 }
 
 
