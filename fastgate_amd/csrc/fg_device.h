@@ -184,6 +184,33 @@ __device__ __forceinline__ bool splitk_last_arriver(int* counter, int S) {
   return s_last != 0;
 }
 
+// Σ_z part[z][off..off+3] in ascending z.  The loads of a batch are all issued before the first
+// add: one memory round trip per batch instead of one per partial (a plain `for z` loop compiles
+// to load, wait, add).  Slots past S re-read the last partial and contribute +0, which leaves
+// every sum unchanged (a sum that started from +0 is never -0).
+template <int BATCH>
+__device__ __forceinline__ float4_t sum_partials_batched(const float* part, int S, size_t MN,
+                                                         size_t off) {
+  float4_t sum = {0.f, 0.f, 0.f, 0.f};
+  for (int z0 = 0; z0 < S; z0 += BATCH) {
+    float4_t v[BATCH];
+#pragma unroll
+    for (int u = 0; u < BATCH; ++u) {
+      const int z = z0 + u < S ? z0 + u : S - 1;
+      v[u] = load_partial4(part, (size_t)z * MN + off);
+    }
+#pragma unroll
+    for (int u = 0; u < BATCH; ++u) {
+      const float4_t zero = {0.f, 0.f, 0.f, 0.f};
+      sum += z0 + u < S ? v[u] : zero;
+    }
+  }
+  return sum;
+}
+__device__ __forceinline__ float4_t sum_partials(const float* part, int S, size_t MN, size_t off) {
+  return S <= 4 ? sum_partials_batched<4>(part, S, MN, off) : sum_partials_batched<8>(part, S, MN, off);
+}
+
 // C[m0..m0+mcnt)[n0..n0+ncnt) = fp16( Σ_z part[z] (+ C) ); ncnt and n0 are multiples of 4.
 __device__ __forceinline__ void splitk_reduce_tile(const float* part, half_t* C, int S, int M, int N,
                                                    int m0, int mcnt, int n0, int ncnt,
@@ -195,8 +222,8 @@ __device__ __forceinline__ void splitk_reduce_tile(const float* part, half_t* C,
     const int m = m0 + e / nq, n = n0 + (e % nq) * 4;
     if (m >= M) continue;
     const size_t off = (size_t)m * N + n;
-    float4_t sum = {0.f, 0.f, 0.f, 0.f};
-    for (int z = 0; z < S; ++z) sum += load_partial4(part, (size_t)z * MN + off);
+    const float4_t sum0 = sum_partials(part, S, MN, off);
+    float4_t sum = sum0;
     half4v* c = reinterpret_cast<half4v*>(C + off);
     if (flags & kFlagAccumulate) {
       const half4v old = *c;

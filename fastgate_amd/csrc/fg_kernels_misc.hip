@@ -13,8 +13,22 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
                                                             const void* bias) {
   const size_t i = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
   if (i >= MN) return;
-  float4_t sum = *reinterpret_cast<const float4_t*>(ws + i);
-  for (int s = 1; s < S; ++s) sum += *reinterpret_cast<const float4_t*>(ws + (size_t)s * MN + i);
+  // batches of four loads in flight before the first add (a plain loop compiles to load, wait,
+  // add); slots past S re-read the last partial and contribute +0
+  float4_t sum = {0.f, 0.f, 0.f, 0.f};
+  for (int s0 = 0; s0 < S; s0 += 4) {
+    float4_t v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int z = s0 + u < S ? s0 + u : S - 1;
+      v[u] = *reinterpret_cast<const float4_t*>(ws + (size_t)z * MN + i);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const float4_t zero = {0.f, 0.f, 0.f, 0.f};
+      sum += s0 + u < S ? v[u] : zero;
+    }
+  }
   typedef half_t half4_t __attribute__((ext_vector_type(4)));
   half4_t* c = reinterpret_cast<half4_t*>(C + i);
   if (flags & kFlagAccumulate) {
