@@ -218,7 +218,11 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
       p->m_block = 16;
     }
     p->tile_n = 128;
-    p->unroll = (p->kernel == FG_KERNEL_KN_DOT2 && K >= 2048) ? 2 : 1;
+    // one 32-row unit in flight per wave and step: with the split-K tail no longer waiting on
+    // each partial in turn, deeper splits of shorter steps win (v_dot2, M = 1, two units / one:
+    // K = N = 4096 10.5 / 9.7 us, K=3072 N=12288 16.7 / 15.5, K=4096 N=11008 18.5 / 17.3)
+    p->unroll = 1;
+    p->fused = M <= 16;  // 26.5 / 25.8 us at K = N = 8192, M = 16 (second kernel / in-launch)
     items = ceil_div(K / 32, p->unroll);
   }
   {
@@ -254,10 +258,13 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
           }
         }
       } else if ((size_t)N * K >= ((size_t)1 << 18)) {  // 1024 x 1024: 7.7 us with S = 8 against 9.0 without
+        // up to four rows the partials are small enough for two workgroups per CU to pay
+        // (K = N = 8192, S = 8 / S = 4: M=1 24.4 / 25.3 us, M=4 25.0 / 25.4, M=8 25.7 / 25.2)
+        const int target = (M <= 4 && tiles <= 64 && (size_t)N * K <= ((size_t)1 << 26)) ? 2 * kCUs : kCUs;
         double best_ratio = 1e30;
         for (int S = 1; S <= 16; S *= 2) {
           if (items / (p->waves * S) < 1) break;
-          const double r = (double)tiles * S / kCUs;
+          const double r = (double)tiles * S / target;
           const double ratio = r > 1.0 ? r : 1.0 / (r * r);  // idle CUs cost more than a deeper split
           if (ratio < best_ratio - 1e-9) {
             best_ratio = ratio;
@@ -266,6 +273,18 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
         }
       }
       p->splitk = best;
+      // the v_dot2 kernel wants eight waves on every CU: K=4096 N=16384, M = 1, S = 2:
+      // 26.9 us with four waves a workgroup, 24.3 with eight
+      if (p->kernel == FG_KERNEL_KN_DOT2 && p->waves == 4 && tiles * best < 2 * kCUs &&
+          items / (8 * best) >= 2) {
+        p->waves = 8;
+      }
+      // 9..16 rows at 8192 x 8192: 26.0 us with eight waves against 26.5 with four (at 16384 x 16384
+      // four stay ahead, 82.3 against 89)
+      if (p->kernel == FG_KERNEL_KN_MFMA && M > 8 && p->waves == 4 &&
+          (size_t)N * K <= ((size_t)1 << 26) && items / (8 * best) >= 2) {
+        p->waves = 8;
+      }
     } else if (wide_band_split) {
       p->splitk = wide_band_split;
       p->fused = 1;
