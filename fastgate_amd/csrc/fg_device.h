@@ -207,11 +207,18 @@ __device__ __forceinline__ float4_t sum_partials_batched(const float* part, int 
   }
   return sum;
 }
+// DEEP: splits beyond four are common for the caller ([K,N] kernels), worth eight loads in flight
+// and the registers they take.
+template <bool DEEP>
 __device__ __forceinline__ float4_t sum_partials(const float* part, int S, size_t MN, size_t off) {
-  return S <= 4 ? sum_partials_batched<4>(part, S, MN, off) : sum_partials_batched<8>(part, S, MN, off);
+  if constexpr (DEEP) {
+    if (S > 4) return sum_partials_batched<8>(part, S, MN, off);
+  }
+  return sum_partials_batched<4>(part, S, MN, off);
 }
 
 // C[m0..m0+mcnt)[n0..n0+ncnt) = fp16( Σ_z part[z] (+ C) ); ncnt and n0 are multiples of 4.
+template <bool DEEP>
 __device__ __forceinline__ void splitk_reduce_tile(const float* part, half_t* C, int S, int M, int N,
                                                    int m0, int mcnt, int n0, int ncnt,
                                                    int flags, const void* bias) {
@@ -222,7 +229,7 @@ __device__ __forceinline__ void splitk_reduce_tile(const float* part, half_t* C,
     const int m = m0 + e / nq, n = n0 + (e % nq) * 4;
     if (m >= M) continue;
     const size_t off = (size_t)m * N + n;
-    const float4_t sum0 = sum_partials(part, S, MN, off);
+    const float4_t sum0 = sum_partials<DEEP>(part, S, MN, off);
     float4_t sum = sum0;
     half4v* c = reinterpret_cast<half4v*>(C + off);
     if (flags & kFlagAccumulate) {
@@ -240,12 +247,12 @@ __device__ __forceinline__ void splitk_reduce_tile(const float* part, half_t* C,
 // Shared tail of every GEMM kernel: the workgroup has stored its fp32 partial of the tile
 // (m0.., n0..) when gridDim.z > 1; with counters it also completes the split-K sum in place,
 // without counters a second kernel does.
-template <int MROWS, int NCOLS>
+template <int MROWS, int NCOLS, bool DEEP = false>
 __device__ __forceinline__ void finish_splitk(float* ws, int* counters, half_t* C, int M, int N,
                                               int m0, int n0, int flags, const void* bias) {
   if (gridDim.z > 1 && counters != nullptr) {
     if (splitk_last_arriver(counters + blockIdx.y * gridDim.x + blockIdx.x, gridDim.z))
-      splitk_reduce_tile(ws, C, gridDim.z, M, N, m0, MROWS, n0, NCOLS, flags, bias);
+      splitk_reduce_tile<DEEP>(ws, C, gridDim.z, M, N, m0, MROWS, n0, NCOLS, flags, bias);
   }
 }
 

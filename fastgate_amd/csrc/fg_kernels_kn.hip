@@ -120,7 +120,7 @@ __global__ __launch_bounds__(64 * NW) void kn_mfma_kernel(const half_t* __restri
       }
     }
   }
-  finish_splitk<16, 128>(ws, counters, C, M, N, m0, n0, flags, bias);
+  finish_splitk<16, 128, true>(ws, counters, C, M, N, m0, n0, flags, bias);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -200,7 +200,7 @@ __global__ __launch_bounds__(64 * NW) void kn_dot2_kernel(const half_t* __restri
       }
     }
   }
-  finish_splitk<MB, 128>(ws, counters, C, M, N, m0, n0, flags, bias);
+  finish_splitk<MB, 128, true>(ws, counters, C, M, N, m0, n0, flags, bias);
 }
 
 // ---------------------------------------------------------------------------------------
