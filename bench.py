@@ -53,8 +53,11 @@ TRAFFIC_BYTES = {
     "nk_dot2_M1": _traffic(65637.6, 64.0),
     "nk_mfma_r_M8": _traffic(66091.5, 128.0),
     "nk_mfma_r_M16": _traffic(66604.5, 256.0),
-    "kn_dot2_M1": _traffic(65729.1, 154.0),     # 128 KiB of the written bytes are split-K partials
-    "kn_mfma_M8": _traffic(66621.3, 1152.0),    # 1 MiB of split-K partials
+    # [K,N]: split-K partials are written through and read back inside the launch; WRITE_SIZE counts
+    # the write-through stores twice (M=1: 8 x 16 KiB of partials, M=8: 4 x 256 KiB, M=16: 4 x 512 KiB)
+    "kn_dot2_M1": _traffic(65788.6, 290.0),
+    "kn_mfma_M8": _traffic(66635.0, 2186.0),
+    "kn_mfma_M16": _traffic(67650.0, 4362.0),
 }
 
 
