@@ -475,28 +475,39 @@ __global__ __launch_bounds__(256) void w4a16_kernel(const uint8_t* __restrict__ 
 // on the matrix pipe, and the VALU only converts.  16-column tiles, 8 waves interleaving over K.
 // XROWS = activation rows staged (2 covers M <= 2, 8 covers M <= 8).
 // ---------------------------------------------------------------------------------------
-template <int XROWS, int NW>
+template <int XROWS, int NW, int BW, int CB>
 __global__ __launch_bounds__(64 * NW) void w8a16_r_kernel(const int8_t* __restrict__ Wq,
                                                           const half_t* __restrict__ X,
                                                           const half_t* __restrict__ scale,
                                                           float scalar_scale, float zero_point,
                                                           half_t* __restrict__ Y, int M, int N, int K) {
-  constexpr int RSW = 256 + 16;      // LDS bytes per staged weight row
-  constexpr int RSX = 512 + 16;      // ... per staged activation row
-  constexpr int WSTRIP = 16 * RSW;
+  // BW: weight bytes (= k) per row and band, 256 or 128.  CB: 16-column blocks per tile sharing the
+  // staged activations (tile = 16 * CB columns).  BW = 128 with CB = 2 reads half the activation
+  // bytes per weight byte of BW = 256 with CB = 1.
+  constexpr int BX = 2 * BW;           // activation bytes per row and band
+  constexpr int LPW = BW / 16;         // lanes per weight row piece
+  constexpr int RPW = 64 / LPW;        // weight rows per load instruction
+  constexpr int WI = 16 * CB / RPW;    // weight load instructions per step
+  constexpr int LPX = BX / 16;         // lanes per activation row piece
+  constexpr int RPX = 64 / LPX;        // activation rows per load instruction
+  constexpr int XI = XROWS / RPX;      // activation load instructions per step
+  constexpr int UNITS = BW / 32;       // 32-wide MFMA K units per band
+  constexpr int RSW = BW + 16;         // LDS bytes per staged weight row
+  constexpr int RSX = BX + 16;         // ... per staged activation row
+  constexpr int WSTRIP = 16 * CB * RSW;
   constexpr int XSTRIP = XROWS * RSX;
   constexpr int WAVE_LDS = WSTRIP + XSTRIP;
-  constexpr int XI = XROWS / 2;      // activation load instructions per step (2 rows each)
-  static_assert(WAVE_LDS >= 2 * 256 * (int)sizeof(float), "reduction scratch fits");
+  static_assert(XROWS % RPX == 0, "whole load instructions");
+  static_assert(WAVE_LDS >= 2 * CB * 256 * (int)sizeof(float), "reduction scratch fits");
   __shared__ __attribute__((aligned(16))) unsigned char smem[NW * WAVE_LDS];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int nw = blockDim.x >> 6;
-  const int j = lane & 15, g = lane >> 4;        // operand order
-  const int hw = lane >> 4, cw = lane & 15;      // weight load order: row 4i + hw, piece cw
-  const int hx = lane >> 5, cx = lane & 31;      // activation load order: row 2i + hx, piece cx
-  const int n0 = blockIdx.x * 16;
-  const int nbands = (K + 255) >> 8;             // K % 128 == 0: the last band may be half
+  const int j = lane & 15, g = lane >> 4;          // operand order
+  const int hw = lane / LPW, cw = lane % LPW;      // weight load order: row RPW*i + hw, piece cw
+  const int hx = lane / LPX, cx = lane % LPX;      // activation load order: row RPX*i + hx, piece cx
+  const int n0 = blockIdx.x * (16 * CB);
+  const int nbands = (K + BW - 1) / BW;            // K % 128 == 0: the last band may be partial
   const bool use_zp = zero_point != 0.f;
   unsigned char* wstrip = smem + wave * WAVE_LDS;
   unsigned char* xstrip = wstrip + WSTRIP;
@@ -506,46 +517,52 @@ __global__ __launch_bounds__(64 * NW) void w8a16_r_kernel(const int8_t* __restri
   const half_t* Xp = X + (size_t)hx * K + cx * 8;
   bool xrow[XI];
 #pragma unroll
-  for (int i = 0; i < XI; ++i) xrow[i] = (2 * i + hx) < M;
+  for (int i = 0; i < XI; ++i) xrow[i] = (RPX * i + hx) < M;
   const int stw_off = hw * RSW + cw * 16;
   const int stx_off = hx * RSX + cx * 16;
   const int ldw_off = j * RSW + g * 8;
   const int ldx_off = (j % XROWS) * RSX + g * 16;  // MFMA rows beyond XROWS re-read staged rows; unused
 
-  auto load_band = [&](int band, u32x4(&w)[4], u32x4(&x)[XI]) {
-    const bool okw = band < nbands && (band * 256 + cw * 16) < K;
-    const bool okx = band < nbands && (band * 256 + cx * 8) < K;
+  auto load_band = [&](int band, u32x4(&w)[WI], u32x4(&x)[XI]) {
+    const bool okw = band < nbands && (band * BW + cw * 16) < K;
+    const bool okx = band < nbands && (band * BW + cx * 8) < K;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) w[i] = okw ? load16<true>(Wp + (size_t)(4 * i) * K + (size_t)band * 256) : zero;
+    for (int i = 0; i < WI; ++i)
+      w[i] = okw ? load16<true>(Wp + (size_t)(RPW * i) * K + (size_t)band * BW) : zero;
 #pragma unroll
     for (int i = 0; i < XI; ++i)
-      x[i] = (okx && xrow[i]) ? load16<false>(Xp + (size_t)(2 * i) * K + (size_t)band * 256) : zero;
+      x[i] = (okx && xrow[i]) ? load16<false>(Xp + (size_t)(RPX * i) * K + (size_t)band * BW) : zero;
   };
-  float4_t acc = {0.f, 0.f, 0.f, 0.f}, xacc = {0.f, 0.f, 0.f, 0.f};
+  float4_t acc[CB], xacc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int b = 0; b < CB; ++b) acc[b] = float4_t{0.f, 0.f, 0.f, 0.f};
   const half8_t ones8 = {static_cast<half_t>(1.f), static_cast<half_t>(1.f), static_cast<half_t>(1.f),
                          static_cast<half_t>(1.f), static_cast<half_t>(1.f), static_cast<half_t>(1.f),
                          static_cast<half_t>(1.f), static_cast<half_t>(1.f)};
-  auto multiply = [&](const u32x4(&w)[4], const u32x4(&x)[XI]) {
+  auto multiply = [&](const u32x4(&w)[WI], const u32x4(&x)[XI]) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(wstrip + stw_off + 4 * i * RSW) = w[i];
+    for (int i = 0; i < WI; ++i) *reinterpret_cast<u32x4*>(wstrip + stw_off + RPW * i * RSW) = w[i];
 #pragma unroll
-    for (int i = 0; i < XI; ++i) *reinterpret_cast<u32x4*>(xstrip + stx_off + 2 * i * RSX) = x[i];
+    for (int i = 0; i < XI; ++i) *reinterpret_cast<u32x4*>(xstrip + stx_off + RPX * i * RSX) = x[i];
     wave_lds_sync();
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
+    for (int u = 0; u < UNITS; ++u) {
       const u32x4 xv = *reinterpret_cast<const u32x4*>(xstrip + ldx_off + u * 64);
-      const u32x2 wv = *reinterpret_cast<const u32x2*>(wstrip + ldw_off + u * 32);
-      half2_t h0, h1, h2, h3;
-      i8x4_to_half2x2(wv.x, h0, h1);
-      i8x4_to_half2x2(wv.y, h2, h3);
-      const half8_t wb = {h0[0], h0[1], h1[0], h1[1], h2[0], h2[1], h3[0], h3[1]};
-      acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(xv), wb, acc, 0, 0, 0);
+#pragma unroll
+      for (int b = 0; b < CB; ++b) {
+        const u32x2 wv = *reinterpret_cast<const u32x2*>(wstrip + b * 16 * RSW + ldw_off + u * 32);
+        half2_t h0, h1, h2, h3;
+        i8x4_to_half2x2(wv.x, h0, h1);
+        i8x4_to_half2x2(wv.y, h2, h3);
+        const half8_t wb = {h0[0], h0[1], h1[0], h1[1], h2[0], h2[1], h3[0], h3[1]};
+        acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(xv), wb, acc[b], 0, 0, 0);
+      }
       if (use_zp) xacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(xv), ones8, xacc, 0, 0, 0);
     }
     wave_lds_sync();
   };
 
-  u32x4 w0[4], w1[4], x0[XI], x1[XI];
+  u32x4 w0[WI], w1[WI], x0[XI], x1[XI];
   const int nsteps = (nbands + nw - 1) / nw;
   int step = stagger_start(nsteps, 0);
   auto next_band = [&]() {
@@ -562,22 +579,25 @@ __global__ __launch_bounds__(64 * NW) void w8a16_r_kernel(const int8_t* __restri
     multiply(w1, x1);
   }
 
-  // acc[r] = D[m = 4g + r][column j] (xacc: Σ x of row m in every column); waves meet in LDS
+  // acc[b][r] = D[m = 4g + r][column 16b + j] (xacc: sum of x of row m in every column); the waves
+  // meet in LDS: red[wave][0] = products [16][16*CB], red[wave][1] = activation sums [16][16]
+  constexpr int TN = 16 * CB;
   __syncthreads();
-  float(*red)[2][256] = reinterpret_cast<float(*)[2][256]>(smem);
+  float(*red)[2][16 * TN] = reinterpret_cast<float(*)[2][16 * TN]>(smem);
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
-    red[wave][0][(4 * g + r) * 16 + j] = acc[r];
+#pragma unroll
+    for (int b = 0; b < CB; ++b) red[wave][0][(4 * g + r) * TN + 16 * b + j] = acc[b][r];
     red[wave][1][(4 * g + r) * 16 + j] = xacc[r];
   }
   __syncthreads();
-  for (int e = threadIdx.x; e < 256; e += blockDim.x) {
-    const int m = e >> 4, n = n0 + (e & 15);
+  for (int e = threadIdx.x; e < 16 * TN; e += blockDim.x) {
+    const int m = e / TN, n = n0 + e % TN;
     if (m < M) {
       float sum = 0.f, xs = 0.f;
       for (int wv = 0; wv < nw; ++wv) {
         sum += red[wv][0][e];
-        xs += red[wv][1][e];
+        xs += red[wv][1][m * 16 + (e & 15)];
       }
       float sc = scalar_scale;
       if (scale != nullptr) sc *= static_cast<float>(scale[n]);
@@ -723,7 +743,7 @@ static int i8_waves(int K) {
 // Measured (us per call; lanes-along-K kernel / 4x4x4 MFMA kernel / row-load kernel):
 //   K = N = 8192   M=1 12.6 / 13.5 / 14.3   M=2 15.1 / 13.9 / 14.2   M=4 21.1 / 15.4 / 14.9   M=8 32.9 / 20.7 / 17.2
 //   K = N = 16384  M=1 41.2 /  -   / 44.8   M=2  -   / 50.2 / 45.8   M=4  -   / 52.7 / 47.8   M=8  -   / 66.9 / 49.7
-// The row-load kernel exists with 8 waves only.
+// (16-column tiles on 256-byte bands).  The row-load kernel exists with 8 waves only.
 bool launch_w8a16(const W8A16Args& a, hipStream_t s) {
   auto* Wq = static_cast<const int8_t*>(a.Wq);
   auto* X = static_cast<const half_t*>(a.x);
@@ -736,11 +756,26 @@ bool launch_w8a16(const W8A16Args& a, hipStream_t s) {
     hipLaunchKernelGGL((w8a16_mfma_kernel<1, 4, 2>), dim3(a.N / 16), dim3(256), 0, s, Wq, X, sc,
                        a.scalar_scale, a.zero_point, Y, a.M, a.N, a.K);
   } else if (a.M <= 2) {
-    hipLaunchKernelGGL((w8a16_r_kernel<2, 8>), dim3(a.N / 16), dim3(512), 0, s, Wq, X, sc,
+    hipLaunchKernelGGL((w8a16_r_kernel<2, 8, 256, 1>), dim3(a.N / 16), dim3(512), 0, s, Wq, X, sc,
                        a.scalar_scale, a.zero_point, Y, a.M, a.N, a.K);
   } else if (a.M <= 8) {
-    hipLaunchKernelGGL((w8a16_r_kernel<8, 8>), dim3(a.N / 16), dim3(512), 0, s, Wq, X, sc,
-                       a.scalar_scale, a.zero_point, Y, a.M, a.N, a.K);
+    // 32-column tiles on 128-byte bands read half the activation bytes per weight byte.  They pay
+    // where N/32 workgroups still put two workgroups (16 waves) on every CU -- K = N = 16384, M=8:
+    // 44.8 us against 49.3; K=4096 N=16384: 14.9 / 17.3 -- and lose where they leave one (K = N =
+    // 8192, M=8: 17.2 / 16.6: the conversion wants the waves).
+    const int t32 = a.N / 32;
+    const bool wide = a.N % 32 == 0 && t32 >= 512 && t32 % 512 == 0;
+    if (wide) {
+      if (a.M <= 4)
+        hipLaunchKernelGGL((w8a16_r_kernel<4, 8, 128, 2>), dim3(t32), dim3(512), 0, s, Wq, X, sc,
+                           a.scalar_scale, a.zero_point, Y, a.M, a.N, a.K);
+      else
+        hipLaunchKernelGGL((w8a16_r_kernel<8, 8, 128, 2>), dim3(t32), dim3(512), 0, s, Wq, X, sc,
+                           a.scalar_scale, a.zero_point, Y, a.M, a.N, a.K);
+    } else {
+      hipLaunchKernelGGL((w8a16_r_kernel<8, 8, 256, 1>), dim3(a.N / 16), dim3(512), 0, s, Wq, X, sc,
+                         a.scalar_scale, a.zero_point, Y, a.M, a.N, a.K);
+    }
   } else {
     return false;
   }

@@ -43,6 +43,25 @@ def test_w8a16_matches_oracle(device, M, N, K):
     assert_close_f16(_w8a16(Wq, x, scale, 0.5, 3.0, device), ref, "scale 0.5 zp 3")
 
 
+@pytest.mark.parametrize("M", [3, 4, 5, 7, 8])
+@pytest.mark.parametrize("N,K", [(16384, 128), (16384, 384), (16384, 1152), (32768, 384)])
+def test_w8a16_wide_tiles_for_wide_outputs(device, M, N, K):
+    # N / 32 a multiple of 512: 32-column tiles on 128-byte bands, 4- or 8-row activation
+    # strips; exact small integers first (any LDS layout mistake changes the bits), then random data
+    g = gen(4100 + M + N + K)
+    xi = torch.randint(-3, 4, (M, K), generator=g).half()
+    Wsmall = torch.randint(-8, 9, (N, K), generator=g, dtype=torch.int8)
+    ref, _ = oracle.gemv_w8a16(Wsmall.numpy(), xi.numpy(), None, 1.0, 0.0)
+    got = _w8a16(Wsmall, xi, None, 1.0, 0.0, device)
+    exact = np.abs(ref.astype(np.float32)) <= 2048
+    assert (got[exact] == ref[exact]).all() and exact.mean() > 0.9
+    Wq = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8)
+    x = normal((M, K), g)
+    scale = (torch.rand(N, generator=g) * 0.009 + 0.001).half()
+    ref, _ = oracle.gemv_w8a16(Wq.numpy(), x.numpy(), scale.numpy(), 0.5, 3.0)
+    assert_close_f16(_w8a16(Wq, x, scale, 0.5, 3.0, device), ref, "scale 0.5 zp 3")
+
+
 @pytest.mark.parametrize("M", [2, 3])
 def test_w8a16_large_weights_take_the_row_load_kernel(device, M):
     # above 2^27 weights M = 2..3 switches to the LDS-staged kernel (2-row and 8-row activation
