@@ -1,0 +1,94 @@
+"""Non-finite and extreme values: NaN / inf in the inputs stay in the outputs they belong to,
+fp16 overflow of a sum becomes inf, subnormal inputs are multiplied (not flushed), exactly as the
+CPU oracle (fp16 products, fp32 accumulation) has it."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from fastgate_amd import capi
+from helpers import capi_gemm, gen, normal, ptr, stream_ptr
+
+pytestmark = pytest.mark.gpu
+
+KN, NK = capi.FG_W_KN, capi.FG_W_NK
+
+
+def _gemm(A, W, layout, device):
+    M = A.shape[0]
+    N = W.shape[1] if layout == KN else W.shape[0]
+    C = torch.zeros((M, N), dtype=torch.half, device=device)
+    capi_gemm(A.to(device), W.to(device), C, layout)
+    torch.cuda.synchronize()
+    return C.cpu().numpy()
+
+
+def _same_class(got, ref):
+    """NaN where ref is NaN, the same inf where ref is inf, finite elsewhere."""
+    assert (np.isnan(got) == np.isnan(ref)).all()
+    inf = np.isinf(ref)
+    assert (got[inf] == ref[inf]).all()
+    assert np.isfinite(got[~inf & ~np.isnan(ref)]).all()
+
+
+@pytest.mark.parametrize("layout", [KN, NK])
+@pytest.mark.parametrize("M", [1, 2, 5, 8, 16])
+def test_nan_and_inf_stay_in_their_row_and_column(device, layout, M):
+    K, N = 1152, 384
+    g = gen(700 + M)
+    A = normal((M, K), g)
+    Wnk = normal((N, K), g, 0.05)
+    A[M - 1, 17] = float("nan")            # poisons output row M-1 only
+    Wnk[5, 900] = float("inf")             # poisons output column 5 (sign follows A[:, 900])
+    Wnk[300, 3] = float("-inf")
+    Wnk[301, 10] = float("inf")
+    Wnk[301, 11] = float("-inf")           # inf - inf (unless A is 0 there): NaN in column 301
+    W = Wnk if layout == NK else Wnk.t().contiguous()
+    ref, _ = oracle.gemm_f16(A.numpy(), W.numpy(), layout)
+    got = _gemm(A, W, layout, device)
+    _same_class(got, ref)
+    assert np.isnan(got[M - 1]).all()
+    clean = np.ones(N, bool)
+    clean[[5, 300, 301]] = False
+    fin = np.isfinite(ref)
+    assert fin[: M - 1][:, clean].all()
+    assert np.abs(got[fin].astype(np.float32) - ref[fin].astype(np.float32)).max(initial=0.0) < 2e-2
+
+
+@pytest.mark.parametrize("layout", [KN, NK])
+def test_overflow_of_the_sum_is_inf_and_subnormals_count(device, layout):
+    K, N, M = 256, 128, 3
+    # 256 products of 60000 * 1 overflow fp16 (65504) but not fp32: +-inf after the final rounding
+    A = torch.ones((M, K), dtype=torch.half)
+    A[1] = -1.0
+    A[2, 1:] = 0.0                          # row 2 sees a single product: finite
+    Wnk = torch.full((N, K), 60000.0, dtype=torch.half)
+    W = Wnk if layout == NK else Wnk.t().contiguous()
+    got = _gemm(A, W, layout, device)
+    assert (got[0] == np.inf).all() and (got[1] == -np.inf).all() and (got[2] == 60000.0).all()
+    # subnormal weights (2^-24) times 2^10 activations: 256 * 2^-14 = 2^-6, exact
+    sub = torch.tensor(np.full((N, K), 1, np.uint16).view(np.float16))   # smallest subnormal
+    W = sub if layout == NK else sub.t().contiguous()
+    A = torch.full((M, K), 1024.0, dtype=torch.half)
+    got = _gemm(A, W, layout, device)
+    assert (got == np.float16(2.0 ** -6)).all()
+
+
+def test_int8_gemv_with_non_finite_activations(device):
+    L = capi.lib()
+    N, K = 256, 512
+    g = gen(720)
+    Wq = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8)
+    Wq[:, 7] = 0                            # a zero weight times inf is NaN, as in the oracle
+    for M in (1, 2, 4, 8):
+        x = normal((M, K), g)
+        x[0, 7] = float("inf")
+        x[M - 1, 100] = float("nan")
+        ref, _ = oracle.gemv_w8a16(Wq.numpy(), x.numpy(), None, 1.0, 0.0)
+        y = torch.zeros((M, N), dtype=torch.half, device=device)
+        Wd, xd = Wq.to(device), x.to(device)
+        capi.check(L.fg_gemv_w8a16(ptr(Wd), ptr(xd), None, 1.0, 0.0, ptr(y), M, N, K, stream_ptr()), "w8a16")
+        torch.cuda.synchronize()
+        got = y.cpu().numpy()
+        _same_class(got, ref.reshape(M, N))
+        assert np.isnan(got[0]).all() and np.isnan(got[M - 1]).all()
