@@ -75,13 +75,14 @@ int finish_plan(int M, int N, int K, fg_plan_t* p) {
       if (!nk_mfma4_supported(p->m_block, p->tile_n, p->unroll)) return FG_ERR_UNSUPPORTED;
       break;
     case FG_KERNEL_NK_MFMA_R:
-      if (p->tile_n != 32) p->tile_n = 16;
+      if (p->tile_n != 32 && p->tile_n != 48 && p->tile_n != 64) p->tile_n = 16;
       p->m_block = 16;
       if (p->band == 0) {
         if (p->unroll != 1 && p->unroll != 2) return FG_ERR_UNSUPPORTED;
         p->band = 256 * p->unroll;
       }
       if (p->band != 128 && p->band != 256 && p->band != 512) return FG_ERR_UNSUPPORTED;
+      if (p->tile_n > 32 && p->band != 128) return FG_ERR_UNSUPPORTED;
       p->unroll = p->band == 512 ? 2 : 1;
       break;
     case FG_KERNEL_NK_MFMA_T:
@@ -205,6 +206,20 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
           wide_tiles = true;
           wide_band_waves = one_round ? 8 : 4;
           wide_band_split = s32;
+        }
+      }
+      // N = 12288 (and 24576) lands on whole CUs with 48-column tiles instead: three column blocks
+      // share a staged band.  Measured at N = 12288, M = 16 (us, 48 columns / the 16-column form):
+      // K=3072 14.4 / 15.9, K=6144 25.2 / 28.2, K=12288 47.0 / 52.6; M = 8: 14.0 / 15.1, then level.
+      if (!wide_band_waves && !wide_tiles && N % 48 == 0 && M >= 8 && M <= 16 && splitk <= 1) {
+        const int t48 = N / 48;
+        if ((t48 <= kCUs && 4 * t48 >= 3 * kCUs) || (t48 == 2 * kCUs && M >= 9)) {
+          p->tile_n = 48;
+          p->unroll = 1;
+          p->band = 128;
+          wide_tiles = true;
+          wide_band_waves = 8;
+          wide_band_split = 1;
         }
       }
     }

@@ -765,13 +765,25 @@ static bool nk_mfma_r_cb(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
 }
 
 // band = bytes of K per row and step: 512 (two rows per load instruction, four waves at most),
-// 256 or 128 (four or eight rows per instruction, up to eight waves).  tile_n = 16 or 32 (two
-// 16-column blocks sharing the staged activations).
+// 256 or 128 (four or eight rows per instruction, up to eight waves).  tile_n = 16, 32, 48 or 64
+// (one to four 16-column blocks sharing the staged activations; 48 and 64 on 128-byte bands only).
 bool launch_nk_mfma_r(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
   if (p.m_block != 16) return false;
   if (p.waves > 4 && !(p.waves == 8 && p.band <= 256)) return false;
   if (p.tile_n == 16) return nk_mfma_r_cb<1>(p, a, s);
   if (p.tile_n == 32) return nk_mfma_r_cb<2>(p, a, s);
+  if (p.tile_n == 48 || p.tile_n == 64) {  // three or four column blocks: 128-byte bands only
+    if (p.band != 128) return false;
+    const bool half_m = a.M <= 8;
+    if (p.tile_n == 48) {
+      if (half_m) nk_mfma_r_go<8, 128, 3>(p, a, s);
+      else nk_mfma_r_go<16, 128, 3>(p, a, s);
+    } else {
+      if (half_m) nk_mfma_r_go<8, 128, 4>(p, a, s);
+      else nk_mfma_r_go<16, 128, 4>(p, a, s);
+    }
+    return true;
+  }
   return false;
 }
 

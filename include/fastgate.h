@@ -54,7 +54,7 @@ enum {
   FG_KERNEL_NK_MFMA_T = 7, /* [N,K] weights, 16x16x32 MFMA fed through a wave-private LDS
                               transpose: loads are `unroll` (8/16) rows x 1 KB, every wave keeps
                               the A operands of its fixed K range in registers               */
-  FG_KERNEL_NK_MFMA_R = 8  /* [N,K] weights, 16x16x32 MFMA, 16-column tiles, weights AND
+  FG_KERNEL_NK_MFMA_R = 8  /* [N,K] weights, 16x16x32 MFMA, 16- to 64-column tiles, weights AND
                               activations loaded as contiguous row pieces and transposed in
                               wave-private LDS; fills the chip without split-K                */
 };

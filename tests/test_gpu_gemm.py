@@ -281,3 +281,38 @@ def test_split_deeper_than_k_has_idle_workgroups_that_contribute_zero(device, la
         assert_close_f16(got, ref, "S=16 on K=128, M=%d" % M)
         got, _ = _run(A, W, layout, device, splitk=3)
         assert_close_f16(got, ref, "S=3 on K=128, M=%d" % M)
+
+
+@pytest.mark.parametrize("tile", [48, 64])
+@pytest.mark.parametrize("waves", [1, 2, 4, 8])
+@pytest.mark.parametrize("splitk,fused", [(1, 0), (2, 0), (3, 1)])
+def test_row_load_mfma_kernel_three_and_four_column_blocks(device, tile, waves, splitk, fused):
+    N = 768 if tile == 48 else 512
+    for K in (128, 384, 2048, 4480):
+        for M in (1, 5, 8, 9, 16, 19):
+            A, W = _case(M, N, K, NK, 90 + M + K)
+            ref, _ = oracle.gemm_f16(A.numpy(), W.numpy(), NK)
+            kw = dict(kernel=capi.FG_KERNEL_NK_MFMA_R, tile_n=tile, waves=waves, splitk=splitk, fused=fused, band=128)
+            got, p = _run(A, W, NK, device, plan=make_plan(**kw))
+            assert p.tile_n == tile and p.grid_x == N // tile and p.band == 128
+            assert_close_f16(got, ref, "mfma_r tile %d M=%d K=%d" % (tile, M, K))
+    g = gen(92)
+    A = torch.randint(-2, 3, (16, 768), generator=g).half()
+    W = torch.randint(-3, 4, (N, 768), generator=g).half()
+    ref, _ = oracle.gemm_f16(A.numpy(), W.numpy(), NK)
+    got, _ = _run(A, W, NK, device, plan=make_plan(kernel=capi.FG_KERNEL_NK_MFMA_R, tile_n=tile, waves=waves, splitk=splitk, fused=fused, band=128))
+    assert (got == ref).all()
+    # wider tiles exist on 128-byte bands only
+    with pytest.raises(capi.FastgateError):
+        _run(A, W, NK, device, plan=make_plan(kernel=capi.FG_KERNEL_NK_MFMA_R, tile_n=tile, waves=4, band=256))
+
+
+@pytest.mark.parametrize("M", [8, 16])
+def test_planner_takes_48_column_tiles_at_n_12288(device, M):
+    N, K = 12288, 384
+    assert capi.plan(M, N, K, NK, 0).tile_n == 48
+    A, W = _case(M, N, K, NK, 95 + M)
+    ref, _ = oracle.gemm_f16(A.numpy(), W.numpy(), NK)
+    got, p = _run(A, W, NK, device)
+    assert p.tile_n == 48 and p.band == 128 and p.grid_x == 256
+    assert_close_f16(got, ref, "N=12288 M=%d" % M)
