@@ -75,14 +75,20 @@ int finish_plan(int M, int N, int K, fg_plan_t* p) {
       if (!nk_mfma4_supported(p->m_block, p->tile_n, p->unroll)) return FG_ERR_UNSUPPORTED;
       break;
     case FG_KERNEL_NK_MFMA_R:
-      if (p->tile_n != 32 && p->tile_n != 48 && p->tile_n != 64) p->tile_n = 16;
+      // 16, 32, 48, 64, or any width from 17 to 47 that divides N (one partly filled column
+      // block; 128-byte bands, 8 waves, no split-K)
+      if (p->tile_n != 32 && p->tile_n != 48 && p->tile_n != 64 &&
+          !(p->tile_n > 16 && p->tile_n < 48 && N % p->tile_n == 0)) {
+        p->tile_n = 16;
+      }
+      if (p->tile_n % 16 != 0 && (p->splitk != 1 || p->waves != 8)) return FG_ERR_UNSUPPORTED;
       p->m_block = 16;
       if (p->band == 0) {
         if (p->unroll != 1 && p->unroll != 2) return FG_ERR_UNSUPPORTED;
         p->band = 256 * p->unroll;
       }
       if (p->band != 128 && p->band != 256 && p->band != 512) return FG_ERR_UNSUPPORTED;
-      if (p->tile_n > 32 && p->band != 128) return FG_ERR_UNSUPPORTED;
+      if ((p->tile_n > 32 || p->tile_n % 16 != 0) && p->band != 128) return FG_ERR_UNSUPPORTED;
       p->unroll = p->band == 512 ? 2 : 1;
       break;
     case FG_KERNEL_NK_MFMA_T:
@@ -215,6 +221,23 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
         const int t48 = N / 48;
         if ((t48 <= kCUs && 4 * t48 >= 3 * kCUs) || (t48 == 2 * kCUs && M >= 9)) {
           p->tile_n = 48;
+          p->unroll = 1;
+          p->band = 128;
+          wide_tiles = true;
+          wide_band_waves = 8;
+          wide_band_split = 1;
+        }
+      }
+      // Otherwise N / 256 columns per workgroup, one workgroup per CU, when that is between 17 and
+      // 47 (a partly filled last column block; masked loads cost a little, so for M <= 8 only
+      // where the 16-column grid would not reach two workgroups per CU).  Measured (us, this / the
+      // 16-column form): N=11008 K=4096 M=16 17.4 / 19.0 (M=8: 17.4 / 17.0); N=10240 K=8192 M=16
+      // 28.4 / 33.0; N=9216 K=4096 M=4 17.0 / 15.1; N = K = 5120 M=16 13.3 / 16.4, M=8 12.1 / 14.1, M=4 12.3 / 13.1.
+      if (!wide_band_waves && !wide_tiles && N % kCUs == 0 && M >= 4 && M <= 16 && splitk <= 1) {
+        const int tw = N / kCUs;
+        const bool thin16 = N / 16 < 3 * kCUs / 2;  // 16-column tiles would leave CUs with one workgroup
+        if (tw >= 20 && tw < 48 && tw % 16 != 0 && K >= 1024 && (M >= 9 || thin16)) {
+          p->tile_n = tw;
           p->unroll = 1;
           p->band = 128;
           wide_tiles = true;

@@ -407,7 +407,7 @@ __global__ __launch_bounds__(256) void nk_mfma_t_kernel(const half_t* __restrict
 // waves, so two 8-wave workgroups fit a CU (16 waves per CU; M = 16 at K = N = 8192: 24.6 us
 // against 26.0 us with four waves on 512-byte bands).
 // ---------------------------------------------------------------------------------------
-template <int AROWS, int BAND, bool FULL, int NW, int CB>
+template <int AROWS, int BAND, bool FULL, int NW, int CB, bool RAGGED = false>
 __global__ __launch_bounds__(64 * NW) void nk_mfma_r_kernel(const half_t* __restrict__ A,
                                                         const half_t* __restrict__ W,
                                                         half_t* __restrict__ C,
@@ -415,7 +415,8 @@ __global__ __launch_bounds__(64 * NW) void nk_mfma_r_kernel(const half_t* __rest
                                                         int N, int K, int flags, const void* bias) {
   // AROWS: rows of A staged per step (8 covers M <= 8, 16 covers M <= 16).  BAND: bytes of K per
   // row and step (512, 256 or 128).  FULL: K is a multiple of the band and the bands divide evenly
-  // over the waves -- no masks needed.
+  // over the waves -- no masks needed.  RAGGED: the tile is N / gridDim.x columns wide, fewer than
+  // the 16 * CB the column blocks hold; the spare rows are never loaded and never stored.
   constexpr int LPR = BAND / 16;       // lanes per row piece
   constexpr int RPI = 64 / LPR;        // rows per load instruction
   constexpr int WI = 16 * CB / RPI;    // load instructions per step for the weights (CB blocks of 16 rows)
@@ -433,7 +434,8 @@ __global__ __launch_bounds__(64 * NW) void nk_mfma_r_kernel(const half_t* __rest
   const int nw = blockDim.x >> 6;
   const int j = lane & 15, g = lane >> 4;       // operand order: row j, 8 k at 8g within a unit
   const int h = lane / LPR, c = lane % LPR;     // load order: row RPI*i + h, 16-byte piece c
-  const int n0 = blockIdx.x * (16 * CB);
+  const int tw = RAGGED ? N / (int)gridDim.x : 16 * CB;  // columns of this tile
+  const int n0 = blockIdx.x * tw;
   const int m0 = blockIdx.y * 16;
   const int slots = nw * gridDim.z;
   const int slot = blockIdx.z * nw + wave;
@@ -457,7 +459,9 @@ __global__ __launch_bounds__(64 * NW) void nk_mfma_r_kernel(const half_t* __rest
     const bool ok = FULL || (band < nbands && (band * BK + c * 8) < K);
 #pragma unroll
     for (int i = 0; i < WI; ++i)
-      w[i] = ok ? load16<true>(Wp + (size_t)(RPI * i) * K + (size_t)band * BK) : zero;
+      w[i] = (ok && (!RAGGED || RPI * i + h < tw))
+                 ? load16<true>(Wp + (size_t)(RPI * i) * K + (size_t)band * BK)
+                 : zero;
 #pragma unroll
     for (int i = 0; i < AI; ++i)
       a[i] = (ok && arow[i]) ? load16<false>(Ap + (size_t)(RPI * i) * K + (size_t)band * BK) : zero;
@@ -514,7 +518,7 @@ __global__ __launch_bounds__(64 * NW) void nk_mfma_r_kernel(const half_t* __rest
     float sum = 0.f;
     for (int wv = 0; wv < nw; ++wv) sum += red[wv][e];
     const int mg = m0 + e / TN, n = n0 + e % TN;
-    if (e / TN < AROWS && mg < M) {
+    if (e / TN < AROWS && mg < M && (!RAGGED || e % TN < tw)) {
       if (gridDim.z == 1) {
         half_t* cp = C + (size_t)mg * N + n;
         *cp = finish_value(sum, cp, n, bias, flags);
@@ -772,6 +776,20 @@ bool launch_nk_mfma_r(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
   if (p.waves > 4 && !(p.waves == 8 && p.band <= 256)) return false;
   if (p.tile_n == 16) return nk_mfma_r_cb<1>(p, a, s);
   if (p.tile_n == 32) return nk_mfma_r_cb<2>(p, a, s);
+  if (p.tile_n % 16 != 0) {
+    // tile = N / grid.x columns in two or three column blocks, the last one partly filled: lets
+    // N / 256 columns go to each of 256 workgroups when that is not a multiple of 16
+    if (p.band != 128 || p.waves != 8 || p.grid_z != 1 || p.tile_n < 17 || p.tile_n > 47) return false;
+    const bool half_m = a.M <= 8;
+    if (p.tile_n < 32) {
+      if (half_m) FG_LAUNCH((nk_mfma_r_kernel<8, 128, false, 8, 2, true>), p, a, s);
+      else FG_LAUNCH((nk_mfma_r_kernel<16, 128, false, 8, 2, true>), p, a, s);
+    } else {
+      if (half_m) FG_LAUNCH((nk_mfma_r_kernel<8, 128, false, 8, 3, true>), p, a, s);
+      else FG_LAUNCH((nk_mfma_r_kernel<16, 128, false, 8, 3, true>), p, a, s);
+    }
+    return true;
+  }
   if (p.tile_n == 48 || p.tile_n == 64) {  // three or four column blocks: 128-byte bands only
     if (p.band != 128) return false;
     const bool half_m = a.M <= 8;

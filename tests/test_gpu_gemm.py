@@ -316,3 +316,40 @@ def test_planner_takes_48_column_tiles_at_n_12288(device, M):
     got, p = _run(A, W, NK, device)
     assert p.tile_n == 48 and p.band == 128 and p.grid_x == 256
     assert_close_f16(got, ref, "N=12288 M=%d" % M)
+
+
+@pytest.mark.parametrize("N,tile", [(384, 24), (640, 40), (1408, 44), (2176, 34), (640, 20), (1408, 22)])
+def test_row_load_mfma_kernel_tiles_that_are_not_multiples_of_16(device, N, tile):
+    # a partly filled last column block: the spare rows are never loaded and never stored
+    for K in (128, 384, 2048, 4480):
+        for M in (1, 5, 8, 9, 16, 19):
+            A, W = _case(M, N, K, NK, 97 + M + K)
+            ref, _ = oracle.gemm_f16(A.numpy(), W.numpy(), NK)
+            got, p = _run(A, W, NK, device, plan=make_plan(kernel=capi.FG_KERNEL_NK_MFMA_R, tile_n=tile, waves=8, band=128))
+            assert p.tile_n == tile and p.grid_x == N // tile and p.grid_z == 1
+            assert_close_f16(got, ref, "mfma_r tile %d M=%d K=%d" % (tile, M, K))
+            C0 = normal((M, N), gen(98), 2.0)
+            refa, _ = oracle.gemm_f16(A.numpy(), W.numpy(), NK, C=C0.numpy(), accumulate=True)
+            got, _ = _run(A, W, NK, device, accumulate=True, C0=C0, plan=make_plan(kernel=capi.FG_KERNEL_NK_MFMA_R, tile_n=tile, waves=8, band=128))
+            assert_close_f16(got, refa, "mfma_r tile %d accumulate M=%d K=%d" % (tile, M, K))
+    g = gen(99)
+    A = torch.randint(-2, 3, (16, 768), generator=g).half()
+    W = torch.randint(-3, 4, (N, 768), generator=g).half()
+    ref, _ = oracle.gemm_f16(A.numpy(), W.numpy(), NK)
+    got, _ = _run(A, W, NK, device, plan=make_plan(kernel=capi.FG_KERNEL_NK_MFMA_R, tile_n=tile, waves=8, band=128))
+    assert (got == ref).all()
+    # such tiles exist without split-K and with eight waves only
+    for bad in (dict(splitk=2), dict(waves=4)):
+        kw = dict(kernel=capi.FG_KERNEL_NK_MFMA_R, tile_n=tile, waves=8, band=128)
+        kw.update(bad)
+        with pytest.raises(capi.FastgateError):
+            _run(A, W, NK, device, plan=make_plan(**kw))
+
+
+def test_planner_gives_each_cu_n_over_256_columns_at_n_11008(device):
+    N, K, M = 11008, 1152, 16
+    A, W = _case(M, N, K, NK, 101)
+    ref, _ = oracle.gemm_f16(A.numpy(), W.numpy(), NK)
+    got, p = _run(A, W, NK, device)
+    assert p.tile_n == 43 and p.grid_x == 256 and p.band == 128 and p.waves == 8
+    assert_close_f16(got, ref, "N=11008 M=16")
