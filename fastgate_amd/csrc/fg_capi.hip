@@ -323,6 +323,45 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
           (size_t)N * K <= ((size_t)1 << 26) && items / (8 * best) >= 2) {
         p->waves = 8;
       }
+      // The rules above only try powers of two.  When their choice leaves the CUs unevenly loaded
+      // (tiles * S just over a multiple of 256: 80 tiles x 4 = 320 workgroups take 36 us where
+      // 80 x 3 = 240 take 29), search every S with either one 8-wave workgroup per CU or two
+      // 4-wave ones, scored by how evenly the CUs are filled, how evenly K divides over the wave
+      // slots, the partial traffic and the length of each wave's chain of loads.  Fitted to
+      // sweeps over N in {5120, 6144, 9216, 10240, 11008, 12288, 13824, 14336} x K in {3072..13824}.
+      {
+        auto score = [&](int S, int w) {
+          const int n = tiles * S;
+          const int per_cu = ceil_div(n, kCUs);
+          const double fill = (double)n / ((double)per_cu * kCUs);
+          const double per_wave = (double)items / (w * S);
+          const double chain = per_wave >= 8.0 ? 1.0 : std::sqrt(per_wave / 8.0);
+          const double partials = 1.0 / (1.0 + 4.0 * S * M / K);
+          return fill * balance(items, w * S) * partials * chain;
+        };
+        const int n0 = tiles * p->splitk;
+        const double fill0 = (double)n0 / ((double)ceil_div(n0, kCUs) * kCUs);
+        if (fill0 < 0.85 && M <= 16 && (size_t)N * K >= ((size_t)1 << 22)) {
+          double best_score = score(p->splitk, p->waves) * 1.05;  // switch for a clear win only
+          int best_s = 0, best_w = 0;
+          for (int S = 1; S <= 16; ++S) {
+            const int per_cu = ceil_div(tiles * S, kCUs);
+            if (per_cu > 2) break;
+            const int w = per_cu == 1 ? 8 : 4;
+            if (items / (w * S) < 2) break;
+            const double sc = score(S, w);
+            if (sc > best_score + 1e-9) {
+              best_score = sc;
+              best_s = S;
+              best_w = w;
+            }
+          }
+          if (best_s) {
+            p->splitk = best_s;
+            p->waves = best_w;
+          }
+        }
+      }
     } else if (wide_band_split) {
       p->splitk = wide_band_split;
       p->fused = 1;
