@@ -127,6 +127,79 @@ int finish_plan(int M, int N, int K, fg_plan_t* p) {
   return FG_OK;
 }
 
+// Wider tiles of the row-load kernel on 128-byte bands.  Two, three or a ragged number of column
+// blocks share a staged band of activations and a band carries half the activation bytes, so the
+// L2 traffic for A drops to a quarter or less of the 16-column / 256-byte form -- but the grid
+// shrinks with the tile, so it has to land on whole CUs: 192..256 workgroups of 8 waves (one a
+// CU) or 448..512 (two a CU).  Candidates, measured against the 16-column form (us):
+//   32 columns            K = N = 8192 M=16 22.8 / 24.7, M=8 22.9 / 23.3; K = N = 6144 M=16 16.6 / 18.9;
+//                         K=2048 N=8192 M=16 7.9 / 9.0; K=4096 N=16384 M=16 22.4 / 24.3 (4 waves)
+//   32 columns, split-K   N=3072 K=12288 M=16 S=2 18.2 / 19.4 (M <= 8: 16.3 / 16.1, so M >= 9 only);
+//                         N=2560 K=10240 M=16 S=3 13.3 / 16.7; N=5120 K=13824 S=3 (two a CU) 24.8 / 27.0
+//   48 columns            N = 12288: K=3072 M=16 14.4 / 15.9, K=12288 47.0 / 52.6
+//   N/256 or N/512 columns with a partly filled last block (masked loads cost a little):
+//                         N=11008 K=4096 M=16 17.4 / 19.0 (M=8: 17.4 / 17.0); N=10240 K=8192 M=16
+//                         28.4 / 33.0; N = K = 5120 M=8 12.1 / 14.1; N=6144 K=4096 M=16 11.2 / 12.9
+//                         (24 columns, against 32); N=13824 K=5120 M=16 26.1 / 30.3 (27 columns, two a CU)
+// 384 workgroups (N = 12288 at 32 columns) leave half the CUs with one: 46+ us against 45.
+struct WideTile {
+  int tile_n = 0, waves = 0, splitk = 1;
+};
+WideTile pick_wide_tile(int M, int N, int K, int splitk) {
+  WideTile best;
+  double best_fill = 0.0;
+  // a later candidate replaces an earlier one only when it fills the CUs better by `margin`
+  auto offer = [&](int tile, int waves, int S, int wgs, bool allowed, double margin = 0.04) {
+    if (!allowed) return;
+    const double fill = (double)wgs / (double)(ceil_div(wgs, kCUs) * kCUs);
+    if (fill > best_fill + margin) {
+      best_fill = fill;
+      best = WideTile{tile, waves, S};
+    }
+  };
+  const bool auto_split = splitk == 0;
+  if (N % 32 == 0) {
+    const int t32 = N / 32;
+    offer(32, 8, 1, t32, t32 <= kCUs && 4 * t32 >= 3 * kCUs && (M >= 4 || t32 < kCUs));
+    offer(32, 4, 1, t32, 8 * t32 >= 7 * 2 * kCUs && t32 <= 2 * kCUs && (t32 == 2 * kCUs ? M >= 5 : M >= 9));
+  }
+  if (N % 48 == 0) {
+    const int t48 = N / 48;
+    offer(48, 8, 1, t48, M >= 8 && ((t48 <= kCUs && 4 * t48 >= 3 * kCUs) || (t48 == 2 * kCUs && M >= 9)));
+  }
+  if (N % 32 == 0 && auto_split && N / 32 < 3 * kCUs / 4) {
+    // split-K keeps at least 3072 k per split (six 128-byte bands for each of eight waves)
+    const int t32 = N / 32;
+    for (int S = 2; S <= 4; ++S) {
+      const int wgs = t32 * S;
+      const bool long_k = K / S >= 3072 && (S > 2 || K >= 8192);
+      offer(32, 8, S, wgs, long_k && M >= 9 && wgs <= kCUs && 4 * wgs >= 3 * kCUs);
+    }
+    // two workgroups a CU, only where no split lands on one a CU
+    bool one_a_cu = false;
+    for (int S = 1; S <= 4; ++S) one_a_cu |= t32 * S <= kCUs && 4 * t32 * S >= 3 * kCUs;
+    for (int S = 2; S <= 4 && !one_a_cu; ++S) {
+      const int wgs = t32 * S;
+      offer(32, 8, S, wgs, K / S >= 3072 && M >= 4 && wgs <= 2 * kCUs && 8 * wgs >= 7 * 2 * kCUs);
+    }
+  }
+  // Ragged tiles pay for their masked loads and empty operand slots: they need a clearly better
+  // fill (N = 7168, M = 9: 28 columns 19.4 us, 32 columns 18.2), three column blocks (33..47 columns) against 48 columns too (N = 9216:
+  // 36 columns 17.3 us, 48 columns 15.5), and two ragged workgroups a CU lose to 448 workgroups of
+  // 32 columns (N=14336 K=4096 M=16: 23.9 / 22.0).
+  if (K >= 1024 && N % kCUs == 0) {
+    const int tw = N / kCUs;
+    const bool thin16 = N / 16 < 3 * kCUs / 2;  // 16-column tiles would leave CUs with one workgroup
+    offer(tw, 8, 1, kCUs, tw >= 20 && tw < 48 && tw % 16 != 0 && (M >= 9 || (thin16 && M >= 4)),
+          tw > 32 ? 0.3 : 0.15);
+  }
+  if (K >= 1024 && N % (2 * kCUs) == 0) {
+    const int tw = N / (2 * kCUs);
+    offer(tw, 8, 1, 2 * kCUs, tw >= 20 && tw < 48 && tw % 16 != 0 && M >= 9, 0.15);
+  }
+  return best;
+}
+
 int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
   std::memset(p, 0, sizeof(*p));
   p->stream_w = 1;
@@ -153,8 +226,9 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
       p->unroll = (K >= 16384 || M > 2) ? 2 : 1;
       items = ceil_div(K / 8, 64 * p->unroll);
       p->stagger = items <= 16;  // at most 4 steps for 4 waves
-    } else if (M <= 8 && K >= 16384 && N >= 8192) {
-      // (K = N = 16384: M = 4 78.7 us against 79.9 for the row-load kernel, M = 8 77.5 / 78.9)
+    } else if (M <= 8 && K >= 16384 && N >= 16384) {
+      // (K = N = 16384: M = 4 78.7 us against 79.9 for the row-load kernel, M = 8 77.5 / 78.9; at
+      // N = 8192, K = 28672 the row-load kernel is ahead, M = 8 69.8 / 78.3)
       p->kernel = FG_KERNEL_NK_MFMA4;
       p->m_block = M <= 4 ? 4 : 8;
       if (K >= 16384) {
@@ -187,62 +261,15 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
       }
       items = ceil_div(K, 128 * p->unroll);
       row_tiles = true;
-      // 32-column tiles on 128-byte bands: two column blocks share the staged activations and a
-      // band carries half the activation bytes, so the L2 traffic for A is a quarter of the
-      // 16-column / 256-byte form -- but the grid is only N/32 workgroups, so it has to land on
-      // (nearly) whole CUs: 192..256 workgroups of 8 waves, or 512 of 4.  Measured (us, this form
-      // / the rule above): K = N = 8192 M=16 22.8 / 24.7, M=8 22.9 / 23.3; K = N = 6144 M=16
-      // 16.6 / 18.9, M=4 14.3 / 15.7; K=2048 N=8192 M=16 7.9 / 9.0; K=4096 N=16384 M=16 22.4 / 24.3;
-      // K=12288 N=3072 with two-way split-K M=16 18.2 / 19.4 (M <= 8: 16.3 / 16.1, so not there).
-      // 384 workgroups (N = 12288) leave half the CUs with one: 46+ us against 45 at K = 12288.
-      const int t32 = N / 32;
-      int s32 = 0;
-      if (N % 32 == 0) {
-        if (t32 >= 192) s32 = 1;
-        else if (2 * t32 >= 192 && K >= 8192 && M >= 9) s32 = 2;
-      }
-      if (s32 && M <= 16 && !wide_tiles && (splitk == 0 || (splitk == 1 && s32 == 1))) {
-        const int wgs = t32 * s32;
-        const bool one_round = wgs <= kCUs && 4 * wgs >= 3 * kCUs;
-        const bool two_rounds = wgs == 2 * kCUs && M >= 5;
-        if ((one_round && (M >= 4 || t32 < kCUs)) || two_rounds) {
-          p->tile_n = 32;
+      if (!wide_tiles && M <= 16 && splitk <= 1) {
+        const WideTile wt = pick_wide_tile(M, N, K, splitk);
+        if (wt.tile_n) {
+          p->tile_n = wt.tile_n;
           p->unroll = 1;
           p->band = 128;
           wide_tiles = true;
-          wide_band_waves = one_round ? 8 : 4;
-          wide_band_split = s32;
-        }
-      }
-      // N = 12288 (and 24576) lands on whole CUs with 48-column tiles instead: three column blocks
-      // share a staged band.  Measured at N = 12288, M = 16 (us, 48 columns / the 16-column form):
-      // K=3072 14.4 / 15.9, K=6144 25.2 / 28.2, K=12288 47.0 / 52.6; M = 8: 14.0 / 15.1, then level.
-      if (!wide_band_waves && !wide_tiles && N % 48 == 0 && M >= 8 && M <= 16 && splitk <= 1) {
-        const int t48 = N / 48;
-        if ((t48 <= kCUs && 4 * t48 >= 3 * kCUs) || (t48 == 2 * kCUs && M >= 9)) {
-          p->tile_n = 48;
-          p->unroll = 1;
-          p->band = 128;
-          wide_tiles = true;
-          wide_band_waves = 8;
-          wide_band_split = 1;
-        }
-      }
-      // Otherwise N / 256 columns per workgroup, one workgroup per CU, when that is between 17 and
-      // 47 (a partly filled last column block; masked loads cost a little, so for M <= 8 only
-      // where the 16-column grid would not reach two workgroups per CU).  Measured (us, this / the
-      // 16-column form): N=11008 K=4096 M=16 17.4 / 19.0 (M=8: 17.4 / 17.0); N=10240 K=8192 M=16
-      // 28.4 / 33.0; N=9216 K=4096 M=4 17.0 / 15.1; N = K = 5120 M=16 13.3 / 16.4, M=8 12.1 / 14.1, M=4 12.3 / 13.1.
-      if (!wide_band_waves && !wide_tiles && N % kCUs == 0 && M >= 4 && M <= 16 && splitk <= 1) {
-        const int tw = N / kCUs;
-        const bool thin16 = N / 16 < 3 * kCUs / 2;  // 16-column tiles would leave CUs with one workgroup
-        if (tw >= 20 && tw < 48 && tw % 16 != 0 && K >= 1024 && (M >= 9 || thin16)) {
-          p->tile_n = tw;
-          p->unroll = 1;
-          p->band = 128;
-          wide_tiles = true;
-          wide_band_waves = 8;
-          wide_band_split = 1;
+          wide_band_waves = wt.waves;
+          wide_band_split = wt.splitk;
         }
       }
     }
