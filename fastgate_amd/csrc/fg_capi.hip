@@ -401,6 +401,9 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
       while (S > 1 && items / (p->waves * S) < 2) --S;  // keep two bands per wave
       p->splitk = S;
       p->fused = 1;
+      // with only two 256-byte bands left per wave, four of 128 bytes pipeline better
+      // (N=1024 K=8192 S=4: M=8 7.8 us against 8.9, M=16 8.0 / 9.4)
+      if (S > 1 && p->unroll == 1 && items / (p->waves * S) <= 2) p->band = 128;
     } else {
       p->splitk = pick_splitk(tiles, p->waves, items, M, N, K, kCUs);
     }
