@@ -65,7 +65,17 @@ def algorithmic_bytes(M: int) -> int:
     return 2 * K * N + 2 * M * K + 2 * M * N
 
 
-def run_sweep(torch, sg, capi, dev, steps, warmup):
+MODEL_SHAPES = [
+    # (label, N, K): projection shapes of common decoder layers, weights [N,K] or [K,N]
+    ("7B attn 4096x4096", 4096, 4096), ("7B up 11008x4096", 11008, 4096), ("7B down 4096x11008", 4096, 11008),
+    ("13B attn 5120x5120", 5120, 5120), ("13B up 13824x5120", 13824, 5120), ("13B down 5120x13824", 5120, 13824),
+    ("8B up 14336x4096", 14336, 4096), ("8B down 4096x14336", 4096, 14336), ("8B qkv 6144x4096", 6144, 4096),
+    ("70B attn 8192x8192", 8192, 8192), ("70B up 28672x8192", 28672, 8192), ("70B down 8192x28672", 8192, 28672),
+    ("70B kv 1024x8192", 1024, 8192), ("DiT up 12288x3072", 12288, 3072), ("DiT down 3072x12288", 3072, 12288),
+]
+
+
+def run_sweep(torch, sg, capi, dev, steps, warmup, models=False):
     """Per-shape timing of the benchmark configurations: us per call, GB/s on algorithmic bytes,
     fraction of the 8 TB/s peak, and the plan (kernel, split-K, tile) the library chose."""
     import ctypes
@@ -117,6 +127,15 @@ def run_sweep(torch, sg, capi, dev, steps, warmup):
                      "GBps": round(by / us_call / 1e3, 1), "TFLOPs": round(2.0 * M * Nn * Kk / us_call / 1e6, 2),
                      "frac_hbm_peak": round(by / us_call / 1e3 / HBM_PEAK_GBPS, 4),
                      "frac_read_ceiling": round(by / us_call / 1e3 / ceiling, 4)})
+
+    if models:
+        for li, (label, Nn, Kk) in enumerate(MODEL_SHAPES):
+            for M in (1, 8, 16):
+                fp16_case(label, "edgemm_m8n128k64x4_bt", M, Kk, Nn, capi.FG_W_NK, 3000 + li)
+                fp16_case(label, "edgemm_m8n128k64x4", M, Kk, Nn, capi.FG_W_KN, 3000 + li)
+        return {"sweep": rows, "read_ceiling_GBps": round(ceiling, 1), "hbm_peak_GBps": HBM_PEAK_GBPS,
+                "steps": steps, "warmup": warmup, "data": "synthetic", "dtype": "f16",
+                "device": torch.cuda.get_device_name(0)}
 
     fp16_case("C1 fastgemv", "fastgemv", 1, 4096, 4096, capi.FG_W_NK, 1001)
     fp16_case("C2 edgemm", "edgemm_m8n128k64x4", 8, 4096, 11008, capi.FG_W_KN, 1002)
@@ -206,6 +225,8 @@ def main() -> int:
                     help="instead of the headline step, time every benchmark configuration (the fastgemv, "
                          "edgemm, flat-GEMM and int8 shapes and the M x K=N shape sweep on both weight "
                          "layouts) and print one JSON object with the plan and roofline figures per shape")
+    ap.add_argument("--sweep-models", action="store_true",
+                    help="as --sweep, over the projection shapes of common decoder layers (both layouts, M = 1, 8, 16)")
     ap.add_argument("--cpu-repeats", type=int, default=8, help="repetitions of the step on the CPU oracle (0 = skip)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -245,8 +266,8 @@ def main() -> int:
                                                                  "launches": 5}}}))
         return 0
 
-    if args.sweep:
-        print(json.dumps(run_sweep(torch, sg, capi, dev, args.steps, args.warmup)))
+    if args.sweep or args.sweep_models:
+        print(json.dumps(run_sweep(torch, sg, capi, dev, args.steps, args.warmup, models=args.sweep_models)))
         return 0
 
     # ---- synthetic inputs, seeded on the CPU so the CPU baseline sees the same bits ----------

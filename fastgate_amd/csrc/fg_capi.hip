@@ -136,7 +136,8 @@ int finish_plan(int M, int N, int K, fg_plan_t* p) {
 //                         K=2048 N=8192 M=16 7.9 / 9.0; K=4096 N=16384 M=16 22.4 / 24.3 (4 waves)
 //   32 columns, split-K   N=3072 K=12288 M=16 S=2 18.2 / 19.4 (M <= 8: 16.3 / 16.1, so M >= 9 only);
 //                         N=2560 K=10240 M=16 S=3 13.3 / 16.7; N=5120 K=13824 S=3 (two a CU) 24.8 / 27.0
-//   48 columns            N = 12288: K=3072 M=16 14.4 / 15.9, K=12288 47.0 / 52.6
+//   48 columns            N = 12288: K=3072 M=16 14.4 / 15.9, K=12288 47.0 / 52.6; N=3072 K=12288 split 4 ways
+//   64 columns            N = 28672, K = 8192
 //   N/256 or N/512 columns with a partly filled last block (masked loads cost a little):
 //                         N=11008 K=4096 M=16 17.4 / 19.0 (M=8: 17.4 / 17.0); N=10240 K=8192 M=16
 //                         28.4 / 33.0; N = K = 5120 M=8 12.1 / 14.1; N=6144 K=4096 M=16 11.2 / 12.9
@@ -167,6 +168,11 @@ WideTile pick_wide_tile(int M, int N, int K, int splitk) {
     const int t48 = N / 48;
     offer(48, 8, 1, t48, M >= 8 && ((t48 <= kCUs && 4 * t48 >= 3 * kCUs) || (t48 == 2 * kCUs && M >= 9)));
   }
+  if (N % 64 == 0) {
+    // very wide outputs (N=28672 K=8192 M=16: 64 columns 72.1 us, 32 columns 74.0, 16 columns 81+)
+    const int t64 = N / 64;
+    offer(64, 8, 1, t64, M >= 9 && K >= 8192 && t64 <= 2 * kCUs && 8 * t64 >= 7 * 2 * kCUs);
+  }
   if (N % 32 == 0 && auto_split && N / 32 < 3 * kCUs / 4) {
     // split-K keeps at least 3072 k per split (six 128-byte bands for each of eight waves)
     const int t32 = N / 32;
@@ -174,6 +180,14 @@ WideTile pick_wide_tile(int M, int N, int K, int splitk) {
       const int wgs = t32 * S;
       const bool long_k = K / S >= 3072 && (S > 2 || K >= 8192);
       offer(32, 8, S, wgs, long_k && M >= 9 && wgs <= kCUs && 4 * wgs >= 3 * kCUs);
+    }
+    if (N % 48 == 0) {
+      // (N=3072 K=12288 M=16: 48 columns split 4 ways 16.4 us, 32 columns split 2 ways 17.9)
+      const int t48 = N / 48;
+      for (int S = 2; S <= 4; ++S) {
+        const int wgs = t48 * S;
+        offer(48, 8, S, wgs, K / S >= 3072 && M >= 9 && wgs <= kCUs && 4 * wgs >= 3 * kCUs);
+      }
     }
     // two workgroups a CU, only where no split lands on one a CU
     bool one_a_cu = false;
@@ -252,13 +266,6 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
       p->m_block = 16;
       p->tile_n = 16;
       p->unroll = (K >= 16384 && N >= 8192) ? 2 : 1;
-      if (M > 8 && K >= 8192 && N / 32 >= 2 * kCUs) {
-        // plenty of tiles: two 16-column blocks share the staged activations, four waves
-        // (K = N = 16384, M=16: 79.0 us against 84.8)
-        p->tile_n = 32;
-        p->unroll = 1;
-        wide_tiles = true;
-      }
       items = ceil_div(K, 128 * p->unroll);
       row_tiles = true;
       if (!wide_tiles && M <= 16 && splitk <= 1) {
