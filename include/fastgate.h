@@ -72,7 +72,8 @@ typedef struct fg_plan_t {
   int fused;    /* with S > 1: 1 = the workgroup that finishes a tile last sums the
                    partials in the same launch (one counter atomic per workgroup),
                    0 = a second kernel does                                            */
-  int tile_n;   /* output columns per workgroup                                       */
+  int tile_n;   /* output columns per workgroup; FG_KERNEL_NK_MFMA_R takes 16, 32, 48, 64 or,
+                   with band = 128, 8 waves and no split, any divisor of N from 17 to 47  */
   int m_block;  /* rows of A per workgroup (grid.y = ceil(M / m_block))               */
   int waves;    /* wavefronts per workgroup; they interleave over K, reduced in LDS   */
   int unroll;   /* independent 16-byte load groups in flight per lane and step        */
