@@ -219,10 +219,9 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
   p->stream_w = 1;
   // Split-K can finish inside the launch (the last workgroup of a tile sums the partials) or
   // in a second kernel.  Measured at K = N = 8192, S = 4 (us per call, second kernel / in-launch):
-  // [K,N] M=1 26.4 / 25.7, M=8 26.2 / 25.5, M=16 26.4 / 27.0; [N,K] transposing kernel M=8
-  // 26.2 / 25.6, M=16 27.4 / 27.8.  Either way the dependent tail costs 3-4 us; in-launch wins
-  // while the partials of a tile are small.
-  p->fused = M <= 8;
+  // [K,N] M=1 26.4 / 25.0, M=8 26.2 / 25.2, M=16 26.5 / 25.9.  Beyond one block of 16 rows the
+  // second kernel takes over.
+  p->fused = M <= 16;
   int items = 1;
   bool row_tiles = false;   // the 16-column row-load kernel picks its own split
   bool wide_tiles = false;  // ... in its 32-column form
@@ -294,7 +293,6 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
     // each partial in turn, deeper splits of shorter steps win (v_dot2, M = 1, two units / one:
     // K = N = 4096 10.5 / 9.7 us, K=3072 N=12288 16.7 / 15.5, K=4096 N=11008 18.5 / 17.3)
     p->unroll = 1;
-    p->fused = M <= 16;  // 26.5 / 25.8 us at K = N = 8192, M = 16 (second kernel / in-launch)
     items = ceil_div(K / 32, p->unroll);
   }
   {

@@ -353,3 +353,35 @@ def test_planner_gives_each_cu_n_over_256_columns_at_n_11008(device):
     got, p = _run(A, W, NK, device)
     assert p.tile_n == 43 and p.grid_x == 256 and p.band == 128 and p.waves == 8
     assert_close_f16(got, ref, "N=11008 M=16")
+
+
+def test_in_launch_split_k_is_stable_over_many_back_to_back_calls(device):
+    # 600 calls that complete split-K inside the launch, alternating shapes and layouts on ONE
+    # workspace with no host synchronisation in between: every output must equal the first
+    # output of its shape bit for bit, and the counters must end at zero
+    from helpers import ptr, stream_ptr
+    L = capi.lib()
+    hdr = L.fg_workspace_header_bytes()
+    ws = torch.full((hdr + 16 * 16 * 4096 * 4,), 0xFF, dtype=torch.uint8, device=device)
+    capi.check(L.fg_workspace_init(ptr(ws), ws.numel(), stream_ptr()), "init")
+    cases = []
+    for i, (M, N, K, layout, S) in enumerate([(1, 4096, 4096, KN, 8), (8, 2048, 4096, KN, 5), (16, 1024, 8192, KN, 3),
+                                              (16, 3072, 6144, NK, 4), (5, 4096, 2048, KN, 16), (12, 1024, 8192, NK, 4)]):
+        A, W = _case(M, N, K, layout, 500 + i)
+        Ad, Wd = A.to(device), W.to(device)
+        p = capi.plan(M, N, K, layout, S)
+        assert p.splitk == S and p.fused == 1, p.as_dict()
+        outs = [torch.full((M, N), float("nan"), dtype=torch.half, device=device) for _ in range(100)]
+        ref, _ = oracle.gemm_f16(A.numpy(), W.numpy(), layout)
+        cases.append((M, N, K, layout, S, Ad, Wd, outs, ref))
+    for it in range(100):
+        for (M, N, K, layout, S, Ad, Wd, outs, _) in cases:
+            st = L.fg_gemm_f16(ptr(Ad), ptr(Wd), ptr(outs[it]), M, N, K, layout, 0, S, ptr(ws), ws.numel(), stream_ptr())
+            assert st == 0
+    torch.cuda.synchronize()
+    assert int(ws[:hdr].view(torch.int32).abs().sum()) == 0
+    for (M, N, K, layout, S, Ad, Wd, outs, ref) in cases:
+        first = outs[0].cpu().numpy()
+        assert_close_f16(first, ref, "M=%d N=%d K=%d S=%d" % (M, N, K, S))
+        stack = torch.stack(outs).view(torch.int16)
+        assert bool((stack == stack[0]).all()), (M, N, K, layout, S)
