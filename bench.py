@@ -216,8 +216,8 @@ def run_sweep(torch, sg, capi, dev, steps, warmup, models=False):
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--calibrate-traffic", action="store_true",
                     help="only run kernels of known traffic (1 GiB read probe, 256 MiB device copy) for "
                          "scaling rocprofv3's FETCH_SIZE / WRITE_SIZE counters, then exit")
