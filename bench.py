@@ -50,8 +50,8 @@ def _traffic(fetch_kib: float, write_kib: float) -> int:
 
 
 TRAFFIC_BYTES = {
-    "nk_dot2_M1": _traffic(65637.6, 64.0),
-    "nk_mfma_r_M8": _traffic(66091.5, 128.0),
+    "nk_dot2_M1": _traffic(65630.6, 64.0),
+    "nk_mfma_r_M8": _traffic(66083.0, 128.0),
     "nk_mfma_r_M16": _traffic(66604.5, 256.0),
     # [K,N]: split-K partials are written through and read back inside the launch; WRITE_SIZE counts
     # the write-through stores twice (M=1: 8 x 16 KiB of partials, M=8: 4 x 256 KiB, M=16: 4 x 512 KiB)
