@@ -118,6 +118,11 @@ def run_sweep(torch, sg, capi, dev, steps, warmup, models=False):
         else:
             call = lambda i: fn(a, ws[i % nbuf], c)
         us_call = time_us(call)
+        # the vendor GEMM (hipBLASLt through at::matmul_out) on the same buffers, as the reference's
+        # scripts print their cuBLAS column
+        vend = sg.hgemm_tr if layout == capi.FG_W_NK else sg.hgemm
+        c2 = c.view(M, Nn)
+        us_vendor = time_us(lambda i: vend(a, ws[i % nbuf], c2))
         by = 2 * Kk * Nn + 2 * M * Kk + 2 * M * Nn
         p = capi.plan(M, Nn, Kk, layout, 0).as_dict()
         rows.append({"config": name, "op": op, "M": M, "K": Kk, "N": Nn,
@@ -126,7 +131,8 @@ def run_sweep(torch, sg, capi, dev, steps, warmup, models=False):
                      "tile_n": p["tile_n"], "bytes": by, "us_per_call": round(us_call, 2),
                      "GBps": round(by / us_call / 1e3, 1), "TFLOPs": round(2.0 * M * Nn * Kk / us_call / 1e6, 2),
                      "frac_hbm_peak": round(by / us_call / 1e3 / HBM_PEAK_GBPS, 4),
-                     "frac_read_ceiling": round(by / us_call / 1e3 / ceiling, 4)})
+                     "frac_read_ceiling": round(by / us_call / 1e3 / ceiling, 4),
+                     "vendor_us_per_call": round(us_vendor, 2)})
 
     if models:
         for li, (label, Nn, Kk) in enumerate(MODEL_SHAPES):
