@@ -508,8 +508,14 @@ int fg_gemm_f16(const void* A, const void* W, void* C, int M, int N, int K, int 
                 int accumulate, int splitk, void* ws, size_t ws_bytes, void* stream) {
   if (A == nullptr || W == nullptr || C == nullptr) return FG_ERR_INVALID_ARG;
   fg_plan_t p;
-  const int st = fg_plan(M, N, K, w_layout, splitk, &p);
+  int st = fg_plan(M, N, K, w_layout, splitk, &p);
   if (st != FG_OK) return st;
+  if (splitk == 0 && p.splitk > 1 && (ws == nullptr || ws_bytes < p.workspace_bytes)) {
+    // the library's own choice of a split needs a workspace the caller did not bring: run
+    // unsplit (slower where the grid then leaves CUs idle) instead of failing
+    st = fg_plan(M, N, K, w_layout, 1, &p);
+    if (st != FG_OK) return st;
+  }
   return fg::run_gemm(A, W, C, M, N, K, accumulate, p, ws, ws_bytes,
                       static_cast<hipStream_t>(stream));
 }

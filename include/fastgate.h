@@ -91,7 +91,9 @@ typedef struct fg_plan_t {
 /*
  * C = A·W (accumulate = 0) or C += A·W (accumulate = 1; C holds fp16 on entry and the sum
  * is formed in fp32 before the single rounding).
- *   splitk  0 = library heuristic, S >= 1 = forced (the reference's trailing `int bz`).
+ *   splitk  0 = library heuristic, S >= 1 = forced (the reference's trailing `int bz`).  With 0 and
+ *           no (or too small a) workspace the call runs unsplit instead of failing; a forced
+ *           S > 1 without workspace is FG_ERR_WORKSPACE.
  *   ws      device scratch of at least fg_workspace_bytes() bytes when the plan's
  *           splitk > 1, else may be NULL.  Its first fg_workspace_header_bytes() bytes hold
  *           arrival counters: zero them once with fg_workspace_init() (or allocate zeroed

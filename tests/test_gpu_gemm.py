@@ -385,3 +385,26 @@ def test_in_launch_split_k_is_stable_over_many_back_to_back_calls(device):
         assert_close_f16(first, ref, "M=%d N=%d K=%d S=%d" % (M, N, K, S))
         stack = torch.stack(outs).view(torch.int16)
         assert bool((stack == stack[0]).all()), (M, N, K, layout, S)
+
+
+@pytest.mark.parametrize("layout", [KN, NK])
+def test_without_a_workspace_the_library_runs_unsplit(device, layout):
+    # the planner would split these shapes; with no workspace (or too small a one) the call must
+    # still give the right result, and a forced split must still be refused
+    from helpers import ptr, stream_ptr
+    L = capi.lib()
+    M, N, K = 8, 1024, 4096
+    assert layout == NK or capi.plan(M, N, K, layout, 0).splitk > 1
+    A, W = _case(M, N, K, layout, 610)
+    ref, _ = oracle.gemm_f16(A.numpy(), W.numpy(), layout)
+    Ad, Wd = A.to(device), W.to(device)
+    C = torch.full((M, N), float("nan"), dtype=torch.half, device=device)
+    assert L.fg_gemm_f16(ptr(Ad), ptr(Wd), ptr(C), M, N, K, layout, 0, 0, None, 0, stream_ptr()) == capi.FG_OK
+    torch.cuda.synchronize()
+    assert_close_f16(C.cpu().numpy(), ref, "no workspace")
+    small = torch.zeros(1024, dtype=torch.uint8, device=device)
+    C.fill_(float("nan"))
+    assert L.fg_gemm_f16(ptr(Ad), ptr(Wd), ptr(C), M, N, K, layout, 0, 0, ptr(small), small.numel(), stream_ptr()) == capi.FG_OK
+    torch.cuda.synchronize()
+    assert_close_f16(C.cpu().numpy(), ref, "workspace too small")
+    assert L.fg_gemm_f16(ptr(Ad), ptr(Wd), ptr(C), M, N, K, layout, 0, 4, None, 0, stream_ptr()) == capi.FG_ERR_WORKSPACE
