@@ -133,6 +133,22 @@ def main():
         y_val[0, n] = s / float(1 << 24)
     np.savez_compressed(HERE / "gemv_int8.npz", Wq=Wq, xq=xq, acc=acc.astype(np.int32), x=x.view(np.uint16),
                         y_expected=y_bits, y_exact=y_val)
+    # 6. int4 GEMV: two unsigned nibbles per byte, even element in the low nibble, zero point 8
+    K, N = 256, 128
+    Wq4 = rng.integers(0, 256, (N, K // 2)).astype(np.uint8)
+    x = rng.standard_normal((2, K)).astype(np.float16)
+    y_bits = np.zeros((2, N), np.uint16)
+    y_val = np.zeros((2, N), np.float64)
+    for m in range(2):
+        xi = [f16_to_int24(int(v)) for v in x.view(np.uint16)[m]]
+        for n in range(N):
+            s = 0
+            for b in range(K // 2):
+                byte = int(Wq4[n, b])
+                s += xi[2 * b] * ((byte & 15) - 8) + xi[2 * b + 1] * ((byte >> 4) - 8)  # units of 2^-24
+            y_bits[m, n] = round_f16(s, 24)
+            y_val[m, n] = s / float(1 << 24)
+    np.savez_compressed(HERE / "gemv_int4.npz", Wq4=Wq4, x=x.view(np.uint16), y_expected=y_bits, y_exact=y_val)
     print("wrote", sorted(p.name for p in HERE.glob("*.npz")))
 
 

@@ -265,3 +265,15 @@ def test_w4a16_pybind_and_errors(device):
     xd = x.to(device)
     assert L.fg_gemv_w4a16(ptr(W), ptr(xd), None, 1.0, 0.0, ptr(y), 5, N, K, stream_ptr()) == capi.FG_ERR_INVALID_ARG
     assert L.fg_gemv_w4a16(ptr(W), ptr(xd), None, 1.0, 0.0, ptr(y), 1, 100, K, stream_ptr()) == capi.FG_ERR_ALIGN128
+
+
+def test_w4a16_golden_vectors(device):
+    # exact-integer expected values (tests/golden/make_golden.py), two rows at once and one by one
+    from pathlib import Path
+    z = np.load(Path(__file__).resolve().parent / "golden" / "gemv_int4.npz")
+    Wq4 = torch.from_numpy(z["Wq4"])
+    x = torch.from_numpy(z["x"].view(np.float16).copy())
+    want = z["y_expected"].view(np.float16)
+    assert_close_f16(_w4a16(Wq4, x, None, 1.0, 8.0, device), want, "golden int4, M=2")
+    for m in range(2):
+        assert_close_f16(_w4a16(Wq4, x[m:m + 1].contiguous(), None, 1.0, 8.0, device), want[m:m + 1], "golden int4 row %d" % m)

@@ -120,6 +120,14 @@ def test_golden_int8():
     assert (oracle.fastgemv_int8(z["Wq"], x).view(np.uint16) == y.view(np.uint16).reshape(-1)).all()
 
 
+def test_golden_int4():
+    z = np.load(GOLD / "gemv_int4.npz")
+    x = z["x"].view(np.float16)
+    y, y32 = oracle.gemv_w4a16(z["Wq4"], x, None, 1.0, 8.0)
+    np.testing.assert_allclose(y32, z["y_exact"], rtol=2e-5, atol=1e-4)
+    assert _ulps(y.view(np.uint16), z["y_expected"]).max() <= 1
+
+
 # ---- closed forms and brute force ------------------------------------------------------------
 def test_ones_times_ones_is_K():
     for K in (128, 1024, 2048):
