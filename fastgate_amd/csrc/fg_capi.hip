@@ -82,13 +82,14 @@ int finish_plan(int M, int N, int K, fg_plan_t* p) {
         p->tile_n = 16;
       }
       if (p->tile_n % 16 != 0 && (p->splitk != 1 || p->waves != 8)) return FG_ERR_UNSUPPORTED;
-      p->m_block = 16;
+      p->m_block = p->m_block == 32 ? 32 : 16;  // 32: two row blocks per workgroup (128-byte bands)
       if (p->band == 0) {
         if (p->unroll != 1 && p->unroll != 2) return FG_ERR_UNSUPPORTED;
         p->band = 256 * p->unroll;
       }
       if (p->band != 128 && p->band != 256 && p->band != 512) return FG_ERR_UNSUPPORTED;
-      if ((p->tile_n > 32 || p->tile_n % 16 != 0) && p->band != 128) return FG_ERR_UNSUPPORTED;
+      if ((p->tile_n > 32 || p->tile_n % 16 != 0 || p->m_block == 32) && p->band != 128) return FG_ERR_UNSUPPORTED;
+      if (p->m_block == 32 && (p->tile_n % 16 != 0 || p->tile_n > 48)) return FG_ERR_UNSUPPORTED;
       p->unroll = p->band == 512 ? 2 : 1;
       break;
     case FG_KERNEL_NK_MFMA_T:
@@ -267,8 +268,17 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
       p->unroll = (K >= 16384 && N >= 8192) ? 2 : 1;
       items = ceil_div(K, 128 * p->unroll);
       row_tiles = true;
-      if (!wide_tiles && M <= 16 && splitk <= 1) {
-        const WideTile wt = pick_wide_tile(M, N, K, splitk);
+      if (M > 16) {
+        // 32 rows of A per workgroup (two MFMA row blocks on 128-byte bands): 17..32 rows read the
+        // weights once instead of twice
+        p->m_block = 32;
+        p->unroll = 1;
+        p->band = 128;
+        items = ceil_div(K, 64);
+      }
+      if (!wide_tiles && M <= 32 && splitk <= 1) {
+        WideTile wt = pick_wide_tile(M < 16 ? M : 16, N, K, splitk);
+        if (M > 16 && (wt.tile_n % 16 != 0 || wt.tile_n > 48)) wt = WideTile{};  // no ragged or 64-column form
         if (wt.tile_n) {
           p->tile_n = wt.tile_n;
           p->unroll = 1;

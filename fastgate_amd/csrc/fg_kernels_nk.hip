@@ -413,7 +413,8 @@ __global__ __launch_bounds__(64 * NW) void nk_mfma_r_kernel(const half_t* __rest
                                                         half_t* __restrict__ C,
                                                         float* __restrict__ ws, int* counters, int M,
                                                         int N, int K, int flags, const void* bias) {
-  // AROWS: rows of A staged per step (8 covers M <= 8, 16 covers M <= 16).  BAND: bytes of K per
+  // AROWS: rows of A staged per step (8 covers M <= 8, 16 covers M <= 16, 32 two MFMA row blocks per
+  // workgroup so that 17..32 rows still read the weights once).  BAND: bytes of K per
   // row and step (512, 256 or 128).  FULL: K is a multiple of the band and the bands divide evenly
   // over the waves -- no masks needed.  RAGGED: the tile is N / gridDim.x columns wide, fewer than
   // the 16 * CB the column blocks hold; the spare rows are never loaded and never stored.
@@ -426,8 +427,9 @@ __global__ __launch_bounds__(64 * NW) void nk_mfma_r_kernel(const half_t* __rest
   constexpr int RS = BAND + 16;        // LDS bytes per staged row
   constexpr int WSTRIP = 16 * CB * RS;  // weights of one wave
   constexpr int ASTRIP = AROWS * RS;   // activations of one wave (rows beyond AROWS re-read row j%8)
+  constexpr int MBLK = AROWS == 32 ? 2 : 1;  // 16-row MFMA blocks per workgroup
   constexpr int WAVE_LDS = WSTRIP + ASTRIP;
-  static_assert(WAVE_LDS >= CB * 256 * (int)sizeof(float), "reduction scratch fits");
+  static_assert(WAVE_LDS >= CB * MBLK * 256 * (int)sizeof(float), "reduction scratch fits");
   __shared__ __attribute__((aligned(16))) unsigned char smem[NW * WAVE_LDS];  // NW = most waves
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -436,7 +438,7 @@ __global__ __launch_bounds__(64 * NW) void nk_mfma_r_kernel(const half_t* __rest
   const int h = lane / LPR, c = lane % LPR;     // load order: row RPI*i + h, 16-byte piece c
   const int tw = RAGGED ? N / (int)gridDim.x : 16 * CB;  // columns of this tile
   const int n0 = blockIdx.x * tw;
-  const int m0 = blockIdx.y * 16;
+  const int m0 = blockIdx.y * (16 * MBLK);
   const int slots = nw * gridDim.z;
   const int slot = blockIdx.z * nw + wave;
   const int nbands = (K + BK - 1) / BK;  // K % 128 == 0: the last band may be partial
@@ -453,7 +455,7 @@ __global__ __launch_bounds__(64 * NW) void nk_mfma_r_kernel(const half_t* __rest
   // an 8-row A strip the MFMA rows 8..15 re-read rows 0..7; their results are never stored.
   const int st_off = h * RS + c * 16;
   const int ldw_off = j * RS + g * 16;
-  const int lda_off = (AROWS == 16 ? j : (j & 7)) * RS + g * 16;
+  const int lda_off = (AROWS >= 16 ? j : (j & 7)) * RS + g * 16;
 
   auto load_band = [&](int band, u32x4(&w)[WI], u32x4(&a)[AI]) {
     const bool ok = FULL || (band < nbands && (band * BK + c * 8) < K);
@@ -466,9 +468,11 @@ __global__ __launch_bounds__(64 * NW) void nk_mfma_r_kernel(const half_t* __rest
     for (int i = 0; i < AI; ++i)
       a[i] = (ok && arow[i]) ? load16<false>(Ap + (size_t)(RPI * i) * K + (size_t)band * BK) : zero;
   };
-  float4_t acc[CB];
+  float4_t acc[CB][MBLK];
 #pragma unroll
-  for (int b = 0; b < CB; ++b) acc[b] = float4_t{0.f, 0.f, 0.f, 0.f};
+  for (int b = 0; b < CB; ++b)
+#pragma unroll
+    for (int mb = 0; mb < MBLK; ++mb) acc[b][mb] = float4_t{0.f, 0.f, 0.f, 0.f};
   auto multiply = [&](const u32x4(&w)[WI], const u32x4(&a)[AI]) {
 #pragma unroll
     for (int i = 0; i < WI; ++i) *reinterpret_cast<u32x4*>(wstrip + st_off + RPI * i * RS) = w[i];
@@ -477,11 +481,16 @@ __global__ __launch_bounds__(64 * NW) void nk_mfma_r_kernel(const half_t* __rest
     wave_lds_sync();
 #pragma unroll
     for (int u = 0; u < UNITS; ++u) {
-      const u32x4 av = *reinterpret_cast<const u32x4*>(astrip + lda_off + u * 64);
+      u32x4 av[MBLK];
+#pragma unroll
+      for (int mb = 0; mb < MBLK; ++mb)
+        av[mb] = *reinterpret_cast<const u32x4*>(astrip + mb * 16 * RS + lda_off + u * 64);
 #pragma unroll
       for (int b = 0; b < CB; ++b) {
         const u32x4 bv = *reinterpret_cast<const u32x4*>(wstrip + b * 16 * RS + ldw_off + u * 64);
-        acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(av), as_half8(bv), acc[b], 0, 0, 0);
+#pragma unroll
+        for (int mb = 0; mb < MBLK; ++mb)
+          acc[b][mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(av[mb]), as_half8(bv), acc[b][mb], 0, 0, 0);
       }
     }
     wave_lds_sync();
@@ -505,16 +514,19 @@ __global__ __launch_bounds__(64 * NW) void nk_mfma_r_kernel(const half_t* __rest
     multiply(w1, a1);
   }
 
-  // acc[b][r] = D[m = 4g + r][column 16b + j]; the waves' partials meet in LDS
+  // acc[b][mb][r] = D[m = 16 mb + 4g + r][column 16b + j]; the waves' partials meet in LDS
   constexpr int TN = 16 * CB;
+  constexpr int TM = 16 * MBLK;
   __syncthreads();
-  float(*red)[16 * TN] = reinterpret_cast<float(*)[16 * TN]>(smem);
+  float(*red)[TM * TN] = reinterpret_cast<float(*)[TM * TN]>(smem);
 #pragma unroll
   for (int b = 0; b < CB; ++b)
 #pragma unroll
-    for (int r = 0; r < 4; ++r) red[wave][(4 * g + r) * TN + 16 * b + j] = acc[b][r];
+    for (int mb = 0; mb < MBLK; ++mb)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) red[wave][(16 * mb + 4 * g + r) * TN + 16 * b + j] = acc[b][mb][r];
   __syncthreads();
-  for (int e = threadIdx.x; e < 16 * TN; e += blockDim.x) {
+  for (int e = threadIdx.x; e < TM * TN; e += blockDim.x) {
     float sum = 0.f;
     for (int wv = 0; wv < nw; ++wv) sum += red[wv][e];
     const int mg = m0 + e / TN, n = n0 + e % TN;
@@ -527,7 +539,7 @@ __global__ __launch_bounds__(64 * NW) void nk_mfma_r_kernel(const half_t* __rest
       }
     }
   }
-  finish_splitk<16, TN>(ws, counters, C, M, N, m0, n0, flags, bias);
+  finish_splitk<TM, TN>(ws, counters, C, M, N, m0, n0, flags, bias);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -749,6 +761,11 @@ static void nk_mfma_r_go(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
 
 template <int CB>
 static bool nk_mfma_r_cb(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
+  if (p.m_block == 32) {  // two 16-row blocks per workgroup, 128-byte bands
+    if (p.band != 128) return false;
+    nk_mfma_r_go<32, 128, CB>(p, a, s);
+    return true;
+  }
   const bool half_m = a.M <= 8;  // one block row whose A strip needs only 8 rows
   switch (p.band) {
     case 128:
@@ -772,7 +789,8 @@ static bool nk_mfma_r_cb(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
 // 256 or 128 (four or eight rows per instruction, up to eight waves).  tile_n = 16, 32, 48 or 64
 // (one to four 16-column blocks sharing the staged activations; 48 and 64 on 128-byte bands only).
 bool launch_nk_mfma_r(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
-  if (p.m_block != 16) return false;
+  if (p.m_block != 16 && p.m_block != 32) return false;
+  if (p.m_block == 32 && (p.tile_n % 16 != 0 || p.tile_n > 48)) return false;
   if (p.waves > 4 && !(p.waves == 8 && p.band <= 256)) return false;
   if (p.tile_n == 16) return nk_mfma_r_cb<1>(p, a, s);
   if (p.tile_n == 32) return nk_mfma_r_cb<2>(p, a, s);
@@ -793,6 +811,10 @@ bool launch_nk_mfma_r(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
   if (p.tile_n == 48 || p.tile_n == 64) {  // three or four column blocks: 128-byte bands only
     if (p.band != 128) return false;
     const bool half_m = a.M <= 8;
+    if (p.m_block == 32) {
+      nk_mfma_r_go<32, 128, 3>(p, a, s);
+      return true;
+    }
     if (p.tile_n == 48) {
       if (half_m) nk_mfma_r_go<8, 128, 3>(p, a, s);
       else nk_mfma_r_go<16, 128, 3>(p, a, s);

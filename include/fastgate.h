@@ -17,7 +17,8 @@
  *   W      fp16 weights, w_layout FG_W_KN = [K,N] row-major, FG_W_NK = [N,K] row-major
  *   C      fp16 [M,N] row-major, caller allocated
  *   K, N   multiples of 128 (the reference's only documented constraint, README.md:6-12)
- *   M      any positive value; the kernels are meant for M = 1..16
+ *   M      any positive value; the kernels are meant for M = 1..16 (one pass over the weights up
+ *          to 32 rows with [N,K] weights, one more pass per further 32 / 16 rows)
  *   arithmetic: fp16 products, fp32 accumulation, one rounding to fp16 at the end
  */
 #ifndef FASTGATE_H_

@@ -408,3 +408,40 @@ def test_without_a_workspace_the_library_runs_unsplit(device, layout):
     torch.cuda.synchronize()
     assert_close_f16(C.cpu().numpy(), ref, "workspace too small")
     assert L.fg_gemm_f16(ptr(Ad), ptr(Wd), ptr(C), M, N, K, layout, 0, 4, None, 0, stream_ptr()) == capi.FG_ERR_WORKSPACE
+
+
+@pytest.mark.parametrize("tile", [16, 32, 48])
+@pytest.mark.parametrize("waves", [2, 4, 8])
+@pytest.mark.parametrize("splitk,fused", [(1, 0), (2, 0), (3, 1)])
+def test_row_load_mfma_kernel_with_32_row_blocks(device, tile, waves, splitk, fused):
+    # two MFMA row blocks per workgroup: 17..32 rows read the weights once; more rows add block rows
+    N = 768 if tile == 48 else 384
+    for K in (128, 384, 2048, 4480):
+        for M in (17, 24, 31, 32, 33, 47, 64):
+            A, W = _case(M, N, K, NK, 110 + M + K)
+            ref, _ = oracle.gemm_f16(A.numpy(), W.numpy(), NK)
+            kw = dict(kernel=capi.FG_KERNEL_NK_MFMA_R, tile_n=tile, m_block=32, waves=waves, splitk=splitk, fused=fused, band=128)
+            got, p = _run(A, W, NK, device, plan=make_plan(**kw))
+            assert p.m_block == 32 and p.grid_y == -(-M // 32) and p.tile_n == tile
+            assert_close_f16(got, ref, "mfma_r 32-row blocks tile %d M=%d K=%d" % (tile, M, K))
+    g = gen(111)
+    A = torch.randint(-2, 3, (32, 768), generator=g).half()
+    W = torch.randint(-3, 4, (N, 768), generator=g).half()
+    ref, _ = oracle.gemm_f16(A.numpy(), W.numpy(), NK)
+    got, _ = _run(A, W, NK, device, plan=make_plan(kernel=capi.FG_KERNEL_NK_MFMA_R, tile_n=tile, m_block=32, waves=waves, splitk=splitk, fused=fused, band=128))
+    assert (got == ref).all()
+    C0 = normal((32, N), gen(112), 2.0)
+    refa, _ = oracle.gemm_f16(A.numpy(), W.numpy(), NK, C=C0.numpy(), accumulate=True)
+    got, _ = _run(A, W, NK, device, accumulate=True, C0=C0, plan=make_plan(kernel=capi.FG_KERNEL_NK_MFMA_R, tile_n=tile, m_block=32, waves=waves, splitk=splitk, fused=fused, band=128))
+    assert_close_f16(got, refa, "32-row blocks, accumulate")
+
+
+@pytest.mark.parametrize("M", [17, 32, 40])
+def test_planner_uses_32_row_blocks_beyond_16_rows(device, M):
+    for (N, K) in ((1024, 2048), (8192, 256), (12288, 384)):
+        p = capi.plan(M, N, K, NK, 0)
+        assert p.kernel == capi.FG_KERNEL_NK_MFMA_R and p.m_block == 32 and p.band == 128, p.as_dict()
+        A, W = _case(M, N, K, NK, 120 + M)
+        ref, _ = oracle.gemm_f16(A.numpy(), W.numpy(), NK)
+        got, _ = _run(A, W, NK, device)
+        assert_close_f16(got, ref, "auto plan M=%d N=%d K=%d" % (M, N, K))

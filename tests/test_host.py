@@ -63,7 +63,7 @@ def test_plan_is_consistent(layout, M, N, K):
     if M <= 2 and N * K < 1 << 28:
         assert p.kernel in (capi.FG_KERNEL_KN_DOT2, capi.FG_KERNEL_NK_DOT2), d
     if p.kernel == capi.FG_KERNEL_NK_MFMA_R:
-        assert p.tile_n in (16, 32, 48) and p.m_block == 16, d
+        assert p.tile_n in (16, 32, 48) and p.m_block == (32 if M > 16 else 16), d
     if p.kernel == capi.FG_KERNEL_NK_MFMA_T:
         assert p.splitk == -(-(K // 32) // 64) and p.waves == 4 and p.tile_n % p.unroll == 0, d
     # a forced split is honoured
@@ -263,5 +263,8 @@ def test_eed_backend_reexports_every_operator(sg):
 def test_row_count_beyond_the_grid_limit_is_rejected():
     import ctypes
     p = capi.Plan()
-    assert capi.lib().fg_plan(16 * 65535 + 1, 128, 128, capi.FG_W_NK, 0, ctypes.byref(p)) == capi.FG_ERR_INVALID_ARG
-    assert capi.lib().fg_plan(16 * 65535, 128, 128, capi.FG_W_NK, 0, ctypes.byref(p)) == capi.FG_OK
+    # [N,K] weights: 32 rows per block row beyond 16 rows; [K,N]: 16
+    assert capi.lib().fg_plan(32 * 65535 + 1, 128, 128, capi.FG_W_NK, 0, ctypes.byref(p)) == capi.FG_ERR_INVALID_ARG
+    assert capi.lib().fg_plan(32 * 65535, 128, 128, capi.FG_W_NK, 0, ctypes.byref(p)) == capi.FG_OK
+    assert capi.lib().fg_plan(16 * 65535 + 1, 128, 128, capi.FG_W_KN, 0, ctypes.byref(p)) == capi.FG_ERR_INVALID_ARG
+    assert capi.lib().fg_plan(16 * 65535, 128, 128, capi.FG_W_KN, 0, ctypes.byref(p)) == capi.FG_OK
