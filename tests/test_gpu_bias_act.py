@@ -69,7 +69,7 @@ def test_every_kernel_family(device, name, layout, kw, splitk, fused):
 
 
 @pytest.mark.parametrize("layout", [KN, NK])
-@pytest.mark.parametrize("M", [1, 2, 4, 8, 16])
+@pytest.mark.parametrize("M", [1, 2, 4, 8, 16, 24])
 def test_library_plans_at_ffn_shapes(device, layout, M):
     # scaled-down feed-forward pair (K:N = 1:4 and 4:1): the planner's own choices
     for K, N in ((768, 3072), (3072, 768)):
