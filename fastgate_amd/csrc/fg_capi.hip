@@ -575,7 +575,7 @@ int fg_gemm_f16_bias_act(const void* A, const void* W, const void* bias, int act
 int fg_gemv_w8a16(const void* Wq, const void* x, const void* scale, float scalar_scale,
                   float zero_point, void* y, int M, int N, int K, void* stream) {
   if (Wq == nullptr || x == nullptr || y == nullptr) return FG_ERR_INVALID_ARG;
-  if (M <= 0 || M > 8 || N <= 0 || K <= 0) return FG_ERR_INVALID_ARG;
+  if (M <= 0 || M > 16 || N <= 0 || K <= 0) return FG_ERR_INVALID_ARG;
   if (N % 128 != 0 || K % 128 != 0) return FG_ERR_ALIGN128;
   if ((reinterpret_cast<uintptr_t>(Wq) | reinterpret_cast<uintptr_t>(x)) & 15) {
     return FG_ERR_INVALID_ARG;

@@ -126,142 +126,6 @@ __global__ __launch_bounds__(512) void w8a16_kernel(const int8_t* __restrict__ W
   }
 }
 
-// ---------------------------------------------------------------------------------------
-// w8a16 for M <= 4 on v_mfma_f32_4x4x4_16B_f16.  Block b = lane/4 owns 16 k positions of a
-// 256-wide K chunk, its four lanes j own four neighbouring weight rows: one load instruction
-// reads 4 rows x 256 contiguous bytes, and the activation fragment of a block (row m = j, the
-// same 16 k, 32 bytes) is fetched once per chunk and reused for all R4 row quads -- an eighth
-// of the activation traffic of the lanes-along-K kernel above, and the 8 v_dot2 per 16 weights
-// move to the matrix pipe, leaving the VALU to the int8 -> fp16 conversion.
-// acc[r][i] at lane (b,j) is the partial y[m=i][n0 + 4r + j] over block b's k positions.
-// ---------------------------------------------------------------------------------------
-typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
-
-__device__ __forceinline__ half4_t i8x4_to_half4(uint32_t w) {
-  half2_t lo, hi;
-  i8x4_to_half2x2(w, lo, hi);
-  return half4_t{lo[0], lo[1], hi[0], hi[1]};
-}
-__device__ __forceinline__ half4_t pair_half4(uint32_t a, uint32_t b) {
-  return __builtin_bit_cast(half4_t, u32x2{a, b});
-}
-
-template <int MG, int R4, int U>
-__global__ __launch_bounds__(256) void w8a16_mfma_kernel(const int8_t* __restrict__ Wq,
-                                                         const half_t* __restrict__ X,
-                                                         const half_t* __restrict__ scale,
-                                                         float scalar_scale, float zero_point,
-                                                         half_t* __restrict__ Y, int M, int N, int K) {
-  __shared__ float red[16][R4 * MG * 16];
-  __shared__ float redx[16][MG * 4];
-  const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
-  const int nw = blockDim.x >> 6;
-  const int j = lane & 3, b = lane >> 2;
-  const int n0 = blockIdx.x * (4 * R4);
-  const int nchunks = (K + 255) >> 8;  // K % 128 == 0: the last chunk may be half
-  const bool use_zp = zero_point != 0.f;
-
-  float4_t acc[R4][MG];
-  float4_t xacc[MG];
-#pragma unroll
-  for (int g = 0; g < MG; ++g) {
-    xacc[g] = float4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int r = 0; r < R4; ++r) acc[r][g] = float4_t{0.f, 0.f, 0.f, 0.f};
-  }
-  const half4_t ones = {static_cast<half_t>(1.f), static_cast<half_t>(1.f), static_cast<half_t>(1.f),
-                        static_cast<half_t>(1.f)};
-  const u32x4 zero = {0u, 0u, 0u, 0u};
-  const int8_t* Wp = Wq + (size_t)(n0 + j) * K + b * 16;
-  const half_t* Xp = X + (size_t)j * K + b * 16;
-
-  const int nsteps = (nchunks + nw * U - 1) / (nw * U);
-  int step = stagger_start(nsteps, 0);
-  for (int it = 0; it < nsteps; ++it) {
-    const int c0 = (step * nw + wave) * U;
-    step = step + 1 == nsteps ? 0 : step + 1;
-    u32x4 w[U][R4];
-    u32x4 x[U][MG][2];
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int c = c0 + u;
-      const bool ok = c * 256 + b * 16 < K;
-#pragma unroll
-      for (int r = 0; r < R4; ++r)
-        w[u][r] = ok ? load16<true>(Wp + (size_t)(4 * r) * K + (size_t)c * 256) : zero;
-#pragma unroll
-      for (int g = 0; g < MG; ++g) {
-        const bool okx = ok && (4 * g + j) < M;
-        const half_t* xp = Xp + (size_t)(4 * g) * K + (size_t)c * 256;
-        x[u][g][0] = okx ? load16<false>(xp) : zero;
-        x[u][g][1] = okx ? load16<false>(xp + 8) : zero;
-      }
-    }
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      half4_t xq[MG][4];
-#pragma unroll
-      for (int g = 0; g < MG; ++g) {
-        xq[g][0] = pair_half4(x[u][g][0].x, x[u][g][0].y);
-        xq[g][1] = pair_half4(x[u][g][0].z, x[u][g][0].w);
-        xq[g][2] = pair_half4(x[u][g][1].x, x[u][g][1].y);
-        xq[g][3] = pair_half4(x[u][g][1].z, x[u][g][1].w);
-      }
-#pragma unroll
-      for (int r = 0; r < R4; ++r)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const half4_t wq = i8x4_to_half4(w[u][r][q]);
-#pragma unroll
-          for (int g = 0; g < MG; ++g)
-            acc[r][g] = __builtin_amdgcn_mfma_f32_4x4x4f16(xq[g][q], wq, acc[r][g], 0, 0, 0);
-        }
-      if (use_zp) {
-#pragma unroll
-        for (int g = 0; g < MG; ++g)
-#pragma unroll
-          for (int q = 0; q < 4; ++q)
-            xacc[g] = __builtin_amdgcn_mfma_f32_4x4x4f16(xq[g][q], ones, xacc[g], 0, 0, 0);
-      }
-    }
-  }
-
-  // Sum the 16 blocks: 4 per DPP row with row_ror:4 / row_ror:8, the 4 rows and the waves in LDS.
-#pragma unroll
-  for (int g = 0; g < MG; ++g)
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-#pragma unroll
-      for (int r = 0; r < R4; ++r) {
-        float v = acc[r][g][i];
-        v += dpp_f32<0x124>(v);
-        v += dpp_f32<0x128>(v);
-        if ((lane & 12) == 0) red[wave * 4 + (lane >> 4)][((r * MG + g) * 4 + i) * 4 + j] = v;
-      }
-      float xs = xacc[g][i];
-      xs += dpp_f32<0x124>(xs);
-      xs += dpp_f32<0x128>(xs);
-      if ((lane & 15) == 0) redx[wave * 4 + (lane >> 4)][g * 4 + i] = xs;
-    }
-  __syncthreads();
-  for (int e = threadIdx.x; e < R4 * MG * 16; e += blockDim.x) {
-    // e = m * (4*R4) + r*4 + jj : consecutive threads write consecutive columns
-    const int jj = e & 3, r = (e >> 2) % R4, m = (e >> 2) / R4, g = m >> 2, i = m & 3;
-    float sum = 0.f, xs = 0.f;
-    for (int p = 0; p < nw * 4; ++p) {
-      sum += red[p][((r * MG + g) * 4 + i) * 4 + jj];
-      xs += redx[p][m];
-    }
-    const int n = n0 + 4 * r + jj;
-    if (m < M) {
-      float sc = scalar_scale;
-      if (scale != nullptr) sc *= static_cast<float>(scale[n]);
-      Y[(size_t)m * N + n] = static_cast<half_t>((sum - zero_point * xs) * sc);
-    }
-  }
-}
-
 template <int MB, int RN, int U>
 __global__ __launch_bounds__(256) void i8i8_kernel(const int8_t* __restrict__ Wq,
                                                    const int8_t* __restrict__ Xq,
@@ -473,7 +337,7 @@ __global__ __launch_bounds__(256) void w4a16_kernel(const uint8_t* __restrict__ 
 // of one weight row per lane, converted to 8 fp16 there, against 16 bytes of one activation row.
 // The activations are fetched once per 16 weight rows instead of once per 4, the dot products run
 // on the matrix pipe, and the VALU only converts.  16-column tiles, 8 waves interleaving over K.
-// XROWS = activation rows staged (2 covers M <= 2, 8 covers M <= 8).
+// XROWS = activation rows staged: 4, 8 or 16.
 // ---------------------------------------------------------------------------------------
 template <int XROWS, int NW, int BW, int CB>
 __global__ __launch_bounds__(64 * NW) void w8a16_r_kernel(const int8_t* __restrict__ Wq,
@@ -740,45 +604,47 @@ static int i8_waves(int K) {
   return pieces >= 4 ? 4 : (pieces >= 2 ? 2 : 1);
 }
 
-// Measured (us per call; lanes-along-K kernel / 4x4x4 MFMA kernel / row-load kernel):
-//   K = N = 8192   M=1 12.6 / 13.5 / 14.3   M=2 15.1 / 13.9 / 14.2   M=4 21.1 / 15.4 / 14.9   M=8 32.9 / 20.7 / 17.2
-//   K = N = 16384  M=1 41.2 /  -   / 44.8   M=2  -   / 50.2 / 45.8   M=4  -   / 52.7 / 47.8   M=8  -   / 66.9 / 49.7
-// (16-column tiles on 256-byte bands).  The row-load kernel exists with 8 waves only.
+// Measured (us per call; lanes-along-K kernel / row-load kernel on 256-byte bands):
+//   K = N = 8192   M=1 12.6 / 14.3   M=2 15.1 / 14.2   M=4 21.1 / 14.9   M=8 32.9 / 17.2
+//   K = N = 16384  M=1 41.2 / 44.8   M=8  -   / 49.7
+// The row-load kernel exists with 8 waves only.
 bool launch_w8a16(const W8A16Args& a, hipStream_t s) {
   auto* Wq = static_cast<const int8_t*>(a.Wq);
   auto* X = static_cast<const half_t*>(a.x);
   auto* sc = static_cast<const half_t*>(a.scale);
   auto* Y = static_cast<half_t*>(a.y);
+  const int t32 = a.N / 32;
+  // 32-column tiles on 128-byte bands read half the activation bytes per weight byte.  They pay
+  // where N/32 workgroups still put two workgroups (16 waves) on every CU -- K = N = 16384, M=8:
+  // 44.8 us against 49.3; K=4096 N=16384: 14.9 / 17.3 -- and lose where they leave one (K = N =
+  // 8192, M=8: 17.2 / 16.6: the conversion wants the waves).
+  const bool wide = a.N % 32 == 0 && t32 >= 512 && t32 % 512 == 0;
+  // 16-column tiles: 128-byte bands (smaller strips, more steps in flight) except for long rows
+  // with at most one workgroup per CU -- M=8, 128- / 256-byte bands: K = N = 8192 14.5 / 15.7,
+  // K = N = 4096 7.0 / 7.3, K=4096 N=14336 14.6 / 16.1, K=14336 N=4096 15.9 / 15.6.
+  const bool bw256 = a.N / 16 < 512 && a.K > 8192;
+#define FG_W8A16_R(XR, BW, CB)                                                                    \
+  hipLaunchKernelGGL((w8a16_r_kernel<XR, 8, BW, CB>), dim3(a.N / (16 * CB)), dim3(512), 0, s, Wq, \
+                     X, sc, a.scalar_scale, a.zero_point, Y, a.M, a.N, a.K)
   if (a.M == 1) {  // 4 rows per workgroup, one load group in flight
     hipLaunchKernelGGL((w8a16_kernel<1, 4, 1>), dim3(a.N / 4), dim3(64 * i8_waves(a.K)), 0, s, Wq, X,
                        sc, a.scalar_scale, a.zero_point, Y, a.M, a.N, a.K);
-  } else if (a.M <= 3 && (size_t)a.N * a.K <= ((size_t)1 << 27)) {
-    hipLaunchKernelGGL((w8a16_mfma_kernel<1, 4, 2>), dim3(a.N / 16), dim3(256), 0, s, Wq, X, sc,
-                       a.scalar_scale, a.zero_point, Y, a.M, a.N, a.K);
-  } else if (a.M <= 2) {
-    hipLaunchKernelGGL((w8a16_r_kernel<2, 8, 256, 1>), dim3(a.N / 16), dim3(512), 0, s, Wq, X, sc,
-                       a.scalar_scale, a.zero_point, Y, a.M, a.N, a.K);
+  } else if (a.M <= 4) {  // 2 rows take the 4-row strip too: K=14336 N=4096 M=2 13.1 us
+    if (wide) FG_W8A16_R(4, 128, 2);
+    else if (bw256) FG_W8A16_R(4, 256, 1);
+    else FG_W8A16_R(4, 128, 1);
   } else if (a.M <= 8) {
-    // 32-column tiles on 128-byte bands read half the activation bytes per weight byte.  They pay
-    // where N/32 workgroups still put two workgroups (16 waves) on every CU -- K = N = 16384, M=8:
-    // 44.8 us against 49.3; K=4096 N=16384: 14.9 / 17.3 -- and lose where they leave one (K = N =
-    // 8192, M=8: 17.2 / 16.6: the conversion wants the waves).
-    const int t32 = a.N / 32;
-    const bool wide = a.N % 32 == 0 && t32 >= 512 && t32 % 512 == 0;
-    if (wide) {
-      if (a.M <= 4)
-        hipLaunchKernelGGL((w8a16_r_kernel<4, 8, 128, 2>), dim3(t32), dim3(512), 0, s, Wq, X, sc,
-                           a.scalar_scale, a.zero_point, Y, a.M, a.N, a.K);
-      else
-        hipLaunchKernelGGL((w8a16_r_kernel<8, 8, 128, 2>), dim3(t32), dim3(512), 0, s, Wq, X, sc,
-                           a.scalar_scale, a.zero_point, Y, a.M, a.N, a.K);
-    } else {
-      hipLaunchKernelGGL((w8a16_r_kernel<8, 8, 256, 1>), dim3(a.N / 16), dim3(512), 0, s, Wq, X, sc,
-                         a.scalar_scale, a.zero_point, Y, a.M, a.N, a.K);
-    }
+    if (wide) FG_W8A16_R(8, 128, 2);
+    else if (bw256) FG_W8A16_R(8, 256, 1);
+    else FG_W8A16_R(8, 128, 1);
+  } else if (a.M <= 16) {
+    // 16-row activation strip on 128-byte bands only (the 256-byte form would need 100 KB of LDS)
+    if (wide) FG_W8A16_R(16, 128, 2);
+    else FG_W8A16_R(16, 128, 1);
   } else {
     return false;
   }
+#undef FG_W8A16_R
   return true;
 }
 

@@ -251,7 +251,7 @@ void fastgemv_int8(at::Tensor mat, at::Tensor vec, at::Tensor res, c10::optional
               " elements");
   const int64_t M = vec.numel() / K;
   TORCH_CHECK(M <= INT32_MAX && N <= INT32_MAX && K <= INT32_MAX, op, ": size overflow");
-  TORCH_CHECK(M <= 8, op, ": at most 8 activation rows");
+  TORCH_CHECK(M <= 16, op, ": at most 16 activation rows");
   TORCH_CHECK(res.numel() == M * N, op, ": res must hold M*N = ", M * N, " elements");
   const void* sp = nullptr;
   if (scale.has_value() && scale->defined()) {

@@ -26,7 +26,7 @@ def _w8a16(Wq, x, scale, scalar_scale, zp, device):
     return y.cpu().numpy()
 
 
-@pytest.mark.parametrize("M", [1, 2, 3, 4, 5, 8])
+@pytest.mark.parametrize("M", [1, 2, 3, 4, 5, 8, 9, 13, 16])
 @pytest.mark.parametrize("N,K", [(128, 128), (256, 1152), (1024, 4096), (4096, 1024)])
 def test_w8a16_matches_oracle(device, M, N, K):
     g = gen(4000 + M + N)
@@ -43,10 +43,10 @@ def test_w8a16_matches_oracle(device, M, N, K):
     assert_close_f16(_w8a16(Wq, x, scale, 0.5, 3.0, device), ref, "scale 0.5 zp 3")
 
 
-@pytest.mark.parametrize("M", [3, 4, 5, 7, 8])
+@pytest.mark.parametrize("M", [3, 4, 5, 7, 8, 9, 12, 16])
 @pytest.mark.parametrize("N,K", [(16384, 128), (16384, 384), (16384, 1152), (32768, 384)])
 def test_w8a16_wide_tiles_for_wide_outputs(device, M, N, K):
-    # N / 32 a multiple of 512: 32-column tiles on 128-byte bands, 4- or 8-row activation
+    # N / 32 a multiple of 512: 32-column tiles on 128-byte bands, 4-, 8- or 16-row activation
     # strips; exact small integers first (any LDS layout mistake changes the bits), then random data
     g = gen(4100 + M + N + K)
     xi = torch.randint(-3, 4, (M, K), generator=g).half()
@@ -62,10 +62,27 @@ def test_w8a16_wide_tiles_for_wide_outputs(device, M, N, K):
     assert_close_f16(_w8a16(Wq, x, scale, 0.5, 3.0, device), ref, "scale 0.5 zp 3")
 
 
+@pytest.mark.parametrize("M", [9, 11, 16])
+@pytest.mark.parametrize("N,K", [(1024, 128), (2048, 640), (8192, 1152)])
+def test_w8a16_16_row_strip_is_exact_on_small_integers(device, M, N, K):
+    # 9..16 activation rows: 16-row strip, 16-column tiles.  Integer data whose sums fp16 holds
+    # exactly: a wrong row, band or byte in the staged strips changes the bits
+    g = gen(4150 + M + N + K)
+    xi = torch.randint(-3, 4, (M, K), generator=g).half()
+    Wsmall = torch.randint(-8, 9, (N, K), generator=g, dtype=torch.int8)
+    ref, _ = oracle.gemv_w8a16(Wsmall.numpy(), xi.numpy(), None, 1.0, 0.0)
+    got = _w8a16(Wsmall, xi, None, 1.0, 0.0, device)
+    exact = np.abs(ref.astype(np.float32)) <= 2048
+    assert (got[exact] == ref[exact]).all() and exact.mean() > 0.9
+    # each row alone gives the same bits as within the batch
+    one = _w8a16(Wsmall, xi[M - 1:M].contiguous(), None, 1.0, 0.0, device)
+    assert (one[0] == got[M - 1]).all()
+
+
 @pytest.mark.parametrize("M", [2, 3])
-def test_w8a16_large_weights_take_the_row_load_kernel(device, M):
-    # above 2^27 weights M = 2..3 switches to the LDS-staged kernel (2-row and 8-row activation
-    # strips); the oracle checks a band of output channels
+def test_w8a16_large_weights_with_a_ragged_last_band(device, M):
+    # K = 65 bands of 128: the last 256-byte band of a row is half empty; the oracle checks
+    # three windows of output channels
     N, K = 16384, 8192 + 128
     g = gen(880 + M)
     x = normal((M, K), g, 1.0)
@@ -158,7 +175,7 @@ def test_int8_error_codes(device):
     W = torch.zeros((128, 128), dtype=torch.int8, device=device)
     x = torch.zeros((1, 128), dtype=torch.half, device=device)
     y = torch.zeros((1, 128), dtype=torch.half, device=device)
-    assert L.fg_gemv_w8a16(ptr(W), ptr(x), None, 1.0, 0.0, ptr(y), 9, 128, 128, stream_ptr()) == capi.FG_ERR_INVALID_ARG
+    assert L.fg_gemv_w8a16(ptr(W), ptr(x), None, 1.0, 0.0, ptr(y), 17, 128, 128, stream_ptr()) == capi.FG_ERR_INVALID_ARG
     assert L.fg_gemv_w8a16(ptr(W), ptr(x), None, 1.0, 0.0, ptr(y), 1, 100, 128, stream_ptr()) == capi.FG_ERR_ALIGN128
     assert L.fg_gemv_w8a16(None, ptr(x), None, 1.0, 0.0, ptr(y), 1, 128, 128, stream_ptr()) == capi.FG_ERR_INVALID_ARG
 
