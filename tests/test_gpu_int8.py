@@ -62,6 +62,25 @@ def test_w8a16_wide_tiles_for_wide_outputs(device, M, N, K):
     assert_close_f16(_w8a16(Wq, x, scale, 0.5, 3.0, device), ref, "scale 0.5 zp 3")
 
 
+@pytest.mark.parametrize("M", [2, 4, 5, 8])
+def test_w8a16_long_rows_with_few_tiles_use_256_byte_bands(device, M):
+    # fewer than 512 tiles and K > 8192: 256-byte bands (4- and 8-row strips); K = 65 bands of
+    # 128 leaves the last 256-byte band half empty.  Exact integers first, then random data
+    N, K = 2048, 8192 + 128
+    g = gen(4170 + M)
+    xi = torch.randint(-1, 2, (M, K), generator=g).half()
+    Wsmall = torch.randint(-2, 3, (N, K), generator=g, dtype=torch.int8)
+    ref, _ = oracle.gemv_w8a16(Wsmall.numpy(), xi.numpy(), None, 1.0, 0.0)
+    got = _w8a16(Wsmall, xi, None, 1.0, 0.0, device)
+    assert np.abs(ref.astype(np.float32)).max() <= 2048
+    assert (got == ref).all()
+    Wq = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8)
+    x = normal((M, K), g)
+    scale = (torch.rand(N, generator=g) * 0.009 + 0.001).half()
+    ref, _ = oracle.gemv_w8a16(Wq.numpy(), x.numpy(), scale.numpy(), 0.5, 3.0)
+    assert_close_f16(_w8a16(Wq, x, scale, 0.5, 3.0, device), ref, "scale 0.5 zp 3")
+
+
 @pytest.mark.parametrize("M", [9, 11, 16])
 @pytest.mark.parametrize("N,K", [(1024, 128), (2048, 640), (8192, 1152)])
 def test_w8a16_16_row_strip_is_exact_on_small_integers(device, M, N, K):

@@ -101,6 +101,23 @@ def test_fastgemv_int8_defaults_and_extension(device, sg):
     assert_close_f16(y.cpu().numpy(), ref.reshape(-1), "per-channel scale")
 
 
+def test_fastgemv_int8_takes_up_to_16_activation_rows(device, sg):
+    g = gen(1014)
+    N, K = 1024, 1152
+    Wq = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8)
+    scale = (torch.rand(N, generator=g) * 0.009 + 0.001).half()
+    for M in (2, 7, 16):
+        x = normal((M, K), g)
+        y = torch.full((M, N), float("nan"), dtype=torch.half, device=device)
+        sg.fastgemv_int8(Wq.to(device), x.to(device), y, scale=scale.to(device))
+        ref, _ = oracle.gemv_w8a16(Wq.numpy(), x.numpy(), scale.numpy())
+        assert_close_f16(y.cpu().numpy(), ref, "M=%d" % M)
+    x = normal((17, K), g)
+    y = torch.empty((17, N), dtype=torch.half, device=device)
+    with pytest.raises(RuntimeError, match="at most 16 activation rows"):
+        sg.fastgemv_int8(Wq.to(device), x.to(device), y)
+
+
 def test_integer_ops(device, sg):
     g = gen(1005)
     N, K = 512, 1024
