@@ -172,6 +172,22 @@ def run_sweep(torch, sg, capi, dev, steps, warmup, models=False):
                  "weights_per_ns": round(Kk * Nn / us_i8 / 1e3, 3),
                  "fp16_M1_weights_per_ns": round(Kk * Nn / us_f16 / 1e3, 3),
                  "weight_throughput_vs_fp16": round(us_f16 / us_i8, 3)})
+    # beyond the benchmark's configurations: the int8 GEMV with 4, 8 and 16 activation rows
+    for Mb in (4, 8, 16):
+        xb = torch.randn((Mb, Kk), device=dev, generator=g).half()
+        yb = torch.empty((Mb, Nn), dtype=torch.half, device=dev)
+        us_b = time_us(lambda i: sg.fastgemv_int8(wq[i % 10], xb, yb, scale=scale))
+        us_fb = next(r["us_per_call"] for r in rows if r["config"] == "C5 sweep" and r["M"] == Mb
+                     and r["K"] == 8192 and r["w_layout"] == "[N,K]")
+        by = Kk * Nn + 2 * Mb * Kk + 2 * Mb * Nn + 2 * Nn
+        rows.append({"config": "extra: int8 batched", "op": "fastgemv_int8", "M": Mb, "K": Kk, "N": Nn,
+                     "w_layout": "[N,K] int8", "seed": 1004, "kernel": "w8a16_r", "splitk": 1, "bytes": by,
+                     "us_per_call": round(us_b, 2), "GBps": round(by / us_b / 1e3, 1),
+                     "frac_hbm_peak": round(by / us_b / 1e3 / HBM_PEAK_GBPS, 4),
+                     "frac_read_ceiling": round(by / us_b / 1e3 / ceiling, 4),
+                     "weights_per_ns": round(Kk * Nn / us_b / 1e3, 3),
+                     "fp16_M1_weights_per_ns": round(Kk * Nn / us_fb / 1e3, 3),
+                     "weight_throughput_vs_fp16": round(us_fb / us_b, 3)})
     # beyond the benchmark's configurations: the same GEMV with 4-bit weights (two per byte)
     del wq
     wq4 = [torch.randint(0, 256, (Nn, Kk // 2), device=dev, generator=g, dtype=torch.uint8) for _ in range(20)]
