@@ -618,7 +618,12 @@ bool launch_w8a16(const W8A16Args& a, hipStream_t s) {
   // where N/32 workgroups still put two workgroups (16 waves) on every CU -- K = N = 16384, M=8:
   // 44.8 us against 49.3; K=4096 N=16384: 14.9 / 17.3 -- and lose where they leave one (K = N =
   // 8192, M=8: 17.2 / 16.6: the conversion wants the waves).
-  const bool wide = a.N % 32 == 0 && t32 >= 512 && t32 % 512 == 0;
+  // With exactly one such workgroup per CU (N = 8192) they pay for long rows or many activation
+  // rows: K=16384 M=8 27.3 -> 25.4 us, K=28672 M=14 55.4 -> 47.8, K=4096 M=16 11.1 -> 10.5, against
+  // K=8192 M=8 14.9 -> 16.9, K=28672 M=4 38.7 -> 40.0.
+  const bool one_per_cu = a.N % 32 == 0 && t32 == 256 &&
+                          (a.M >= 15 || (a.K >= 16384 && (a.M >= 5 || a.K < 24576)));
+  const bool wide = (a.N % 32 == 0 && t32 >= 512 && t32 % 512 == 0) || one_per_cu;
   // 16-column tiles: 128-byte bands (smaller strips, more steps in flight) except for long rows
   // with at most one workgroup per CU -- M=8, 128- / 256-byte bands: K = N = 8192 14.5 / 15.7,
   // K = N = 4096 7.0 / 7.3, K=4096 N=14336 14.6 / 16.1, K=14336 N=4096 15.9 / 15.6.

@@ -62,6 +62,27 @@ def test_w8a16_wide_tiles_for_wide_outputs(device, M, N, K):
     assert_close_f16(_w8a16(Wq, x, scale, 0.5, 3.0, device), ref, "scale 0.5 zp 3")
 
 
+@pytest.mark.parametrize("M,K", [(4, 16384), (8, 16384), (13, 16384), (16, 4096), (6, 24576)])
+def test_w8a16_wide_tiles_with_one_workgroup_per_cu(device, M, K):
+    # N = 8192: 256 tiles of 32 columns, taken for long rows or 15..16 activation rows; the oracle
+    # checks three windows of output channels, exact integers first
+    N = 8192
+    g = gen(4190 + M + K)
+    xi = torch.randint(-1, 2, (M, K), generator=g).half()
+    Wsmall = torch.randint(-2, 3, (N, K), generator=g, dtype=torch.int8)
+    Wq = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8)
+    x = normal((M, K), g)
+    scale = (torch.rand(N, generator=g) * 0.009 + 0.001).half()
+    got_small = _w8a16(Wsmall, xi, None, 1.0, 0.0, device)
+    got = _w8a16(Wq, x, scale, 0.5, 3.0, device)
+    for lo in (0, 4080, N - 96):
+        ref, _ = oracle.gemv_w8a16(Wsmall[lo:lo + 96].numpy(), xi.numpy(), None, 1.0, 0.0)
+        assert np.abs(ref.astype(np.float32)).max() <= 2048
+        assert (got_small[:, lo:lo + 96] == ref).all()
+        ref, _ = oracle.gemv_w8a16(Wq[lo:lo + 96].numpy(), x.numpy(), scale[lo:lo + 96].numpy(), 0.5, 3.0)
+        assert_close_f16(got[:, lo:lo + 96], ref, "rows %d.." % lo)
+
+
 @pytest.mark.parametrize("M", [2, 4, 5, 8])
 def test_w8a16_long_rows_with_few_tiles_use_256_byte_bands(device, M):
     # fewer than 512 tiles and K > 8192: 256-byte bands (4- and 8-row strips); K = 65 bands of
