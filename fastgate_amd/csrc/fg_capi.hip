@@ -232,7 +232,8 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
     // 24.3 / mfma4 22.3; M=8 dot2 27.8 / mfma4 25.6 / row-load 23.3; M=16 mfma4 36 / direct
     // 16x16x32 31.7 / transposing 27.3 / row-load 24.6.  Every rule below is the measured winner of
     // a sweep over K = N in 1024..16384 and the LLaMA / DiT projection shapes for its range.
-    if (M <= 2 || (M <= 4 && N <= 2048 && K >= 8192)) {
+    const bool huge = K >= 16384 && N >= 16384;  // the 4x4x4 MFMA kernel's zone, also for M <= 2
+    if ((M <= 2 && !huge) || (M <= 4 && N <= 2048 && K >= 8192)) {
       // (few, long rows at M = 3..4: v_dot2 8.8-9.3 us against 9.4-9.5 for N = 2048, K = 8192)
       p->kernel = FG_KERNEL_NK_DOT2;
       p->m_block = M <= 2 ? M : 4;
@@ -240,8 +241,9 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
       p->unroll = (K >= 16384 || M > 2) ? 2 : 1;
       items = ceil_div(K / 8, 64 * p->unroll);
       p->stagger = items <= 16;  // at most 4 steps for 4 waves
-    } else if (M <= 8 && K >= 16384 && N >= 16384) {
-      // (K = N = 16384: M = 4 78.7 us against 79.9 for the row-load kernel, M = 8 77.5 / 78.9; at
+    } else if (M <= 8 && huge) {
+      // (K = N = 16384: M = 1 79.8 us against 82.1 for v_dot2, M = 2 79.1 / 81.5, M = 4 78.7 against
+      // 79.9 for the row-load kernel, M = 8 77.5 / 78.9; at
       // N = 8192, K = 28672 the row-load kernel is ahead, M = 8 69.8 / 78.3)
       p->kernel = FG_KERNEL_NK_MFMA4;
       p->m_block = M <= 4 ? 4 : 8;
