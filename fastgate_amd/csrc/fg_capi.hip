@@ -238,9 +238,13 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
       p->kernel = FG_KERNEL_NK_DOT2;
       p->m_block = M <= 2 ? M : 4;
       p->tile_n = 4;
-      p->unroll = (K >= 16384 || M > 2) ? 2 : 1;
+      // two load groups in flight beyond K = 8192 (K=11008 N=4096 M=1 16.7 -> 15.8 us, K=14336
+      // 20.0 -> 19.0); start steps by workgroup id below K = 8192 and between 8192 and 16384, by
+      // workgroup id / 8 at 8192 (22.0 -> 21.8) and from 16384 on (N=4096 23.2 -> 21.6, N=8192
+      // 42.5 -> 40.2, N=14336 71.5 -> 68.8)
+      p->unroll = (K > 8192 || M > 2) ? 2 : 1;
       items = ceil_div(K / 8, 64 * p->unroll);
-      p->stagger = items <= 16;  // at most 4 steps for 4 waves
+      p->stagger = M <= 2 ? (K < 8192 || (K > 8192 && K < 16384)) : items <= 16;
     } else if (M <= 8 && huge) {
       // (K = N = 16384: M = 1 79.8 us against 82.1 for v_dot2, M = 2 79.1 / 81.5, M = 4 78.7 against
       // 79.9 for the row-load kernel, M = 8 77.5 / 78.9; at
