@@ -324,6 +324,7 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
       // [K,N] tiles are 128 columns wide, so the grid needs split-K to cover the chip: the
       // factor that brings tiles*S closest to one workgroup per CU.
       int best = 1;
+      bool half_filled = false;  // fewer workgroups than CUs on purpose
       if ((size_t)N * K < ((size_t)1 << 26) && items >= 16 && M <= 16) {
         // Below 8192 x 8192 the call is latency-bound: 8 waves per workgroup and half the split
         // (about 192 workgroups) shorten every wave's chain of dependent loads.  Measured (us,
@@ -332,12 +333,20 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
         // Here the in-launch reduction also wins for 9..16 rows (M = 16: K=3072 N=12288 17.2 us
         // against 17.9 with the second kernel, K=12288 N=3072 18.9 / 20.0, K=4096 N=11008 19.3 /
         // 20.3); at 8192 x 8192 the second kernel stays 0.6 us ahead for them.
+        // Sixteen tiles or fewer with K <= 8192 leave each wave one or two units at 192 workgroups:
+        // aim at 128 there (N=2048: K=4096 M=1 9.7 -> 8.1 us, M=16 10.8 -> 9.0; K=8192 12.0 -> 10.6).
+        // Eight tiles with long K take a 24-way split (N=1024 K=28672: M=1 15.3 -> 13.8, M=16 17.9
+        // -> 16.2) as long as every wave keeps two units.
         p->waves = 8;
         p->fused = 1;
+        half_filled = tiles <= 16 && K <= 8192;
+        const double target = half_filled ? 128.0 : 192.0;
         double best_dist = 1e30;
-        for (int S = 1; S <= 16; S *= 2) {
+        static const int kSplits[] = {1, 2, 4, 8, 16, 24};
+        for (int S : kSplits) {
           if (items / (p->waves * S) < 1) break;
-          const double dist = std::fabs(std::log2((double)tiles * S / 192.0));
+          if (S > 16 && (tiles > 8 || items / (p->waves * S) < 2)) break;
+          const double dist = std::fabs(std::log2((double)tiles * S / target));
           if (dist < best_dist - 1e-9) {
             best_dist = dist;
             best = S;
@@ -389,7 +398,7 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
         };
         const int n0 = tiles * p->splitk;
         const double fill0 = (double)n0 / ((double)ceil_div(n0, kCUs) * kCUs);
-        if (fill0 < 0.85 && M <= 16 && (size_t)N * K >= ((size_t)1 << 22)) {
+        if (fill0 < 0.85 && !half_filled && M <= 16 && (size_t)N * K >= ((size_t)1 << 22)) {
           double best_score = score(p->splitk, p->waves) * 1.05;  // switch for a clear win only
           int best_s = 0, best_w = 0;
           for (int S = 1; S <= 16; ++S) {

@@ -207,11 +207,12 @@ __device__ __forceinline__ float4_t sum_partials_batched(const float* part, int 
   }
   return sum;
 }
-// DEEP: splits beyond four are common for the caller ([K,N] kernels), worth eight loads in flight
-// and the registers they take.
+// DEEP: splits beyond four are common for the caller ([K,N] kernels), worth eight or sixteen loads
+// in flight and the registers they take.
 template <bool DEEP>
 __device__ __forceinline__ float4_t sum_partials(const float* part, int S, size_t MN, size_t off) {
   if constexpr (DEEP) {
+    if (S > 8) return sum_partials_batched<16>(part, S, MN, off);
     if (S > 4) return sum_partials_batched<8>(part, S, MN, off);
   }
   return sum_partials_batched<4>(part, S, MN, off);
