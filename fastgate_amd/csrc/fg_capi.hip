@@ -296,8 +296,10 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
       }
     }
   } else {
-    if (M <= 2 && (size_t)N * K < ((size_t)1 << 28)) {
-      // (at K = N = 16384 the MFMA kernel streams better even for M = 1: 80 us against 90)
+    if (M <= 2 && (size_t)N * K < ((size_t)1 << (M == 1 ? 28 : 27))) {
+      // (at K = N = 16384 the MFMA kernel streams better even for M = 1: 80 us against 90; two rows
+      // from 2^27 weights on: K=8192 N=16384 43.7 / 46.0, K=28672 N=8192 76.5 / 78.4, K=8192 N=28672
+      // 73.9 / 75.3, where M = 1 is level)
       p->kernel = FG_KERNEL_KN_DOT2;
       p->m_block = M;
     } else {
