@@ -163,6 +163,12 @@ WideTile pick_wide_tile(int M, int N, int K, int splitk) {
   if (N % 32 == 0) {
     const int t32 = N / 32;
     offer(32, 8, 1, t32, t32 <= kCUs && 4 * t32 >= 3 * kCUs && (M >= 4 || t32 < kCUs));
+    // 64 columns on 13/16 of the CUs or more beat two 4-wave workgroups of 32 on each
+    // (N=14336 K=4096: M=8 21.0 -> 20.0 us, M=16 21.9 -> 20.8; N=13824 K=5120 M=8 25.8 -> 24.7)
+    if (N % 64 == 0) {
+      const int t64 = N / 64;
+      offer(64, 8, 1, t64, M >= 8 && K >= 2048 && t64 < kCUs && 16 * t64 >= 13 * kCUs);
+    }
     offer(32, 4, 1, t32, 8 * t32 >= 7 * 2 * kCUs && t32 <= 2 * kCUs && (t32 == 2 * kCUs ? M >= 5 : M >= 9));
   }
   if (N % 48 == 0) {
