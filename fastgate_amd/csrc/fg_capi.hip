@@ -162,7 +162,9 @@ WideTile pick_wide_tile(int M, int N, int K, int splitk) {
   const bool auto_split = splitk == 0;
   if (N % 32 == 0) {
     const int t32 = N / 32;
-    offer(32, 8, 1, t32, t32 <= kCUs && 4 * t32 >= 3 * kCUs && (M >= 4 || t32 < kCUs));
+    // not at K = 4096, where rows 8 KB apart make this form 8-15 % slower than 16-column tiles
+    // (N=8192 M=8 14.6 us against 12.5; K = 3840 and 4352 are unaffected)
+    offer(32, 8, 1, t32, t32 <= kCUs && 4 * t32 >= 3 * kCUs && (M >= 4 || t32 < kCUs) && K != 4096);
     // 64 columns on 13/16 of the CUs or more beat two 4-wave workgroups of 32 on each
     // (N=14336 K=4096: M=8 21.0 -> 20.0 us, M=16 21.9 -> 20.8; N=13824 K=5120 M=8 25.8 -> 24.7)
     if (N % 64 == 0) {
@@ -211,7 +213,10 @@ WideTile pick_wide_tile(int M, int N, int K, int splitk) {
   if (K >= 1024 && N % kCUs == 0) {
     const int tw = N / kCUs;
     const bool thin16 = N / 16 < 3 * kCUs / 2;  // 16-column tiles would leave CUs with one workgroup
-    offer(tw, 8, 1, kCUs, tw >= 20 && tw < 48 && tw % 16 != 0 && (M >= 9 || (thin16 && M >= 4)),
+    // (K = 4096 again, two nearly full column blocks: N=7168 M=9 28 columns 14.4 us against 13.0 for
+    // 16; N=6144 24 columns 10.9 / 11.6 and N=11008 43 columns 17.0 / 18.4 are unaffected)
+    offer(tw, 8, 1, kCUs,
+          tw >= 20 && tw < 48 && tw % 16 != 0 && (M >= 9 || (thin16 && M >= 4)) && !(K == 4096 && tw > 24 && tw < 32),
           tw > 32 ? 0.3 : 0.15);
   }
   if (K >= 1024 && N % (2 * kCUs) == 0) {
