@@ -170,12 +170,16 @@ WideTile pick_wide_tile(int M, int N, int K, int splitk) {
     if (N % 64 == 0) {
       const int t64 = N / 64;
       offer(64, 8, 1, t64, M >= 8 && K >= 2048 && t64 < kCUs && 16 * t64 >= 13 * kCUs);
+      // ... and one 64-column workgroup on every CU for 12 rows and more (N=16384 M=16: K=5120
+      // 30.1 -> 28.0 us, K=14336 73.4 -> 70.5)
+      offer(64, 8, 1, t64, M >= 12 && K >= 5120 && t64 == kCUs);
     }
     offer(32, 4, 1, t32, 8 * t32 >= 7 * 2 * kCUs && t32 <= 2 * kCUs && (t32 == 2 * kCUs ? M >= 5 : M >= 9));
   }
   if (N % 48 == 0) {
     const int t48 = N / 48;
-    offer(48, 8, 1, t48, M >= 8 && ((t48 <= kCUs && 4 * t48 >= 3 * kCUs) || (t48 == 2 * kCUs && M >= 9)));
+    // (one a CU from four rows on: N=9216 M=4 K=4096 14.9 -> 14.2 us, K=8192 27.7 -> 25.5)
+    offer(48, 8, 1, t48, (M >= 4 && t48 <= kCUs && 4 * t48 >= 3 * kCUs) || (t48 == 2 * kCUs && M >= 9));
   }
   if (N % 64 == 0) {
     // very wide outputs (N=28672 K=8192 M=16: 64 columns 72.1 us, 32 columns 74.0, 16 columns 81+)
@@ -440,13 +444,21 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
       // 128 tiles or fewer want two workgroups per CU once K is long (N=2048: K=8192 M=16
       // 10.5 us with S = 2 against 12.4, K=16384 15.7 against 21.7).  The partials of a 16-column
       // tile are small, so the split always completes inside the launch.
-      int S = (tiles > kCUs / 2 || K < 8192) ? 1 : ceil_div(kCUs, tiles);
+      // (from K = 5120 on for 8 rows and more: N=1024 K=6144 M=16 10.2 -> 7.9 us, N=2048 K=6144
+      // M=8 9.0 -> 8.0)
+      int S = (tiles > kCUs / 2 || K < (M >= 8 ? 5120 : 8192)) ? 1 : ceil_div(kCUs, tiles);
       while (S > 1 && items / (p->waves * S) < 2) --S;  // keep two bands per wave
       p->splitk = S;
       p->fused = 1;
       // with only two 256-byte bands left per wave, four of 128 bytes pipeline better
       // (N=1024 K=8192 S=4: M=8 7.8 us against 8.9, M=16 8.0 / 9.4)
       if (S > 1 && p->unroll == 1 && items / (p->waves * S) <= 2) p->band = 128;
+      // the same for short rows of wide outputs (K=2048 M=8: N=10240 10.6 -> 9.4 us, N=12288 M=4
+      // 11.1 -> 10.0; K=1024 N=13824 M=8 8.0 -> 7.7)
+      if (S == 1 && p->unroll == 1 && K >= 1024 && K <= 2048 && N >= 8192) {
+        p->band = 128;
+        p->waves = 8;
+      }
     } else {
       p->splitk = pick_splitk(tiles, p->waves, items, M, N, K, kCUs);
     }

@@ -60,10 +60,10 @@ def test_plan_is_consistent(layout, M, N, K):
     if p.splitk > 1 and p.fused:
         assert p.grid_x * p.grid_y * 4 <= hdr, d   # one counter per output tile
     # v_dot2 is the default for the smallest batches; the MFMA kernels take over above
-    if M <= 2 and N * K < 1 << 28:
+    if M <= 2 and N * K < 1 << 27:
         assert p.kernel in (capi.FG_KERNEL_KN_DOT2, capi.FG_KERNEL_NK_DOT2), d
     if p.kernel == capi.FG_KERNEL_NK_MFMA_R:
-        assert p.tile_n in (16, 32, 48) and p.m_block == (32 if M > 16 else 16), d
+        assert p.tile_n in (16, 32, 48, 64) and p.m_block == (32 if M > 16 else 16), d
     if p.kernel == capi.FG_KERNEL_NK_MFMA_T:
         assert p.splitk == -(-(K // 32) // 64) and p.waves == 4 and p.tile_n % p.unroll == 0, d
     # a forced split is honoured
