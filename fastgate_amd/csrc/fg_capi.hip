@@ -160,11 +160,18 @@ WideTile pick_wide_tile(int M, int N, int K, int splitk) {
     }
   };
   const bool auto_split = splitk == 0;
+  // Rows that do not start on a 2 KB boundary (K not a multiple of 1024) cost the 128-byte-band
+  // tiles their lead: N=12288 K=11008 M=8 48 columns 49.6 us against 42.4 for 16 columns on 256-byte
+  // bands, K=10752 46.4 / 41.9, while K=10240 and K=11264 are 40.2 and 42.6 with 48 columns;
+  // N=8192 K=11008 M=8 32 columns 31.1 / 29.8, N=16384 59.0 / 55.6.  With 9..16 rows the 32-column
+  // forms stay level.
+  const bool odd_pitch = K % 1024 != 0 && K > 4096;
   if (N % 32 == 0) {
     const int t32 = N / 32;
     // not at K = 4096, where rows 8 KB apart make this form 8-15 % slower than 16-column tiles
     // (N=8192 M=8 14.6 us against 12.5; K = 3840 and 4352 are unaffected)
-    offer(32, 8, 1, t32, t32 <= kCUs && 4 * t32 >= 3 * kCUs && (M >= 4 || t32 < kCUs) && K != 4096);
+    offer(32, 8, 1, t32, t32 <= kCUs && 4 * t32 >= 3 * kCUs && (M >= 4 || t32 < kCUs) && K != 4096 &&
+                             (!odd_pitch || M >= 9 || 8 * t32 < 7 * kCUs));
     // 64 columns on 13/16 of the CUs or more beat two 4-wave workgroups of 32 on each
     // (N=14336 K=4096: M=8 21.0 -> 20.0 us, M=16 21.9 -> 20.8; N=13824 K=5120 M=8 25.8 -> 24.7)
     if (N % 64 == 0) {
@@ -174,12 +181,13 @@ WideTile pick_wide_tile(int M, int N, int K, int splitk) {
       // 30.1 -> 28.0 us, K=14336 73.4 -> 70.5)
       offer(64, 8, 1, t64, M >= 12 && K >= 5120 && t64 == kCUs);
     }
-    offer(32, 4, 1, t32, 8 * t32 >= 7 * 2 * kCUs && t32 <= 2 * kCUs && (t32 == 2 * kCUs ? M >= 5 : M >= 9));
+    offer(32, 4, 1, t32, 8 * t32 >= 7 * 2 * kCUs && t32 <= 2 * kCUs && (t32 == 2 * kCUs ? M >= 5 : M >= 9) &&
+                             (!odd_pitch || M >= 9));
   }
   if (N % 48 == 0) {
     const int t48 = N / 48;
     // (one a CU from four rows on: N=9216 M=4 K=4096 14.9 -> 14.2 us, K=8192 27.7 -> 25.5)
-    offer(48, 8, 1, t48, (M >= 4 && t48 <= kCUs && 4 * t48 >= 3 * kCUs) || (t48 == 2 * kCUs && M >= 9));
+    offer(48, 8, 1, t48, !odd_pitch && ((M >= 4 && t48 <= kCUs && 4 * t48 >= 3 * kCUs) || (t48 == 2 * kCUs && M >= 9)));
   }
   if (N % 64 == 0) {
     // very wide outputs (N=28672 K=8192 M=16: 64 columns 72.1 us, 32 columns 74.0, 16 columns 81+)
