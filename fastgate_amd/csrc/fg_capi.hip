@@ -172,6 +172,9 @@ WideTile pick_wide_tile(int M, int N, int K, int splitk) {
     // (N=8192 M=8 14.6 us against 12.5; K = 3840 and 4352 are unaffected)
     offer(32, 8, 1, t32, t32 <= kCUs && 4 * t32 >= 3 * kCUs && (M >= 4 || t32 < kCUs) && K != 4096 &&
                              (!odd_pitch || M >= 9 || 8 * t32 < 7 * kCUs));
+    // short rows of very wide outputs: two 8-wave workgroups of 32 columns on every CU
+    // (K=2048: N=14336 M=8 12.1 -> 11.3 us, N=16384 M=16 13.7 -> 12.7)
+    offer(32, 8, 1, t32, K > 1024 && K <= 2048 && M >= 4 && t32 <= 2 * kCUs && 8 * t32 >= 13 * kCUs);
     // 64 columns on 13/16 of the CUs or more beat two 4-wave workgroups of 32 on each
     // (N=14336 K=4096: M=8 21.0 -> 20.0 us, M=16 21.9 -> 20.8; N=13824 K=5120 M=8 25.8 -> 24.7)
     if (N % 64 == 0) {
@@ -187,7 +190,8 @@ WideTile pick_wide_tile(int M, int N, int K, int splitk) {
   if (N % 48 == 0) {
     const int t48 = N / 48;
     // (one a CU from four rows on: N=9216 M=4 K=4096 14.9 -> 14.2 us, K=8192 27.7 -> 25.5)
-    offer(48, 8, 1, t48, !odd_pitch && ((M >= 4 && t48 <= kCUs && 4 * t48 >= 3 * kCUs) || (t48 == 2 * kCUs && M >= 9)));
+    offer(48, 8, 1, t48, !odd_pitch && ((M >= (t48 < kCUs ? 4 : 8) && t48 <= kCUs && 4 * t48 >= 3 * kCUs) ||
+                                        (t48 == 2 * kCUs && M >= 9)));
   }
   if (N % 64 == 0) {
     // very wide outputs (N=28672 K=8192 M=16: 64 columns 72.1 us, 32 columns 74.0, 16 columns 81+)
@@ -199,7 +203,10 @@ WideTile pick_wide_tile(int M, int N, int K, int splitk) {
     const int t32 = N / 32;
     for (int S = 2; S <= 4; ++S) {
       const int wgs = t32 * S;
-      const bool long_k = K / S >= 3072 && (S > 2 || K >= 8192);
+      // (64 tiles or fewer split four ways from 2048 k a split: N=2048 M=16 K=8192 10.2 -> 9.7 us,
+      // K=11008 12.8 -> 11.9; two ways only beyond K = 8192: N=4096 K=8192 M=16 15.0 against 14.3
+      // for 16 columns unsplit)
+      const bool long_k = t32 <= 64 ? K / S >= 2048 : K / S >= 3072 && (S > 2 || K > 8192);
       offer(32, 8, S, wgs, long_k && M >= 9 && wgs <= kCUs && 4 * wgs >= 3 * kCUs);
     }
     if (N % 48 == 0) {
@@ -207,7 +214,10 @@ WideTile pick_wide_tile(int M, int N, int K, int splitk) {
       const int t48 = N / 48;
       for (int S = 2; S <= 4; ++S) {
         const int wgs = t48 * S;
-        offer(48, 8, S, wgs, K / S >= 3072 && M >= 9 && wgs <= kCUs && 4 * wgs >= 3 * kCUs);
+        // (64 tiles: from 1536 k a split, N=3072 K=6144 M=16 11.3 -> 10.6 us; 8 rows only with long
+        // K, K=14336 18.1 -> 17.3 but K=6144 9.4 -> 10.1)
+        const bool ok48 = t48 <= 64 ? K / S >= 1536 && (M >= 9 || (M == 8 && K >= 12288)) : K / S >= 3072 && M >= 9;
+        offer(48, 8, S, wgs, ok48 && wgs <= kCUs && 4 * wgs >= 3 * kCUs);
       }
     }
     // two workgroups a CU, only where no split lands on one a CU
