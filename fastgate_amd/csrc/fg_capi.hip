@@ -329,10 +329,13 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
       }
     }
   } else {
-    if (M <= 2 && (size_t)N * K < ((size_t)1 << (M == 1 ? 28 : 27))) {
+    const size_t weights = (size_t)N * K;
+    const bool dot2_m1 = weights < ((size_t)1 << 27) || (weights < ((size_t)1 << 28) && N >= 25600);
+    if (M == 1 ? dot2_m1 : (M == 2 && weights < ((size_t)1 << 27))) {
       // (at K = N = 16384 the MFMA kernel streams better even for M = 1: 80 us against 90; two rows
       // from 2^27 weights on: K=8192 N=16384 43.7 / 46.0, K=28672 N=8192 76.5 / 78.4, K=8192 N=28672
-      // 73.9 / 75.3, where M = 1 is level)
+      // 73.9 / 75.3; one row too where such weights still need a split: K=11008 N=16384 56.7 / 59.9,
+      // K=14336 N=16384 71.7 / 77.2, while K=8192 N=28672, unsplit, is 74.9 / 73.8)
       p->kernel = FG_KERNEL_KN_DOT2;
       p->m_block = M;
     } else {
@@ -429,7 +432,11 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
           const double per_wave = (double)items / (w * S);
           const double chain = per_wave >= 8.0 ? 1.0 : std::sqrt(per_wave / 8.0);
           const double partials = 1.0 / (1.0 + 4.0 * S * M / K);
-          return fill * balance(items, w * S) * partials * chain;
+          // 9..16 rows: two 4-wave workgroups a CU write twice the partials of one 8-wave workgroup
+          // for the same K range and lose to it at equal fill (N=5120 K=8192 M=16: 11 splits of 4
+          // waves 20.4 us, 5 of 8 waves 19.2; N=9216 K=4096 18.2 / 17.6)
+          const double two_a_cu = (M > 8 && w == 4) ? 0.88 : 1.0;
+          return fill * balance(items, w * S) * partials * chain * two_a_cu;
         };
         const int n0 = tiles * p->splitk;
         const double fill0 = (double)n0 / ((double)ceil_div(n0, kCUs) * kCUs);
