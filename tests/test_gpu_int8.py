@@ -27,7 +27,7 @@ def _w8a16(Wq, x, scale, scalar_scale, zp, device):
 
 
 @pytest.mark.parametrize("M", [1, 2, 3, 4, 5, 8, 9, 13, 16])
-@pytest.mark.parametrize("N,K", [(128, 128), (256, 1152), (1024, 4096), (4096, 1024)])
+@pytest.mark.parametrize("N,K", [(128, 128), (256, 1152), (1024, 4096), (4096, 1024), (3072, 640)])
 def test_w8a16_matches_oracle(device, M, N, K):
     g = gen(4000 + M + N)
     x = normal((M, K), g)
