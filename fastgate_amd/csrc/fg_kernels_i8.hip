@@ -634,10 +634,11 @@ bool launch_w8a16(const W8A16Args& a, hipStream_t s) {
   if (a.M == 1) {  // 4 rows per workgroup, one load group in flight
     hipLaunchKernelGGL((w8a16_kernel<1, 4, 1>), dim3(a.N / 4), dim3(64 * i8_waves(a.K)), 0, s, Wq, X,
                        sc, a.scalar_scale, a.zero_point, Y, a.M, a.N, a.K);
-  } else if (a.M <= 4 && (a.N <= 2048 || (a.M == 2 && a.N <= 3072))) {
+  } else if (a.M <= 4 && (a.N <= 2048 || (a.M == 2 && a.N <= 6144))) {
     // narrow outputs leave the 16-column tiles of the row-load kernel on half the CUs or fewer: lanes
     // along K, four weight rows a workgroup (N=2048 K=8192: M=2 8.8 -> 6.0 us, M=4 9.0 -> 7.3;
-    // N=1024 K=4096 M=4 5.8 -> 4.4; N=4096 K=8192 M=4 9.6 -> 11.6 the other way)
+    // N=1024 K=4096 M=4 5.8 -> 4.4; N=4096 K=8192 M=4 9.6 -> 11.6 the other way; two rows up to
+    // N = 6144: N=4096 K=8192 9.5 -> 9.1, N=8192 K=4096 8.6 -> 9.0)
     if (a.M <= 2)
       hipLaunchKernelGGL((w8a16_kernel<2, 4, 1>), dim3(a.N / 4), dim3(64 * i8_waves(a.K)), 0, s, Wq, X,
                          sc, a.scalar_scale, a.zero_point, Y, a.M, a.N, a.K);
