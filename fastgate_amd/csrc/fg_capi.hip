@@ -179,7 +179,7 @@ WideTile pick_wide_tile(int M, int N, int K, int splitk) {
     // (N=14336 K=4096: M=8 21.0 -> 20.0 us, M=16 21.9 -> 20.8; N=13824 K=5120 M=8 25.8 -> 24.7)
     if (N % 64 == 0) {
       const int t64 = N / 64;
-      offer(64, 8, 1, t64, M >= 8 && K >= 2048 && t64 < kCUs && 16 * t64 >= 13 * kCUs);
+      offer(64, 8, 1, t64, M >= 5 && K >= 2048 && t64 < kCUs && 16 * t64 >= 13 * kCUs);
       // ... and one 64-column workgroup on every CU for 12 rows and more (N=16384 M=16: K=5120
       // 30.1 -> 28.0 us, K=14336 73.4 -> 70.5)
       offer(64, 8, 1, t64, M >= 12 && K >= 5120 && t64 == kCUs);
@@ -190,7 +190,7 @@ WideTile pick_wide_tile(int M, int N, int K, int splitk) {
   if (N % 48 == 0) {
     const int t48 = N / 48;
     // (one a CU from four rows on: N=9216 M=4 K=4096 14.9 -> 14.2 us, K=8192 27.7 -> 25.5)
-    offer(48, 8, 1, t48, !odd_pitch && ((M >= (t48 < kCUs ? 4 : 8) && t48 <= kCUs && 4 * t48 >= 3 * kCUs) ||
+    offer(48, 8, 1, t48, !odd_pitch && ((M >= (t48 < kCUs ? 3 : 8) && t48 <= kCUs && 4 * t48 >= 3 * kCUs) ||
                                         (t48 == 2 * kCUs && M >= 9)));
   }
   if (N % 64 == 0) {
@@ -216,7 +216,8 @@ WideTile pick_wide_tile(int M, int N, int K, int splitk) {
         const int wgs = t48 * S;
         // (64 tiles: from 1536 k a split, N=3072 K=6144 M=16 11.3 -> 10.6 us; 8 rows only with long
         // K, K=14336 18.1 -> 17.3 but K=6144 9.4 -> 10.1)
-        const bool ok48 = t48 <= 64 ? K / S >= 1536 && (M >= 9 || (M == 8 && K >= 12288)) : K / S >= 3072 && M >= 9;
+        const bool ok48 = (t48 <= 64 && S == 4) ? K / S >= 1536 && (M >= 9 || (M == 8 && K >= 12288))
+                                               : K / S >= 3072 && M >= 9;
         offer(48, 8, S, wgs, ok48 && wgs <= kCUs && 4 * wgs >= 3 * kCUs);
       }
     }
@@ -238,7 +239,7 @@ WideTile pick_wide_tile(int M, int N, int K, int splitk) {
     // (K = 4096 again, two nearly full column blocks: N=7168 M=9 28 columns 14.4 us against 13.0 for
     // 16; N=6144 24 columns 10.9 / 11.6 and N=11008 43 columns 17.0 / 18.4 are unaffected)
     offer(tw, 8, 1, kCUs,
-          tw >= 20 && tw < 48 && tw % 16 != 0 && (M >= 9 || (thin16 && M >= 4)) && !(K == 4096 && tw > 24 && tw < 32),
+          tw >= 20 && tw < 48 && tw % 16 != 0 && (M >= 9 || (thin16 && M >= 3)) && !(K == 4096 && tw > 24 && tw < 32),
           tw > 32 ? 0.3 : 0.15);
   }
   if (K >= 1024 && N % (2 * kCUs) == 0) {
@@ -479,8 +480,8 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
       // (N=1024 K=8192 S=4: M=8 7.8 us against 8.9, M=16 8.0 / 9.4)
       if (S > 1 && p->unroll == 1 && items / (p->waves * S) <= 2) p->band = 128;
       // the same for short rows of wide outputs (K=2048 M=8: N=10240 10.6 -> 9.4 us, N=12288 M=4
-      // 11.1 -> 10.0; K=1024 N=13824 M=8 8.0 -> 7.7)
-      if (S == 1 && p->unroll == 1 && K >= 1024 && K <= 2048 && N >= 8192) {
+      // 11.1 -> 10.0; K=1024 N=13824 M=8 8.0 -> 7.7; K=4096 N=12288 M=6 18.5 -> 16.8)
+      if (S == 1 && p->unroll == 1 && K >= 1024 && (K <= 2048 ? N >= 8192 : (K <= 4096 && N >= 12288))) {
         p->band = 128;
         p->waves = 8;
       }
