@@ -385,6 +385,10 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
         for (int S : kSplits) {
           if (items / (p->waves * S) < 1) break;
           if (S > 16 && (tiles > 8 || items / (p->waves * S) < 2)) break;
+          // 9..16 rows: the partials of a split that leaves a wave one unit cost more than the
+          // idle CUs once there are more than 192 workgroups (N=4096 K=2048 M=12: 8 ways 10.3 us,
+          // 4 ways 8.3; N=2048 K=2048 M=16: 8 ways 7.4, 4 ways 7.9)
+          if (M > 8 && S > 1 && items / (p->waves * S) < 2 && tiles * S > 192) break;
           const double dist = std::fabs(std::log2((double)tiles * S / target));
           if (dist < best_dist - 1e-9) {
             best_dist = dist;
