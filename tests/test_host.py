@@ -79,6 +79,59 @@ def test_plan_fills_the_chip_on_the_metric_shapes():
             assert p.grid_x * p.grid_y * p.grid_z >= 256, p.as_dict()
 
 
+def test_plan_choices_that_were_measured():
+    # each line is a choice the planner makes because a sweep on the GPU said so; a change here
+    # should come with a new measurement
+    def nk(M, N, K):
+        return capi.plan(M, N, K, NK)
+
+    def kn(M, N, K):
+        return capi.plan(M, N, K, KN)
+
+    R = capi.FG_KERNEL_NK_MFMA_R
+    # [N,K]: tile widths
+    assert (nk(8, 8192, 8192).kernel, nk(8, 8192, 8192).tile_n) == (R, 32)
+    assert nk(8, 8192, 4096).tile_n == 16          # rows 8 KB apart: no one-per-CU 32-column tiles
+    assert nk(9, 7168, 4096).tile_n == 16          # ... nor 28-column ones
+    assert nk(16, 11008, 4096).tile_n == 43        # three column blocks are unaffected
+    assert nk(8, 12288, 11008).tile_n == 16        # rows off 2 KB boundaries: no 48-column tiles
+    assert nk(8, 12288, 10240).tile_n == 48
+    assert nk(4, 9216, 4096).tile_n == 48 and nk(3, 9216, 8192).tile_n == 48
+    assert nk(8, 14336, 4096).tile_n == 64 and nk(16, 16384, 8192).tile_n == 64
+    assert nk(8, 14336, 2048).tile_n == 32 and nk(8, 14336, 2048).waves == 8
+    assert nk(3, 5120, 8192).tile_n == 20
+    p = nk(6, 12288, 4096)
+    assert (p.tile_n, p.band) == (16, 128)
+    # [N,K]: splits of narrow outputs
+    assert nk(16, 1024, 6144).splitk > 1 and nk(4, 1024, 6144).splitk == 1
+    p = nk(16, 2048, 8192)
+    assert (p.tile_n, p.splitk) == (32, 4)
+    assert nk(16, 4096, 8192).splitk == 1 and nk(16, 4096, 11008).splitk == 2
+    p = nk(16, 3072, 6144)
+    assert (p.tile_n, p.splitk) == (48, 4)
+    assert nk(9, 3072, 5120).splitk == 1
+    # [N,K]: one and two rows
+    p = nk(1, 8192, 8192)
+    assert (p.kernel, p.unroll, p.stagger) == (capi.FG_KERNEL_NK_DOT2, 1, 0)
+    p = nk(1, 4096, 11008)
+    assert (p.unroll, p.stagger) == (2, 1)
+    p = nk(2, 8192, 16384)
+    assert (p.unroll, p.stagger) == (2, 0)
+    assert nk(1, 16384, 16384).kernel == capi.FG_KERNEL_NK_MFMA4
+    # [K,N]
+    assert kn(1, 2048, 4096).splitk == 8 and kn(1, 2048, 16384).splitk == 16
+    assert kn(16, 1024, 28672).splitk == 24 and kn(16, 1024, 8192).splitk == 16
+    assert kn(2, 16384, 8192).kernel == capi.FG_KERNEL_KN_MFMA
+    assert kn(1, 16384, 8192).kernel == capi.FG_KERNEL_KN_MFMA
+    assert kn(1, 28672, 8192).kernel == capi.FG_KERNEL_KN_DOT2
+    assert kn(1, 8192, 8192).kernel == capi.FG_KERNEL_KN_DOT2
+    p = kn(16, 5120, 8192)
+    assert (p.splitk, p.waves) == (6, 8)
+    p = kn(12, 4096, 2048)
+    assert (p.splitk, p.waves) == (4, 8)
+    assert kn(16, 2048, 2048).splitk == 8
+
+
 def test_plan_rejects_bad_arguments():
     L = capi.lib()
     p = capi.Plan()
