@@ -614,20 +614,26 @@ bool launch_w8a16(const W8A16Args& a, hipStream_t s) {
   auto* sc = static_cast<const half_t*>(a.scale);
   auto* Y = static_cast<half_t*>(a.y);
   const int t32 = a.N / 32;
-  // 32-column tiles on 128-byte bands read half the activation bytes per weight byte.  They pay
-  // where N/32 workgroups still put two workgroups (16 waves) on every CU -- K = N = 16384, M=8:
-  // 44.8 us against 49.3; K=4096 N=16384: 14.9 / 17.3 -- and lose where they leave one (K = N =
-  // 8192, M=8: 17.2 / 16.6: the conversion wants the waves).
-  // With exactly one such workgroup per CU (N = 8192) they pay for long rows or many activation
-  // rows: K=16384 M=8 27.3 -> 25.4 us, K=28672 M=14 55.4 -> 47.8, K=4096 M=16 11.1 -> 10.5, against
-  // K=8192 M=8 14.9 -> 16.9, K=28672 M=4 38.7 -> 40.0.
-  const bool one_per_cu = a.N % 32 == 0 && t32 == 256 &&
-                          (a.M >= 15 || (a.K >= 16384 && (a.M >= 5 || a.K < 24576)));
-  const bool wide = (a.N % 32 == 0 && t32 >= 512 && t32 % 512 == 0) || one_per_cu;
-  // 16-column tiles: 128-byte bands (smaller strips, more steps in flight) except for long rows
-  // with at most one workgroup per CU -- M=8, 128- / 256-byte bands: K = N = 8192 14.5 / 15.7,
-  // K = N = 4096 7.0 / 7.3, K=4096 N=14336 14.6 / 16.1, K=14336 N=4096 15.9 / 15.6.
-  const bool bw256 = a.N / 16 < 512 && a.K > 8192;
+  // 32-column tiles on 128-byte bands read half the activation bytes per weight byte.  Measured
+  // against 16-column tiles (us):
+  //  * two workgroups (16 waves) on every CU, 448..512 tiles or a multiple of 512: K = N = 16384 M=8
+  //    44.8 / 49.3, K=4096 N=16384 14.9 / 17.3, K=4096 N=14336 M=8 13.7 / 14.5 -- but not with rows
+  //    8 KB apart: K=8192 N=16384 M=8 27.6 / 25.2;
+  //  * one workgroup on every CU (N = 8192): long rows or 15..16 activation rows only, K=16384 M=8
+  //    25.4 / 27.3, K=28672 M=14 47.8 / 55.4, K=4096 M=16 10.5 / 11.1, against K=8192 M=8 16.9 /
+  //    14.9, K=28672 M=4 40.0 / 38.7, K=2048 M=16 7.7 / 7.1;
+  //  * 13..16 rows from 160 tiles on: N=5120 K=11008 M=16 19.5 / 23.0, N=14336 K=14336 44.5 / 55.1.
+  const bool aligned = a.N % 32 == 0;
+  const bool two_per_cu = aligned && ((t32 >= 448 && t32 <= 512) || (t32 >= 512 && t32 % 512 == 0)) &&
+                          (a.K != 8192 || a.M > 8);
+  const bool one_per_cu = aligned && t32 == 256 &&
+                          ((a.M >= 15 && a.K >= 4096) || (a.K >= 16384 && (a.M >= 5 || a.K < 24576)));
+  const bool many_rows = aligned && a.M >= 13 && t32 >= 160 && t32 != 256;
+  const bool wide = two_per_cu || one_per_cu || many_rows;
+  // 16-column tiles take 128-byte bands (smaller strips, more steps in flight): M=8, 128- / 256-byte
+  // bands: K = N = 8192 14.5 / 15.7, K = N = 4096 7.0 / 7.3, K=4096 N=14336 14.6 / 16.1, K=11008
+  // N=5120 17.7 / 19.3 -- except long rows of narrow outputs, K=14336 N=4096 M=4 14.8 / 13.9.
+  const bool bw256 = a.N <= 4096 && a.K >= 14336;
 #define FG_W8A16_R(XR, BW, CB)                                                                    \
   hipLaunchKernelGGL((w8a16_r_kernel<XR, 8, BW, CB>), dim3(a.N / (16 * CB)), dim3(512), 0, s, Wq, \
                      X, sc, a.scalar_scale, a.zero_point, Y, a.M, a.N, a.K)

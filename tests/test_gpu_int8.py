@@ -44,9 +44,10 @@ def test_w8a16_matches_oracle(device, M, N, K):
 
 
 @pytest.mark.parametrize("M", [3, 4, 5, 7, 8, 9, 12, 16])
-@pytest.mark.parametrize("N,K", [(16384, 128), (16384, 384), (16384, 1152), (32768, 384)])
+@pytest.mark.parametrize("N,K", [(16384, 128), (16384, 384), (16384, 1152), (32768, 384), (14336, 640), (5120, 384)])
 def test_w8a16_wide_tiles_for_wide_outputs(device, M, N, K):
-    # N / 32 a multiple of 512: 32-column tiles on 128-byte bands, 4-, 8- or 16-row activation
+    # N / 32 a multiple of 512 or 448..512 (13..16 rows: from 160): 32-column tiles on 128-byte
+    # bands, 4-, 8- or 16-row activation
     # strips; exact small integers first (any LDS layout mistake changes the bits), then random data
     g = gen(4100 + M + N + K)
     xi = torch.randint(-3, 4, (M, K), generator=g).half()
@@ -83,11 +84,11 @@ def test_w8a16_wide_tiles_with_one_workgroup_per_cu(device, M, K):
         assert_close_f16(got[:, lo:lo + 96], ref, "rows %d.." % lo)
 
 
-@pytest.mark.parametrize("M", [2, 4, 5, 8])
-def test_w8a16_long_rows_with_few_tiles_use_256_byte_bands(device, M):
-    # fewer than 512 tiles and K > 8192: 256-byte bands (4- and 8-row strips); K = 65 bands of
-    # 128 leaves the last 256-byte band half empty.  Exact integers first, then random data
-    N, K = 2048, 8192 + 128
+@pytest.mark.parametrize("M", [5, 8])
+def test_w8a16_long_rows_of_narrow_outputs_use_256_byte_bands(device, M):
+    # N <= 4096 and K >= 14336: 256-byte bands (8-row strips); K = 113 bands of 128 leaves the
+    # last 256-byte band half empty.  Exact integers first, then random data
+    N, K = 2560, 14336 + 128
     g = gen(4170 + M)
     xi = torch.randint(-1, 2, (M, K), generator=g).half()
     Wsmall = torch.randint(-2, 3, (N, K), generator=g, dtype=torch.int8)
