@@ -201,6 +201,29 @@ def run_sweep(torch, sg, capi, dev, steps, warmup, models=False):
                  "weights_per_ns": round(Kk * Nn / us_i4 / 1e3, 3),
                  "fp16_M1_weights_per_ns": round(Kk * Nn / us_f16 / 1e3, 3),
                  "weight_throughput_vs_fp16": round(us_f16 / us_i4, 3)})
+    # beyond the benchmark's configurations: [K,N] weights of the metric shape padded to a row pitch
+    # of N + 128 elements (a view of a [K, N+128] buffer), as a caller that owns the weights can lay
+    # them out once at load time
+    g = torch.Generator(device=dev).manual_seed(2040)
+    Kp = Np = 8192
+    padded = [(torch.randn((Kp, Np + 128), device=dev, generator=g) * 0.02).half() for _ in range(5)]
+    views = [w[:, :Np] for w in padded]
+    for Mp in (1, 8, 16):
+        ap = torch.randn((Mp, Kp), device=dev, generator=g).half()
+        cp = torch.zeros((Mp, Np), dtype=torch.half, device=dev)
+        us_p = time_us(lambda i: sg.edgemm_m8n128k64x4(ap, views[i % 5], cp))
+        us_d = next(r["us_per_call"] for r in rows if r["config"] == "C5 sweep" and r["M"] == Mp
+                    and r["K"] == Kp and r["w_layout"] == "[K,N]")
+        by = 2 * Kp * Np + 2 * Mp * Kp + 2 * Mp * Np
+        pl = capi.plan(Mp, Np, Kp, capi.FG_W_KN, 0).as_dict()
+        rows.append({"config": "extra: [K,N] row pitch N+128", "op": "edgemm_m8n128k64x4", "M": Mp, "K": Kp,
+                     "N": Np, "w_layout": "[K,N] pitch 8320", "seed": 2040, "kernel": pl["kernel_name"],
+                     "splitk": pl["splitk"], "in_launch_reduce": pl["fused"], "tile_n": pl["tile_n"],
+                     "bytes": by, "us_per_call": round(us_p, 2), "GBps": round(by / us_p / 1e3, 1),
+                     "frac_hbm_peak": round(by / us_p / 1e3 / HBM_PEAK_GBPS, 4),
+                     "frac_read_ceiling": round(by / us_p / 1e3 / ceiling, 4),
+                     "us_per_call_dense": us_d})
+    del padded, views
     # beyond the benchmark's configurations: the feed-forward pair of C3 (16 x 3072 x 12288, then
     # 16 x 12288 x 3072) with bias and GELU, fused into the two GEMM launches against the same two
     # GEMMs followed by separate elementwise launches

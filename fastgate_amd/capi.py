@@ -39,6 +39,7 @@ KERNEL_NAMES = {1: "nk_dot2", 2: "nk_mfma", 3: "kn_dot2", 4: "kn_mfma", 5: "nk_m
 EXPORTS = (
     "fg_gemm_f16",
     "fg_gemm_f16_planned",
+    "fg_gemm_f16_pitched",
     "fg_gemm_f16_bias_act",
     "fg_plan",
     "fg_workspace_bytes",
@@ -103,6 +104,8 @@ def lib() -> ctypes.CDLL:
         pp = ctypes.POINTER(Plan)
         L.fg_gemm_f16.restype = ci
         L.fg_gemm_f16.argtypes = [vp, vp, vp, ci, ci, ci, ci, ci, ci, vp, sz, vp]
+        L.fg_gemm_f16_pitched.restype = ci
+        L.fg_gemm_f16_pitched.argtypes = [vp, vp, vp, ci, ci, ci, ci, ci, ci, vp, sz, vp]
         L.fg_gemm_f16_planned.restype = ci
         L.fg_gemm_f16_planned.argtypes = [vp, vp, vp, ci, ci, ci, ci, ci, pp, vp, sz, vp]
         L.fg_gemm_f16_bias_act.restype = ci

@@ -501,14 +501,17 @@ int check_launch() { return hipGetLastError() == hipSuccess ? FG_OK : FG_ERR_LAU
 // `tail`: bias and activation bits of the kernels' flag word (0 for a plain product).
 int run_gemm(const void* A, const void* W, void* C, int M, int N, int K, int accumulate,
              const fg_plan_t& p, void* ws, size_t ws_bytes, hipStream_t s, int tail = 0,
-             const void* bias = nullptr) {
+             const void* bias = nullptr, int ldw = 0) {
   if (p.splitk > 1 && (ws == nullptr || ws_bytes < p.workspace_bytes)) return FG_ERR_WORKSPACE;
   if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(W) |
        reinterpret_cast<uintptr_t>(C) | reinterpret_cast<uintptr_t>(ws)) & 15) {
     return FG_ERR_INVALID_ARG;  // 16-byte loads and stores
   }
+  const bool kn = p.kernel == FG_KERNEL_KN_DOT2 || p.kernel == FG_KERNEL_KN_MFMA;
+  if (ldw == 0) ldw = kn ? N : K;
+  if (ldw != (kn ? N : K) && (!kn || ldw < N || ldw % 8 != 0)) return FG_ERR_INVALID_ARG;
   GemmArgs a{A, W, C, nullptr, nullptr, M, N, K,
-             (accumulate ? kFlagAccumulate : 0) | (p.stagger ? kFlagStagger : 0) | tail, bias};
+             (accumulate ? kFlagAccumulate : 0) | (p.stagger ? kFlagStagger : 0) | tail, bias, ldw};
   if (p.splitk > 1) {
     a.ws = reinterpret_cast<float*>(static_cast<unsigned char*>(ws) + kWsHeaderBytes);
     a.counters = p.fused ? static_cast<int*>(ws) : nullptr;
@@ -598,6 +601,21 @@ int fg_gemm_f16(const void* A, const void* W, void* C, int M, int N, int K, int 
   }
   return fg::run_gemm(A, W, C, M, N, K, accumulate, p, ws, ws_bytes,
                       static_cast<hipStream_t>(stream));
+}
+
+int fg_gemm_f16_pitched(const void* A, const void* W, void* C, int M, int N, int K, int ldw,
+                        int accumulate, int splitk, void* ws, size_t ws_bytes, void* stream) {
+  if (A == nullptr || W == nullptr || C == nullptr) return FG_ERR_INVALID_ARG;
+  if (ldw < N || ldw % 8 != 0) return FG_ERR_INVALID_ARG;
+  fg_plan_t p;
+  int st = fg_plan(M, N, K, FG_W_KN, splitk, &p);
+  if (st != FG_OK) return st;
+  if (splitk == 0 && p.splitk > 1 && (ws == nullptr || ws_bytes < p.workspace_bytes)) {
+    st = fg_plan(M, N, K, FG_W_KN, 1, &p);
+    if (st != FG_OK) return st;
+  }
+  return fg::run_gemm(A, W, C, M, N, K, accumulate, p, ws, ws_bytes, static_cast<hipStream_t>(stream),
+                      0, nullptr, ldw);
 }
 
 int fg_gemm_f16_planned(const void* A, const void* W, void* C, int M, int N, int K, int w_layout,

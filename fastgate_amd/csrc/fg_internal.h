@@ -21,6 +21,7 @@ struct GemmArgs {
   int accumulate;  // flag word: bit 0 C += A*W; bit 1 plan.stagger (start step = workgroup id %
                    // steps); bit 4 add bias; bits 5-7 activation (FG_ACT_*)
   const void* bias;  // fp16 [N] when bit 4 is set
+  int ldw;           // elements between consecutive rows of W; [K,N] kernels only (else N or K)
 };
 
 // Tile sets that exist as instantiations (the planner and the validators share these).

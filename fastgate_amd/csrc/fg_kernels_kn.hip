@@ -42,7 +42,7 @@ __global__ __launch_bounds__(64 * NW) void kn_mfma_kernel(const half_t* __restri
                                                       const half_t* __restrict__ W,
                                                       half_t* __restrict__ C,
                                                       float* __restrict__ ws, int* counters, int M, int N,
-                                                      int K, int flags, const void* bias) {
+                                                      int K, int flags, const void* bias, int ldw) {
   __shared__ float red[NW][16][128];  // NW = most waves per workgroup
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -60,7 +60,7 @@ __global__ __launch_bounds__(64 * NW) void kn_mfma_kernel(const half_t* __restri
 
   const bool arow = (m0 + j) < M;
   const half_t* Ap = A + (size_t)(m0 + (arow ? j : 0)) * K + g * 8;
-  const half_t* Wp = W + (size_t)(g * 8) * N + n0 + j * 8;
+  const half_t* Wp = W + (size_t)(g * 8) * ldw + n0 + j * 8;
   const u32x4 zero = {0u, 0u, 0u, 0u};
 
   for (int u0 = slot * U; u0 < nunits; u0 += slots * U) {
@@ -72,7 +72,7 @@ __global__ __launch_bounds__(64 * NW) void kn_mfma_kernel(const half_t* __restri
       const bool ok = unit < nunits;
 #pragma unroll
       for (int i = 0; i < 8; ++i)
-        rows[u][i] = ok ? load16<STREAM>(Wp + (size_t)(unit * 32 + i) * N) : zero;
+        rows[u][i] = ok ? load16<STREAM>(Wp + (size_t)(unit * 32 + i) * ldw) : zero;
       a[u] = (ok && arow) ? load16<false>(Ap + (size_t)unit * 32) : zero;
     }
 #pragma unroll
@@ -133,7 +133,7 @@ __global__ __launch_bounds__(64 * NW) void kn_dot2_kernel(const half_t* __restri
                                                       const half_t* __restrict__ W,
                                                       half_t* __restrict__ C,
                                                       float* __restrict__ ws, int* counters, int M, int N,
-                                                      int K, int flags, const void* bias) {
+                                                      int K, int flags, const void* bias, int ldw) {
   __shared__ float red[4 * NW][MB][128];  // NW = most waves per workgroup
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -152,7 +152,7 @@ __global__ __launch_bounds__(64 * NW) void kn_dot2_kernel(const half_t* __restri
     for (int m = 0; m < MB; ++m) acc[i][m] = 0.f;
 
   const half_t* Ap = A + (size_t)m0 * K + g * 8;
-  const half_t* Wp = W + (size_t)(g * 8) * N + n0 + j * 8;
+  const half_t* Wp = W + (size_t)(g * 8) * ldw + n0 + j * 8;
   const u32x4 zero = {0u, 0u, 0u, 0u};
 
   for (int u0 = slot * U; u0 < nunits; u0 += slots * U) {
@@ -164,7 +164,7 @@ __global__ __launch_bounds__(64 * NW) void kn_dot2_kernel(const half_t* __restri
       const bool ok = unit < nunits;
 #pragma unroll
       for (int i = 0; i < 8; ++i)
-        rows[u][i] = ok ? load16<STREAM>(Wp + (size_t)(unit * 32 + i) * N) : zero;
+        rows[u][i] = ok ? load16<STREAM>(Wp + (size_t)(unit * 32 + i) * ldw) : zero;
 #pragma unroll
       for (int m = 0; m < MB; ++m)
         xr[u][m] =
@@ -221,16 +221,16 @@ static void kn_dot2_go(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
   if constexpr (MB <= 2) {
     if (p.waves == 8) {
       hipLaunchKernelGGL((kn_dot2_kernel<MB, U, true, 8>), grid, block, 0, s, A, W, C, a.ws, a.counters, a.M,
-                         a.N, a.K, a.accumulate, a.bias);
+                         a.N, a.K, a.accumulate, a.bias, a.ldw);
       return;
     }
   }
   if (p.stream_w)
     hipLaunchKernelGGL((kn_dot2_kernel<MB, U, true, 4>), grid, block, 0, s, A, W, C, a.ws, a.counters, a.M, a.N,
-                       a.K, a.accumulate, a.bias);
+                       a.K, a.accumulate, a.bias, a.ldw);
   else
     hipLaunchKernelGGL((kn_dot2_kernel<MB, U, false, 4>), grid, block, 0, s, A, W, C, a.ws, a.counters, a.M, a.N,
-                       a.K, a.accumulate, a.bias);
+                       a.K, a.accumulate, a.bias, a.ldw);
 }
 
 template <int MB>
@@ -264,13 +264,13 @@ static void kn_mfma_go(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
   auto* C = static_cast<half_t*>(a.C);
   if (p.waves == 8) {
     hipLaunchKernelGGL((kn_mfma_kernel<U, true, 8>), grid, block, 0, s, A, W, C, a.ws, a.counters, a.M, a.N, a.K,
-                       a.accumulate, a.bias);
+                       a.accumulate, a.bias, a.ldw);
   } else if (p.stream_w) {
     hipLaunchKernelGGL((kn_mfma_kernel<U, true, 4>), grid, block, 0, s, A, W, C, a.ws, a.counters, a.M, a.N, a.K,
-                       a.accumulate, a.bias);
+                       a.accumulate, a.bias, a.ldw);
   } else {
     hipLaunchKernelGGL((kn_mfma_kernel<U, false, 4>), grid, block, 0, s, A, W, C, a.ws, a.counters, a.M, a.N, a.K,
-                       a.accumulate, a.bias);
+                       a.accumulate, a.bias, a.ldw);
   }
 }
 

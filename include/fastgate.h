@@ -114,6 +114,17 @@ typedef struct fg_plan_t {
 int fg_gemm_f16(const void* A, const void* W, void* C, int M, int N, int K, int w_layout,
                 int accumulate, int splitk, void* ws, size_t ws_bytes, void* stream);
 
+/*
+ * fg_gemm_f16 for [K,N] weights whose rows are ldw >= N elements apart (ldw a multiple of 8):
+ * W[k][n] at W + k*ldw + n.  No counterpart in the reference, whose tensors are contiguous.  It is
+ * for callers that own the weights and can pad them once at load time: when N is a multiple of 512
+ * every byte a wave has in flight sits at the same offset within 1 KB, and rows 256 bytes further
+ * apart (ldw = N + 128) make the same call about 9 % faster (M = 16, K = N = 8192: 26.1 -> 23.5 us).
+ * The result is the one fg_gemm_f16 gives on the dense copy, bit for bit.
+ */
+int fg_gemm_f16_pitched(const void* A, const void* W, void* C, int M, int N, int K, int ldw,
+                        int accumulate, int splitk, void* ws, size_t ws_bytes, void* stream);
+
 /* Same computation with an explicit plan (kernel family, tile, split-K, unroll).  Grid and
  * workspace fields of *plan are recomputed and written back. */
 int fg_gemm_f16_planned(const void* A, const void* W, void* C, int M, int N, int K,

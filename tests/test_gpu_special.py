@@ -7,7 +7,7 @@ import torch
 
 import oracle
 from fastgate_amd import capi
-from helpers import capi_gemm, gen, normal, ptr, stream_ptr
+from helpers import assert_close_f16, capi_gemm, gen, normal, ptr, stream_ptr
 
 pytestmark = pytest.mark.gpu
 
@@ -92,3 +92,49 @@ def test_int8_gemv_with_non_finite_activations(device):
         got = y.cpu().numpy()
         _same_class(got, ref.reshape(M, N))
         assert np.isnan(got[0]).all() and np.isnan(got[M - 1]).all()
+
+
+# ---------------------------------------------------------------------------------------
+# [K,N] weights with padded rows
+# ---------------------------------------------------------------------------------------
+@pytest.mark.parametrize("M", [1, 2, 5, 16])
+@pytest.mark.parametrize("N,K,pad", [(512, 1152, 8), (1024, 640, 128), (2048, 4096, 136)])
+def test_pitched_kn_weights_match_the_dense_call_bit_for_bit(device, M, N, K, pad):
+    import fastgate_amd
+
+    sg = fastgate_amd.speedgate
+    g = gen(9100 + M + N + pad)
+    A = normal((M, K), g)
+    W = normal((K, N), g, 0.05)
+    ref, _ = oracle.gemm_f16(A.numpy(), W.numpy(), oracle.W_KN)
+    padded = torch.full((K, N + pad), float("nan"), dtype=torch.half, device=device)
+    padded[:, :N] = W.to(device)
+    view = padded[:, :N]
+    assert not view.is_contiguous() and view.stride(0) == N + pad
+    Ad = A.to(device)
+    dense = torch.full((M, N), float("nan"), dtype=torch.half, device=device)
+    pitched = torch.full((M, N), float("nan"), dtype=torch.half, device=device)
+    sg.edgemm_m8n128k64x4(Ad, W.to(device), dense)
+    sg.edgemm_m8n128k64x4(Ad, view, pitched)
+    assert_close_f16(pitched.cpu().numpy(), ref, "pitch %d" % (N + pad))
+    assert (pitched.cpu().numpy().view(np.uint16) == dense.cpu().numpy().view(np.uint16)).all()
+    # accumulate protocol through a flat_gemm name
+    acc = torch.ones((M, N), dtype=torch.half, device=device)
+    sg.flat_gemm_m8n128k64x4_bz1(Ad, view, acc, 0)
+    ref_acc, _ = oracle.gemm_f16(A.numpy(), W.numpy(), oracle.W_KN, C=np.ones((M, N), np.float16),
+                                 accumulate=True)
+    assert_close_f16(acc.cpu().numpy(), ref_acc, "accumulate, pitch %d" % (N + pad))
+
+
+def test_pitched_entry_point_rejects_bad_pitches(device):
+    L = capi.lib()
+    M, N, K = 4, 256, 256
+    A = torch.zeros((M, K), dtype=torch.half, device=device)
+    W = torch.zeros((K, N + 64), dtype=torch.half, device=device)
+    C = torch.zeros((M, N), dtype=torch.half, device=device)
+    ws = torch.zeros(1 << 20, dtype=torch.uint8, device=device)
+    args = lambda ldw: (ptr(A), ptr(W), ptr(C), M, N, K, ldw, 0, 0, ptr(ws), ws.numel(), stream_ptr())
+    assert L.fg_gemm_f16_pitched(*args(N + 64)) == capi.FG_OK
+    assert L.fg_gemm_f16_pitched(*args(N - 8)) == capi.FG_ERR_INVALID_ARG      # rows overlap
+    assert L.fg_gemm_f16_pitched(*args(N + 4)) == capi.FG_ERR_INVALID_ARG      # not 16-byte rows
+    torch.cuda.synchronize()
