@@ -19,7 +19,7 @@ pytestmark = pytest.mark.gpu
 
 NS = (1024, 2048, 3072, 5120, 6144, 7168, 8192, 9216, 11008, 12288, 14336, 16384)
 KS = (2048, 4096, 6144, 8192, 11008)
-MS = (1, 3, 6, 9, 13, 16)
+MS = (1, 3, 6, 9, 13, 16, 24)
 
 
 @pytest.fixture(scope="module")
