@@ -396,9 +396,11 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
           }
         }
       } else if ((size_t)N * K >= ((size_t)1 << 18)) {  // 1024 x 1024: 7.7 us with S = 8 against 9.0 without
-        // up to four rows the partials are small enough for two workgroups per CU to pay
-        // (K = N = 8192, S = 8 / S = 4: M=1 24.4 / 25.3 us, M=4 25.0 / 25.4, M=8 25.7 / 25.2)
-        const int target = (M <= 4 && tiles <= 64 && (size_t)N * K <= ((size_t)1 << 26)) ? 2 * kCUs : kCUs;
+        // up to eight rows the partials are small enough for two workgroups per CU to pay, the more
+        // so as the two take neighbouring column bands (K = N = 8192, S = 8 / S = 4: M=1 23.1 / 24.3
+        // us, M=4 23.9 / 25.4, M=8 24.7 / 24.9; K=4096 N=16384 M=1 S = 4 / 2: 23.3 / 24.5)
+        const bool two_a_cu = (size_t)N * K <= ((size_t)1 << 26) && ((M <= 8 && tiles <= 64) || (M <= 2 && tiles <= 128));
+        const int target = two_a_cu ? 2 * kCUs : kCUs;
         double best_ratio = 1e30;
         for (int S = 1; S <= 16; S *= 2) {
           if (items / (p->waves * S) < 1) break;

@@ -250,9 +250,11 @@ __device__ __forceinline__ void splitk_reduce_tile(const float* part, half_t* C,
 // without counters a second kernel does.
 template <int MROWS, int NCOLS, bool DEEP = false>
 __device__ __forceinline__ void finish_splitk(float* ws, int* counters, half_t* C, int M, int N,
-                                              int m0, int n0, int flags, const void* bias) {
+                                              int m0, int n0, int flags, const void* bias,
+                                              int tile_x = -1) {
+  if (tile_x < 0) tile_x = blockIdx.x;
   if (gridDim.z > 1 && counters != nullptr) {
-    if (splitk_last_arriver(counters + blockIdx.y * gridDim.x + blockIdx.x, gridDim.z))
+    if (splitk_last_arriver(counters + blockIdx.y * gridDim.x + tile_x, gridDim.z))
       splitk_reduce_tile<DEEP>(ws, C, gridDim.z, M, N, m0, MROWS, n0, NCOLS, flags, bias);
   }
 }
