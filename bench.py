@@ -54,10 +54,10 @@ TRAFFIC_BYTES = {
     "nk_mfma_r_M8": _traffic(66083.0, 128.0),
     "nk_mfma_r_M16": _traffic(66604.5, 256.0),
     # [K,N]: split-K partials are written through and read back inside the launch; WRITE_SIZE counts
-    # the write-through stores twice (M=1: 8 x 16 KiB of partials, M=8: 4 x 256 KiB, M=16: 4 x 512 KiB)
-    "kn_dot2_M1": _traffic(65788.6, 290.0),
-    "kn_mfma_M8": _traffic(66635.0, 2186.0),
-    "kn_mfma_M16": _traffic(67650.0, 4362.0),
+    # the write-through stores twice (M=1: 8 x 16 KiB of partials, M=8: 8 x 256 KiB, M=16: 4 x 512 KiB)
+    "kn_dot2_M1": _traffic(65787.4, 290.0),
+    "kn_mfma_M8": _traffic(67145.6, 4242.0),
+    "kn_mfma_M16": _traffic(67662.0, 4362.0),
 }
 
 
