@@ -468,6 +468,19 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
           }
         }
       }
+      // One or two rows: two 4-wave workgroups a CU on neighbouring column bands instead of one
+      // 8-wave workgroup, where that lands on 448..512 workgroups and leaves every wave four units
+      // (M=1, twice the split with 4 waves / 8 waves: K=14336 N=8192 37.3 / 40.6 us, K=11008 N=8192
+      // 30.4 / 32.4, K=5120 N=16384 28.2 / 29.8; M=2: K=11008 N=4096 17.6 / 18.5, K=4096 N=8192
+      // 14.1 / 14.7)
+      {
+        const int twice = 2 * tiles * p->splitk;
+        if (splitk == 0 && M <= 2 && p->kernel == FG_KERNEL_KN_DOT2 && p->waves == 8 &&
+            p->splitk <= 8 && twice >= 448 && twice <= 2 * kCUs && items / (4 * 2 * p->splitk) >= 4) {
+          p->splitk *= 2;
+          p->waves = 4;
+        }
+      }
     } else if (wide_band_split) {
       p->splitk = wide_band_split;
       p->fused = 1;

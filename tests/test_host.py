@@ -130,6 +130,14 @@ def test_plan_choices_that_were_measured():
     p = kn(12, 4096, 2048)
     assert (p.splitk, p.waves) == (4, 8)
     assert kn(16, 2048, 2048).splitk == 8
+    # one or two rows: two 4-wave workgroups a CU where that lands on 448..512 workgroups
+    for (N, K, S) in ((8192, 14336, 8), (8192, 4096, 8), (16384, 5120, 4), (4096, 11008, 16), (10240, 4096, 6)):
+        p = kn(1, N, K)
+        assert (p.splitk, p.waves) == (S, 4), (N, K, p.as_dict())
+    p = kn(1, 4096, 4096)
+    assert (p.splitk, p.waves) == (8, 8)           # two units a wave only: stays one 8-wave workgroup a CU
+    p = kn(2, 12288, 4096)
+    assert (p.splitk, p.waves) == (2, 8)           # 384 workgroups would fill the CUs unevenly
 
 
 def test_plan_rejects_bad_arguments():
