@@ -57,7 +57,7 @@ TRAFFIC_BYTES = {
     # the write-through stores twice (M=1: 8 x 16 KiB of partials, M=8: 8 x 256 KiB, M=16: 4 x 512 KiB)
     "kn_dot2_M1": _traffic(65787.4, 290.0),
     "kn_mfma_M8": _traffic(67145.6, 4242.0),
-    "kn_mfma_M16": _traffic(67662.0, 4362.0),
+    "kn_mfma_M16": _traffic(67667.5, 4362.0),
 }
 
 

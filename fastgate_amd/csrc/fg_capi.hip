@@ -468,6 +468,15 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
           }
         }
       }
+      // 9..16 rows, four splits of 64 tiles (one workgroup on every CU) and at least eight units a
+      // wave: eight waves with two units in flight (K = N = 8192 M=16 26.2 -> 25.7 us, K=14336
+      // 42.0 -> 41.2; not with rows off 2 KB boundaries, and not with other splits: K=4096 N=12288
+      // 21.1 -> 21.6)
+      if (p->kernel == FG_KERNEL_KN_MFMA && M > 8 && M <= 16 && tiles == 64 && p->splitk == 4 &&
+          K % 1024 == 0 && items / (8 * 4) >= 8 && (size_t)N * K <= ((size_t)1 << 27)) {
+        p->waves = 8;
+        p->unroll = 2;
+      }
       // One or two rows: two 4-wave workgroups a CU on neighbouring column bands instead of one
       // 8-wave workgroup, where that lands on 448..512 workgroups and leaves every wave four units
       // (M=1, twice the split with 4 waves / 8 waves: K=14336 N=8192 37.3 / 40.6 us, K=11008 N=8192
