@@ -171,7 +171,12 @@ __device__ __forceinline__ half_t finish_value(float sum, const half_t* c, int n
 
 __device__ __forceinline__ bool splitk_last_arriver(int* counter, int S) {
   __shared__ int s_last;
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // partial stores have completed
+  // Every wave waits until its own partial stores are acknowledged (write-through: they are in
+  // memory then) before the barrier that precedes the arrival.  The workgroup-scope release
+  // alone does not do that: the waves of a workgroup share a CU, so the compiler emits no wait
+  // for it, and an arrival could overtake a partial on its way through another L2 channel.
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0); expcnt and lgkmcnt left alone
   __syncthreads();
   if (threadIdx.x == 0) {
     const int old = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
