@@ -35,6 +35,12 @@ __global__ __launch_bounds__(512) void w8a16_kernel(const int8_t* __restrict__ W
   const int n0 = blockIdx.x * RN;
   const int nq = K >> 4;  // 16-weight chunks per row
   const bool use_zp = zero_point != 0.f;
+  // scale of the output this thread writes at the end, fetched ahead of the weight stream (a load
+  // issued after the last barrier would add its whole latency to the workgroup's life)
+  static_assert(RN * MB <= 64, "one output per thread of the first wave");
+  float out_scale = scalar_scale;
+  if (scale != nullptr && threadIdx.x < RN * MB)
+    out_scale *= static_cast<float>(scale[n0 + threadIdx.x % RN]);
 
   float acc[RN][MB];
   float xsum[MB];
@@ -118,11 +124,7 @@ __global__ __launch_bounds__(512) void w8a16_kernel(const int8_t* __restrict__ W
       xs += redx[p][m];
     }
     const int n = n0 + r;
-    if (m < M) {
-      float s = scalar_scale;
-      if (scale != nullptr) s *= static_cast<float>(scale[n]);
-      Y[(size_t)m * N + n] = static_cast<half_t>((sum - zero_point * xs) * s);
-    }
+    if (m < M) Y[(size_t)m * N + n] = static_cast<half_t>((sum - zero_point * xs) * out_scale);
   }
 }
 
@@ -234,6 +236,11 @@ __global__ __launch_bounds__(256) void w4a16_kernel(const uint8_t* __restrict__ 
   const int nq = K >> 5;        // 32-weight chunks per row
   const size_t rowb = (size_t)K >> 1;  // bytes per weight row
   const bool use_zp = zero_point != 0.f;
+  // scale of the output this thread writes at the end, fetched ahead of the weight stream
+  static_assert(RN * MB <= 64, "one output per thread of the first wave");
+  float out_scale = scalar_scale;
+  if (scale != nullptr && threadIdx.x < RN * MB)
+    out_scale *= static_cast<float>(scale[n0 + threadIdx.x % RN]);
 
   float acc[RN][MB];
   float xsum[MB], xodd[MB];
@@ -321,11 +328,8 @@ __global__ __launch_bounds__(256) void w4a16_kernel(const uint8_t* __restrict__ 
       xo += redo[p][m];
     }
     const int n = n0 + r;
-    if (m < M) {
-      float s = scalar_scale;
-      if (scale != nullptr) s *= static_cast<float>(scale[n]);
-      Y[(size_t)m * N + n] = static_cast<half_t>((sum - 64.f * xo - zero_point * (xe + xo)) * s);
-    }
+    if (m < M)
+      Y[(size_t)m * N + n] = static_cast<half_t>((sum - 64.f * xo - zero_point * (xe + xo)) * out_scale);
   }
 }
 
@@ -373,6 +377,11 @@ __global__ __launch_bounds__(64 * NW) void w8a16_r_kernel(const int8_t* __restri
   const int n0 = blockIdx.x * (16 * CB);
   const int nbands = (K + BW - 1) / BW;            // K % 128 == 0: the last band may be partial
   const bool use_zp = zero_point != 0.f;
+  // scale of the output this thread writes at the end, fetched ahead of the weight stream
+  static_assert(16 * 16 * CB <= 64 * NW, "one output per thread");
+  float out_scale = scalar_scale;
+  if (scale != nullptr && threadIdx.x < 16 * 16 * CB)
+    out_scale *= static_cast<float>(scale[n0 + threadIdx.x % (16 * CB)]);
   unsigned char* wstrip = smem + wave * WAVE_LDS;
   unsigned char* xstrip = wstrip + WSTRIP;
   const u32x4 zero = {0u, 0u, 0u, 0u};
@@ -463,9 +472,7 @@ __global__ __launch_bounds__(64 * NW) void w8a16_r_kernel(const int8_t* __restri
         sum += red[wv][0][e];
         xs += red[wv][1][m * 16 + (e & 15)];
       }
-      float sc = scalar_scale;
-      if (scale != nullptr) sc *= static_cast<float>(scale[n]);
-      Y[(size_t)m * N + n] = static_cast<half_t>((sum - zero_point * xs) * sc);
+      Y[(size_t)m * N + n] = static_cast<half_t>((sum - zero_point * xs) * out_scale);
     }
   }
 }
@@ -502,6 +509,9 @@ __global__ __launch_bounds__(512) void w4a16_r_kernel(const uint8_t* __restrict_
   const int nbands = (K + 511) >> 9;             // K % 128 == 0: the last band may be partial
   const size_t rowb = (size_t)K >> 1;            // bytes per weight row
   const bool use_zp = zero_point != 0.f;
+  // scale of the output this thread writes at the end, fetched ahead of the weight stream
+  float out_scale = scalar_scale;
+  if (scale != nullptr && threadIdx.x < 256) out_scale *= static_cast<float>(scale[n0 + (threadIdx.x & 15)]);
   unsigned char* wstrip = smem + wave * WAVE_LDS;
   unsigned char* xstrip = wstrip + WSTRIP;
   const u32x4 zero = {0u, 0u, 0u, 0u};
@@ -588,9 +598,7 @@ __global__ __launch_bounds__(512) void w4a16_r_kernel(const uint8_t* __restrict_
         sum += red[wv][0][e];
         xs += red[wv][1][e];
       }
-      float sc = scalar_scale;
-      if (scale != nullptr) sc *= static_cast<float>(scale[n]);
-      Y[(size_t)m * N + n] = static_cast<half_t>((sum - zero_point * xs) * sc);
+      Y[(size_t)m * N + n] = static_cast<half_t>((sum - zero_point * xs) * out_scale);
     }
   }
 }
