@@ -106,8 +106,9 @@ __device__ __forceinline__ void wave_lds_sync() {
 // The workgroups of a tile run on different XCDs, whose L2s are not coherent with each other.
 // Agent-scope fences would fix that by writing back / invalidating a whole L2 (measured: 2-8x
 // slower kernels), so the partials never live in L2 instead: they are written and read with
-// relaxed agent-scope atomic accesses (write-through stores, L2-bypassing loads), and a
-// workgroup-scope release (s_waitcnt on those stores) orders them before the counter update.
+// relaxed agent-scope atomic accesses (write-through stores, L2-bypassing loads), and every wave
+// waits for the acknowledgement of its stores (an explicit s_waitcnt vmcnt(0)) before the barrier
+// that precedes the counter update.
 // ---------------------------------------------------------------------------------------
 __device__ __forceinline__ void store_partial(float* p, float v, bool coherent) {
   if (coherent) __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
