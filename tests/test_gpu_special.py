@@ -1,6 +1,8 @@
 """Non-finite and extreme values: NaN / inf in the inputs stay in the outputs they belong to,
 fp16 overflow of a sum becomes inf, subnormal inputs are multiplied (not flushed), exactly as the
 CPU oracle (fp16 products, fp32 accumulation) has it."""
+import ctypes
+
 import numpy as np
 import pytest
 import torch
@@ -138,3 +140,38 @@ def test_pitched_entry_point_rejects_bad_pitches(device):
     assert L.fg_gemm_f16_pitched(*args(N - 8)) == capi.FG_ERR_INVALID_ARG      # rows overlap
     assert L.fg_gemm_f16_pitched(*args(N + 4)) == capi.FG_ERR_INVALID_ARG      # not 16-byte rows
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("layout,M,N,K", [(KN, 9, 7168, 2048), (KN, 1, 11008, 8192), (KN, 16, 4096, 4096),
+                                          (NK, 16, 3072, 12288)])
+def test_in_launch_split_k_repeats_bit_for_bit(device, layout, M, N, K):
+    """Every wave's partial has to be in memory before its workgroup arrives at the tile counter;
+    an arrival that overtakes a store shows as a rare wrong sum.  Several hundred back-to-back
+    calls on rotating weights must all give the bits of the two-pass completion (a second kernel
+    sums the same partials in the same order)."""
+    L = capi.lib()
+    p = capi.plan(M, N, K, layout, 0)
+    if p.splitk < 2 or not p.fused:
+        pytest.skip("the library does not split this shape inside the launch")
+    g = torch.Generator(device=device).manual_seed(4242 + N + K)
+    shape = (K, N) if layout == KN else (N, K)
+    Ws = [(torch.randn(shape, device=device, generator=g) * 0.02).half() for _ in range(4)]
+    A = torch.randn((M, K), device=device, generator=g).half()
+    ws = torch.zeros(p.workspace_bytes, dtype=torch.uint8, device=device)
+    two = capi.plan(M, N, K, layout, 0)
+    two.fused = 0
+    refs = []
+    for W in Ws:
+        C = torch.empty((M, N), dtype=torch.half, device=device)
+        capi.check(L.fg_gemm_f16_planned(ptr(A), ptr(W), ptr(C), M, N, K, layout, 0, ctypes.byref(two), ptr(ws),
+                                         ws.numel(), stream_ptr()), "two-pass")
+        refs.append(C)
+    assert_close_f16(refs[0].cpu().numpy(), (A.float() @ (Ws[0].float() if layout == KN else Ws[0].float().t())).cpu().numpy(),
+                     "two-pass reference")
+    C = torch.empty((M, N), dtype=torch.half, device=device)
+    bad = torch.zeros((), dtype=torch.int64, device=device)
+    for i in range(400):
+        capi.check(L.fg_gemm_f16(ptr(A), ptr(Ws[i % 4]), ptr(C), M, N, K, layout, 0, 0, ptr(ws), ws.numel(),
+                                 stream_ptr()), "in-launch")
+        bad += (C.view(torch.int16) != refs[i % 4].view(torch.int16)).sum()
+    assert int(bad.item()) == 0
