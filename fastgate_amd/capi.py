@@ -19,6 +19,8 @@ FG_ERR_ALIGN128 = -2
 FG_ERR_WORKSPACE = -3
 FG_ERR_LAUNCH = -4
 FG_ERR_UNSUPPORTED = -5
+FG_ERR_SCRATCH_LIMIT = -6
+FG_STATIC_SCRATCH_BYTES = 65536 + (8 << 20)
 
 FG_W_KN = 0
 FG_W_NK = 1
@@ -40,6 +42,7 @@ EXPORTS = (
     "fg_gemm_f16",
     "fg_gemm_f16_planned",
     "fg_gemm_f16_pitched",
+    "fg_gemm_f16_static",
     "fg_gemm_f16_bias_act",
     "fg_plan",
     "fg_workspace_bytes",
@@ -106,6 +109,8 @@ def lib() -> ctypes.CDLL:
         L.fg_gemm_f16.argtypes = [vp, vp, vp, ci, ci, ci, ci, ci, ci, vp, sz, vp]
         L.fg_gemm_f16_pitched.restype = ci
         L.fg_gemm_f16_pitched.argtypes = [vp, vp, vp, ci, ci, ci, ci, ci, ci, vp, sz, vp]
+        L.fg_gemm_f16_static.restype = ci
+        L.fg_gemm_f16_static.argtypes = [vp, vp, vp, ci, ci, ci, ci, ci, ci, vp]
         L.fg_gemm_f16_planned.restype = ci
         L.fg_gemm_f16_planned.argtypes = [vp, vp, vp, ci, ci, ci, ci, ci, pp, vp, sz, vp]
         L.fg_gemm_f16_bias_act.restype = ci

@@ -3,10 +3,17 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <atomic>
 #include <cmath>
 #include <cstring>
+#include <mutex>
 
 #include "fg_internal.h"
+
+// Split-K scratch of fg_gemm_f16_static: one copy per GPU, held until the process ends.  The name
+// is a host-side stand-in for the symbol, never a device address: host code reaches the memory
+// only through the per-device pointer that static_scratch() obtains with hipGetSymbolAddress.
+static __device__ __align__(256) unsigned char scratch[FG_STATIC_SCRATCH_BYTES];
 
 namespace fg {
 namespace {
@@ -561,6 +568,31 @@ int run_gemm(const void* A, const void* W, void* C, int M, int N, int K, int acc
   return FG_OK;
 }
 
+// Device address of `scratch` on the current device, resolved once per device (with that device
+// current) and kept.  The first resolution also clears the counter header with a fill kernel on
+// `s`; after that every call leaves the counters at zero by itself.  Returns null on failure.
+constexpr int kMaxDevices = 64;
+void* static_scratch(hipStream_t s) {
+  static std::atomic<void*> ptrs[kMaxDevices];
+  static std::mutex mu;
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+  void* p = ptrs[dev].load(std::memory_order_acquire);
+  if (p != nullptr) return p;
+  std::lock_guard<std::mutex> lock(mu);
+  p = ptrs[dev].load(std::memory_order_acquire);
+  if (p != nullptr) return p;
+  if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || p == nullptr) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  (void)hipGetLastError();
+  launch_fill_zero(p, kWsHeaderBytes, s);
+  if (check_launch() != FG_OK) return nullptr;
+  ptrs[dev].store(p, std::memory_order_release);
+  return p;
+}
+
 bool is_nk(int kernel) {
   return kernel == FG_KERNEL_NK_DOT2 || kernel == FG_KERNEL_NK_MFMA ||
          kernel == FG_KERNEL_NK_MFMA4 ||
@@ -583,6 +615,8 @@ const char* fg_strerror(int status) {
     case FG_ERR_WORKSPACE: return "split-K workspace missing or too small";
     case FG_ERR_LAUNCH: return "HIP kernel launch failed";
     case FG_ERR_UNSUPPORTED: return "plan names a kernel/tile combination that is not built";
+    case FG_ERR_SCRATCH_LIMIT:
+      return "shape needs more split-K scratch than the static buffer of fg_gemm_f16_static holds";
     default: return "unknown fastgate status";
   }
 }
@@ -624,6 +658,22 @@ int fg_gemm_f16(const void* A, const void* W, void* C, int M, int N, int K, int 
     if (st != FG_OK) return st;
   }
   return fg::run_gemm(A, W, C, M, N, K, accumulate, p, ws, ws_bytes,
+                      static_cast<hipStream_t>(stream));
+}
+
+int fg_gemm_f16_static(const void* A, const void* W, void* C, int M, int N, int K, int w_layout,
+                       int accumulate, int splitk, void* stream) {
+  if (A == nullptr || W == nullptr || C == nullptr) return FG_ERR_INVALID_ARG;
+  fg_plan_t p;
+  const int st = fg_plan(M, N, K, w_layout, splitk, &p);
+  if (st != FG_OK) return st;
+  if (p.workspace_bytes > (size_t)FG_STATIC_SCRATCH_BYTES) return FG_ERR_SCRATCH_LIMIT;
+  void* ws = nullptr;
+  if (p.splitk > 1) {
+    ws = fg::static_scratch(static_cast<hipStream_t>(stream));
+    if (ws == nullptr) return FG_ERR_LAUNCH;
+  }
+  return fg::run_gemm(A, W, C, M, N, K, accumulate, p, ws, p.splitk > 1 ? (size_t)FG_STATIC_SCRATCH_BYTES : 0,
                       static_cast<hipStream_t>(stream));
 }
 

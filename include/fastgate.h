@@ -39,7 +39,9 @@ typedef enum fg_status {
   FG_ERR_ALIGN128 = -2,    /* K or N not a multiple of 128 (reference: invalid_argument) */
   FG_ERR_WORKSPACE = -3,   /* split-K requested/needed and workspace missing or small */
   FG_ERR_LAUNCH = -4,      /* HIP reported an error at launch (no device, bad stream) */
-  FG_ERR_UNSUPPORTED = -5  /* plan names a kernel/tile combination that does not exist */
+  FG_ERR_UNSUPPORTED = -5, /* plan names a kernel/tile combination that does not exist */
+  FG_ERR_SCRATCH_LIMIT = -6 /* fg_gemm_f16_static: the shape's split-K partials exceed
+                               FG_STATIC_SCRATCH_BYTES                                   */
 } fg_status;
 
 enum { FG_W_KN = 0, FG_W_NK = 1 };
@@ -113,6 +115,23 @@ typedef struct fg_plan_t {
  */
 int fg_gemm_f16(const void* A, const void* W, void* C, int M, int N, int K, int w_layout,
                 int accumulate, int splitk, void* ws, size_t ws_bytes, void* stream);
+
+/*
+ * fg_gemm_f16 without the workspace arguments, for callers that cannot allocate: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the
+ * reference.  The split-K workspace is a static device array of FG_STATIC_SCRATCH_BYTES (a 64 KiB
+ * counter header + 8 MiB of fp32 partials, twice what the library's own plans need for up to 16
+ * rows) that every GPU the library runs on holds until the process ends; the call allocates and
+ * frees nothing.  A plan that needs more (S*M*N*4 bytes of partials > 8 MiB, e.g. a forced
+ * 16-way split of 16 x 16384 outputs) is rejected with FG_ERR_SCRATCH_LIMIT; plans that do not
+ * split have no limit.  `splitk` as in fg_gemm_f16.  Results are those of fg_gemm_f16, bit for bit.  All calls on one GPU share that GPU's array: calls that overlap in time on one
+ * GPU (two streams, two threads) race, so order them on one stream.  The first call on a device
+ * looks the array's address up and clears its counter header; make that call outside graph
+ * capture, with the device of `stream` current.
+ */
+#define FG_STATIC_SCRATCH_BYTES (65536 + (8 << 20))
+int fg_gemm_f16_static(const void* A, const void* W, void* C, int M, int N, int K, int w_layout,
+                       int accumulate, int splitk, void* stream);
 
 /*
  * fg_gemm_f16 for [K,N] weights whose rows are ldw >= N elements apart (ldw a multiple of 8):

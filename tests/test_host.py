@@ -37,8 +37,8 @@ def test_header_is_plain_c():
 
 
 def test_strerror_covers_every_status():
-    texts = {capi.strerror(s) for s in (0, -1, -2, -3, -4, -5)}
-    assert len(texts) == 6 and all(texts)
+    texts = {capi.strerror(s) for s in (0, -1, -2, -3, -4, -5, -6)}
+    assert len(texts) == 7 and all(texts)
     assert "unknown" in capi.strerror(-99)
     assert "128" in capi.strerror(capi.FG_ERR_ALIGN128)
 
