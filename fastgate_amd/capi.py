@@ -20,22 +20,20 @@ FG_ERR_WORKSPACE = -3
 FG_ERR_LAUNCH = -4
 FG_ERR_UNSUPPORTED = -5
 FG_ERR_SCRATCH_LIMIT = -6
-FG_STATIC_SCRATCH_BYTES = 65536 + (8 << 20)
+FG_STATIC_SCRATCH_BYTES = 65536 + 3145728 + (8 << 20)
 
 FG_W_KN = 0
 FG_W_NK = 1
 
 FG_KERNEL_AUTO = 0
 FG_KERNEL_NK_DOT2 = 1
-FG_KERNEL_NK_MFMA = 2
 FG_KERNEL_KN_DOT2 = 3
 FG_KERNEL_KN_MFMA = 4
 FG_KERNEL_NK_MFMA4 = 5
-FG_KERNEL_NK_MFMA_T = 7
 FG_KERNEL_NK_MFMA_R = 8
 FG_ACT_NONE, FG_ACT_RELU, FG_ACT_GELU, FG_ACT_GELU_TANH, FG_ACT_SILU = range(5)
 ACT_IDS = {"none": 0, "relu": 1, "gelu": 2, "gelu_tanh": 3, "silu": 4}
-KERNEL_NAMES = {1: "nk_dot2", 2: "nk_mfma", 3: "kn_dot2", 4: "kn_mfma", 5: "nk_mfma4", 7: "nk_mfma_t", 8: "nk_mfma_r"}
+KERNEL_NAMES = {1: "nk_dot2", 3: "kn_dot2", 4: "kn_mfma", 5: "nk_mfma4", 8: "nk_mfma_r"}
 
 # Every symbol include/fastgate.h declares.
 EXPORTS = (

@@ -5,6 +5,7 @@
 #include <algorithm>
 #include <atomic>
 #include <cmath>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 
@@ -74,10 +75,6 @@ int finish_plan(int M, int N, int K, fg_plan_t* p) {
     case FG_KERNEL_NK_DOT2:
       if (!nk_dot2_supported(p->m_block, p->tile_n, p->unroll)) return FG_ERR_UNSUPPORTED;
       break;
-    case FG_KERNEL_NK_MFMA:
-      p->m_block = 16;
-      if (!nk_mfma_supported(p->tile_n, p->unroll)) return FG_ERR_UNSUPPORTED;
-      break;
     case FG_KERNEL_NK_MFMA4:
       if (!nk_mfma4_supported(p->m_block, p->tile_n, p->unroll)) return FG_ERR_UNSUPPORTED;
       break;
@@ -98,12 +95,6 @@ int finish_plan(int M, int N, int K, fg_plan_t* p) {
       if ((p->tile_n > 32 || p->tile_n % 16 != 0 || p->m_block == 32) && p->band != 128) return FG_ERR_UNSUPPORTED;
       if (p->m_block == 32 && (p->tile_n % 16 != 0 || p->tile_n > 48)) return FG_ERR_UNSUPPORTED;
       p->unroll = p->band == 512 ? 2 : 1;
-      break;
-    case FG_KERNEL_NK_MFMA_T:
-      if (!nk_mfma_t_supported(p->unroll, p->tile_n)) return FG_ERR_UNSUPPORTED;
-      p->m_block = 16;
-      p->waves = 4;
-      p->splitk = nk_mfma_t_slices(K);  // each wave owns a fixed K range of at most 512
       break;
     case FG_KERNEL_KN_DOT2:
       p->tile_n = 128;
@@ -524,7 +515,25 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
       p->splitk = pick_splitk(tiles, p->waves, items, M, N, K, kCUs);
     }
   }
-  return finish_plan(M, N, K, p);
+  const int st = finish_plan(M, N, K, p);
+  if (st != FG_OK) return st;
+  // In-launch completion through one fixed-point atomic per output element (fused = 2) instead of
+  // partials + arrival counter (fused = 1): one memory round trip after the K loop instead of
+  // three, but S * M * N atomics.  Measured over 11 N x 7 K x 6 M on both layouts (us gained over
+  // the counter protocol): every v_dot2 split 0.5 .. 2.5, every [N,K] split 0.3 .. 1.9; the [K,N]
+  // MFMA kernel with eight waves 0.1 .. 1.7 below 2^18 atomics or from eight splits on (up to 0.9
+  // lost otherwise), with four waves 0.8 .. 2.5 only for deep splits of few elements (1 .. 2.5 lost
+  // otherwise: K = 8192 N = 12288 M = 16, five splits, 38.4 -> 40.5).
+  if (p->splitk > 1 && p->fused == 1 && p->splitk <= kFixMaxSplit && (size_t)M * N <= kWsAccElems) {
+    const size_t atomics = (size_t)p->splitk * M * N;
+    bool atomic = true;
+    if (p->kernel == FG_KERNEL_KN_MFMA) {
+      atomic = p->waves >= 8 ? (atomics < ((size_t)1 << 18) || p->splitk >= 8)
+                             : (atomics < ((size_t)1 << 17) && p->splitk >= 8);
+    }
+    if (atomic) p->fused = 2;
+  }
+  return FG_OK;
 }
 
 int check_launch() { return hipGetLastError() == hipSuccess ? FG_OK : FG_ERR_LAUNCH; }
@@ -546,14 +555,16 @@ int run_gemm(const void* A, const void* W, void* C, int M, int N, int K, int acc
   if (p.splitk > 1) {
     a.ws = reinterpret_cast<float*>(static_cast<unsigned char*>(ws) + kWsHeaderBytes);
     a.counters = p.fused ? static_cast<int*>(ws) : nullptr;
+    if (p.fused == 2) {
+      if (p.splitk > kFixMaxSplit || (size_t)M * N > kWsAccElems) return FG_ERR_UNSUPPORTED;
+      a.accumulate |= kFlagFixSplit;
+    }
   }
   (void)hipGetLastError();
   bool ok = false;
   switch (p.kernel) {
     case FG_KERNEL_NK_DOT2: ok = launch_nk_dot2(p, a, s); break;
-    case FG_KERNEL_NK_MFMA: ok = launch_nk_mfma(p, a, s); break;
     case FG_KERNEL_NK_MFMA4: ok = launch_nk_mfma4(p, a, s); break;
-    case FG_KERNEL_NK_MFMA_T: ok = launch_nk_mfma_t(p, a, s); break;
     case FG_KERNEL_NK_MFMA_R: ok = launch_nk_mfma_r(p, a, s); break;
     case FG_KERNEL_KN_DOT2: ok = launch_kn_dot2(p, a, s); break;
     case FG_KERNEL_KN_MFMA: ok = launch_kn_mfma(p, a, s); break;
@@ -594,9 +605,7 @@ void* static_scratch(hipStream_t s) {
 }
 
 bool is_nk(int kernel) {
-  return kernel == FG_KERNEL_NK_DOT2 || kernel == FG_KERNEL_NK_MFMA ||
-         kernel == FG_KERNEL_NK_MFMA4 ||
-         kernel == FG_KERNEL_NK_MFMA_T || kernel == FG_KERNEL_NK_MFMA_R;
+  return kernel == FG_KERNEL_NK_DOT2 || kernel == FG_KERNEL_NK_MFMA4 || kernel == FG_KERNEL_NK_MFMA_R;
 }
 bool is_kn(int kernel) { return kernel == FG_KERNEL_KN_DOT2 || kernel == FG_KERNEL_KN_MFMA; }
 

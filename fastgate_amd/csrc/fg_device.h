@@ -190,6 +190,94 @@ __device__ __forceinline__ bool splitk_last_arriver(int* counter, int S) {
   return s_last != 0;
 }
 
+// ---------------------------------------------------------------------------------------
+// Split-K completion in one memory round trip.  Every output element owns one 64-bit word
+// (zero between calls).  A workgroup adds its fp32 partial, converted to fixed point, together
+// with an arrival count in the low bits, using one relaxed agent-scope atomic add that returns
+// the previous word.  The thread whose add returns S - 1 previous arrivals holds, in
+// (previous + own), the complete sum of that element: it writes C and puts the word back to
+// zero.  Integer addition is associative, so the sum does not depend on arrival order; all
+// communication goes through the one atomic word, so no ordering between different locations is
+// needed (no fence, no write-through wait, no counter, no barrier), and different elements of a
+// tile may be completed by different workgroups.
+//   word = value (54 bits, two's complement, units of 2^-28) | poisoned arrivals (5) | arrivals (5)
+// A partial that fixed point cannot hold (NaN, infinite, or |p| >= 2^20, sixteen times the fp16
+// range) arrives "poisoned": value 0, its class (NaN, +overflow, -overflow) counted in a second
+// word of the element, written before the arrival with release / acquire fences around the
+// pair (that path alone pays for agent-scope fences).
+// ---------------------------------------------------------------------------------------
+constexpr float kFixLimit = 1048576.f;  // 2^20
+constexpr uint32_t kFixNaN = 1u, kFixPos = 1u << 8, kFixNeg = 1u << 16;
+
+// Fixed-point image of p (|p| < 2^20) in units of 2^-28, rounded to nearest: exact for every fp32
+// value of magnitude 2^-4 or more, off by at most 2^-29 below (the smallest fp16 step is 2^-24).
+__device__ __forceinline__ int64_t fix_from_float(float p) {
+  const float scaled = p * 16.f;                         // exact
+  const float hi = __builtin_floorf(scaled);             // |hi| <= 2^24, an integer
+  const float lo = __builtin_rintf((scaled - hi) * 16777216.f);  // [0, 2^24], exact difference
+  return ((int64_t)(int)hi << 24) + (int64_t)(int)lo;
+}
+// Correctly rounded fp32 value of v * 2^-28 (|v| < 2^53).
+__device__ __forceinline__ float fix_to_float(int64_t v) {
+  const double d = (double)(int)(v >> 24) * 16777216.0 + (double)(int)(v & 0xFFFFFF);
+  return (float)d * 3.7252902984619140625e-09f;          // 2^-28
+}
+__device__ __forceinline__ uint32_t fix_class(float p) {
+  if (__builtin_fabsf(p) < kFixLimit) return 0u;
+  return p != p ? kFixNaN : (p > 0.f ? kFixPos : kFixNeg);
+}
+// Word a partial arrives with.
+__device__ __forceinline__ uint64_t fix_word(float p, uint32_t cls) {
+  if (cls) return (1ull << 5) | 1ull;
+  return ((uint64_t)fix_from_float(p) << 10) | 1ull;
+}
+// Sum a complete word stands for; `cls` is the element's class word (read only when poisoned).
+__device__ __forceinline__ float fix_total(uint64_t word, uint32_t cls) {
+  if ((word >> 5) & 31u) {
+    const bool nan = (cls & 0xFFu) != 0, pos = (cls & 0xFF00u) != 0, neg = (cls & 0xFF0000u) != 0;
+    if (nan || (pos && neg)) return __builtin_nanf("");
+    return pos ? __builtin_inff() : -__builtin_inff();
+  }
+  return fix_to_float((int64_t)word >> 10);
+}
+
+// NB elements of one thread: partial p[i] of output element idx[i] (= m * N + n) arrives; the
+// atomics of the batch are issued back to back before the first result is looked at.
+template <int NB>
+__device__ __forceinline__ void fix_arrive(uint64_t* acc, uint32_t* clsw, const size_t (&idx)[NB],
+                                           const float (&p)[NB], const bool (&valid)[NB], int S,
+                                           half_t* C, int N, const void* bias, int flags) {
+  uint64_t own[NB], old[NB];
+#pragma unroll
+  for (int i = 0; i < NB; ++i) {
+    const uint32_t cls = fix_class(p[i]);
+    own[i] = fix_word(p[i], cls);
+    if (valid[i] && cls) {
+      __hip_atomic_fetch_add(clsw + idx[i], cls, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < NB; ++i)
+    old[i] = valid[i] ? __hip_atomic_fetch_add(acc + idx[i], own[i], __ATOMIC_RELAXED,
+                                               __HIP_MEMORY_SCOPE_AGENT)
+                      : 0ull;
+#pragma unroll
+  for (int i = 0; i < NB; ++i) {
+    if (!valid[i] || (int)(old[i] & 31u) != S - 1) continue;
+    const uint64_t word = old[i] + own[i];
+    uint32_t cls = 0;
+    if ((word >> 5) & 31u) {
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+      cls = __hip_atomic_load(clsw + idx[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(clsw + idx[i], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __hip_atomic_store(acc + idx[i], 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    half_t* c = C + idx[i];
+    *c = finish_value(fix_total(word, cls), c, (int)(idx[i] % (size_t)N), bias, flags);
+  }
+}
+
 // Σ_z part[z][off..off+3] in ascending z.  The loads of a batch are all issued before the first
 // add: one memory round trip per batch instead of one per partial (a plain `for z` loop compiles
 // to load, wait, add).  Slots past S re-read the last partial and contribute +0, which leaves
@@ -251,6 +339,22 @@ __device__ __forceinline__ void splitk_reduce_tile(const float* part, half_t* C,
   }
 }
 
+// One element's partial of a split launch: to its slot of the workspace (second kernel or counter
+// protocol), or straight into the element's accumulator word (atomic protocol).
+__device__ __forceinline__ void publish_partial(float* ws, int* counters, half_t* C, int M, int N,
+                                                int mg, int n, float sum, int flags, const void* bias) {
+  if (flags & kFlagFixSplit) {
+    uint64_t* facc = reinterpret_cast<uint64_t*>(reinterpret_cast<unsigned char*>(counters) + kWsCounterBytes);
+    uint32_t* fcls = reinterpret_cast<uint32_t*>(facc + kWsAccElems);
+    const size_t idx[1] = {(size_t)mg * N + n};
+    const float part[1] = {sum};
+    const bool valid[1] = {true};
+    fix_arrive<1>(facc, fcls, idx, part, valid, gridDim.z, C, N, bias, flags);
+  } else {
+    store_partial(ws + ((size_t)blockIdx.z * M + mg) * N + n, sum, counters != nullptr);
+  }
+}
+
 // Shared tail of every GEMM kernel: the workgroup has stored its fp32 partial of the tile
 // (m0.., n0..) when gridDim.z > 1; with counters it also completes the split-K sum in place,
 // without counters a second kernel does.
@@ -259,7 +363,7 @@ __device__ __forceinline__ void finish_splitk(float* ws, int* counters, half_t* 
                                               int m0, int n0, int flags, const void* bias,
                                               int tile_x = -1) {
   if (tile_x < 0) tile_x = blockIdx.x;
-  if (gridDim.z > 1 && counters != nullptr) {
+  if (gridDim.z > 1 && counters != nullptr && !(flags & kFlagFixSplit)) {
     if (splitk_last_arriver(counters + blockIdx.y * gridDim.x + tile_x, gridDim.z))
       splitk_reduce_tile<DEEP>(ws, C, gridDim.z, M, N, m0, MROWS, n0, NCOLS, flags, bias);
   }

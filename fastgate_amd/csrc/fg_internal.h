@@ -26,17 +26,12 @@ struct GemmArgs {
 
 // Tile sets that exist as instantiations (the planner and the validators share these).
 bool nk_dot2_supported(int m_block, int tile_n, int unroll);
-bool nk_mfma_supported(int tile_n, int unroll);
 bool nk_mfma4_supported(int m_block, int tile_n, int unroll);
-bool nk_mfma_t_supported(int rows, int tile_n);
-int nk_mfma_t_slices(int K);
 bool kn_dot2_supported(int m_block, int unroll);
 bool kn_mfma_supported(int unroll);
 
 bool launch_nk_dot2(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
-bool launch_nk_mfma(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
 bool launch_nk_mfma4(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
-bool launch_nk_mfma_t(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
 bool launch_nk_mfma_r(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
 bool launch_kn_dot2(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
 bool launch_kn_mfma(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
@@ -62,8 +57,7 @@ void launch_dequant_i32_f16(const int32_t* acc, const void* scale, float x_scale
                             int N, hipStream_t s);
 
 // Split-K workspace: a header of arrival counters (zero between calls), then the partials.
-constexpr size_t kWsHeaderBytes = 65536;
-constexpr int kWsMaxTiles = (int)(kWsHeaderBytes / sizeof(int));
+constexpr int kWsMaxTiles = (int)(kWsCounterBytes / sizeof(int));
 void launch_fill_zero(void* p, size_t bytes, hipStream_t s);
 
 constexpr int kStreamReadBlocks = 2048;

@@ -104,6 +104,31 @@ __global__ __launch_bounds__(64 * NW) void kn_mfma_kernel(const half_t* __restri
 #pragma unroll
     for (int i = 0; i < 8; ++i) red[wave][4 * g + r][8 * j + i] = acc[i][r];
   __syncthreads();
+  if (gridDim.z > 1 && (flags & kFlagFixSplit)) {
+    // one atomic per output element, consecutive lanes on consecutive columns
+    uint64_t* facc = reinterpret_cast<uint64_t*>(reinterpret_cast<unsigned char*>(counters) + kWsCounterBytes);
+    uint32_t* fcls = reinterpret_cast<uint32_t*>(facc + kWsAccElems);
+    const int rows = M - m0 < 16 ? M - m0 : 16;
+    // up to eight elements a thread (16 rows on four waves), their atomics in flight together
+    constexpr int NB = NW >= 8 ? 4 : 8;
+    for (int base = 0; base < rows * 128; base += NB * blockDim.x) {
+      size_t idx[NB];
+      float part[NB];
+      bool valid[NB];
+#pragma unroll
+      for (int i = 0; i < NB; ++i) {
+        const int e = base + i * (int)blockDim.x + (int)threadIdx.x;
+        valid[i] = e < rows * 128;
+        const int m = valid[i] ? e >> 7 : 0, c = e & 127;
+        float sum = 0.f;
+        for (int w = 0; w < nw; ++w) sum += red[w][m][c];
+        part[i] = sum;
+        idx[i] = (size_t)(m0 + m) * N + n0 + c;
+      }
+      fix_arrive<NB>(facc, fcls, idx, part, valid, gridDim.z, C, N, bias, flags);
+    }
+    return;
+  }
   // 16 x 128 outputs, 8 consecutive columns per thread.
   for (int e = threadIdx.x; e < 256; e += blockDim.x) {
     const int m = e >> 4, c0 = (e & 15) * 8;
@@ -200,6 +225,29 @@ __global__ __launch_bounds__(64 * NW) void kn_dot2_kernel(const half_t* __restri
 #pragma unroll
     for (int i = 0; i < 8; ++i) red[wave * 4 + g][m][8 * j + i] = acc[i][m];
   __syncthreads();
+  if (gridDim.z > 1 && (flags & kFlagFixSplit)) {
+    uint64_t* facc = reinterpret_cast<uint64_t*>(reinterpret_cast<unsigned char*>(counters) + kWsCounterBytes);
+    uint32_t* fcls = reinterpret_cast<uint32_t*>(facc + kWsAccElems);
+    const int rows = M - m0 < MB ? M - m0 : MB;
+    constexpr int NB = MB >= 4 ? 2 : 1;
+    for (int base = 0; base < rows * 128; base += NB * blockDim.x) {
+      size_t idx[NB];
+      float part[NB];
+      bool valid[NB];
+#pragma unroll
+      for (int i = 0; i < NB; ++i) {
+        const int e = base + i * (int)blockDim.x + (int)threadIdx.x;
+        valid[i] = e < rows * 128;
+        const int m = valid[i] ? e >> 7 : 0, nn = e & 127;
+        float sum = 0.f;
+        for (int p = 0; p < nw * 4; ++p) sum += red[p][m][nn];
+        part[i] = sum;
+        idx[i] = (size_t)(m0 + m) * N + n0 + nn;
+      }
+      fix_arrive<NB>(facc, fcls, idx, part, valid, gridDim.z, C, N, bias, flags);
+    }
+    return;
+  }
   for (int e = threadIdx.x; e < MB * 128; e += blockDim.x) {
     const int m = e >> 7, nn = e & 127;
     float sum = 0.f;

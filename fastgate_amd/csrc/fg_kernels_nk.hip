@@ -91,91 +91,11 @@ __global__ __launch_bounds__(256) void nk_dot2_kernel(const half_t* __restrict__
         half_t* c = C + (size_t)mg * N + n;
         *c = finish_value(sum, c, n, bias, flags);
       } else {
-        store_partial(ws + ((size_t)blockIdx.z * M + mg) * N + n, sum, counters != nullptr);
+        publish_partial(ws, counters, C, M, N, mg, n, sum, flags, bias);
       }
     }
   }
   finish_splitk<MB, RN>(ws, counters, C, M, N, m0, n0, flags, bias);
-}
-
-// ---------------------------------------------------------------------------------------
-// MFMA 16x16x32 kernel.  Workgroup tile = 16*TNW columns of C x 16 rows of A.  A 16-byte
-// weight load of lane l (j = l%16, g = l/16) lands directly in the B-operand layout of
-// v_mfma_f32_16x16x32_f16: column n0+16t+j, k = 32*unit + 8g .. +7; the matching A operand is
-// row m0+j at the same k.  One MFMA consumes one load instruction of the wave, but that
-// instruction touches 16 rows x 64 bytes.
-// ---------------------------------------------------------------------------------------
-template <int TNW, int U, bool STREAM>
-__global__ __launch_bounds__(256) void nk_mfma_kernel(const half_t* __restrict__ A,
-                                                      const half_t* __restrict__ W,
-                                                      half_t* __restrict__ C,
-                                                      float* __restrict__ ws, int* counters, int M,
-                                                      int N, int K, int flags, const void* bias) {
-  __shared__ float red[4][TNW][256];
-  const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
-  const int nw = blockDim.x >> 6;
-  const int j = lane & 15, g = lane >> 4;
-  const int n0 = blockIdx.x * (16 * TNW);
-  const int m0 = blockIdx.y * 16;
-  const int slots = nw * gridDim.z;
-  const int slot = blockIdx.z * nw + wave;
-  const int nunits = K >> 5;
-
-  float4_t acc[TNW];
-#pragma unroll
-  for (int t = 0; t < TNW; ++t) acc[t] = float4_t{0.f, 0.f, 0.f, 0.f};
-
-  const bool arow = (m0 + j) < M;
-  const half_t* Ap = A + (size_t)(m0 + (arow ? j : 0)) * K + g * 8;
-  const half_t* Wp = W + (size_t)(n0 + j) * K + g * 8;
-  const u32x4 zero = {0u, 0u, 0u, 0u};
-
-  const int nsteps = (nunits + slots * U - 1) / (slots * U);
-  int step = stagger_start(nsteps, flags);
-  for (int it = 0; it < nsteps; ++it) {
-    const int u0 = (step * slots + slot) * U;
-    step = step + 1 == nsteps ? 0 : step + 1;
-    u32x4 b[U][TNW];
-    u32x4 a[U];
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int unit = u0 + u;
-      const bool ok = unit < nunits;
-#pragma unroll
-      for (int t = 0; t < TNW; ++t)
-        b[u][t] = ok ? load16<STREAM>(Wp + (size_t)t * 16 * K + (size_t)unit * 32) : zero;
-      a[u] = (ok && arow) ? load16<false>(Ap + (size_t)unit * 32) : zero;
-    }
-#pragma unroll
-    for (int u = 0; u < U; ++u)
-#pragma unroll
-      for (int t = 0; t < TNW; ++t)
-        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(a[u]), as_half8(b[u][t]), acc[t],
-                                                        0, 0, 0);
-  }
-
-  // acc[t][r] = D[m = 4g + r][n = j]
-#pragma unroll
-  for (int t = 0; t < TNW; ++t)
-#pragma unroll
-    for (int r = 0; r < 4; ++r) red[wave][t][(4 * g + r) * 16 + j] = acc[t][r];
-  __syncthreads();
-  for (int e = threadIdx.x; e < TNW * 256; e += blockDim.x) {
-    const int t = e >> 8, m = (e >> 4) & 15, nn = e & 15;
-    float sum = 0.f;
-    for (int w = 0; w < nw; ++w) sum += red[w][t][m * 16 + nn];
-    const int mg = m0 + m, n = n0 + t * 16 + nn;
-    if (mg < M) {
-      if (gridDim.z == 1) {
-        half_t* c = C + (size_t)mg * N + n;
-        *c = finish_value(sum, c, n, bias, flags);
-      } else {
-        store_partial(ws + ((size_t)blockIdx.z * M + mg) * N + n, sum, counters != nullptr);
-      }
-    }
-  }
-  finish_splitk<16, 16 * TNW>(ws, counters, C, M, N, m0, n0, flags, bias);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -278,117 +198,11 @@ __global__ __launch_bounds__(256) void nk_mfma4_kernel(const half_t* __restrict_
         half_t* c = C + (size_t)mg * N + n;
         *c = finish_value(sum, c, n, bias, flags);
       } else {
-        store_partial(ws + ((size_t)blockIdx.z * M + mg) * N + n, sum, counters != nullptr);
+        publish_partial(ws, counters, C, M, N, mg, n, sum, flags, bias);
       }
     }
   }
   finish_splitk<4 * MG, 4 * R4>(ws, counters, C, M, N, m0, n0, flags, bias);
-}
-
-// ---------------------------------------------------------------------------------------
-// MFMA 16x16x32 kernel with row-friendly loads ("transposing" variant) for M = 5..16.
-// The 16x16x32 B operand wants 16 rows x 64 B per instruction, which is the worst shape for
-// HBM.  Here a wave instead loads ROWS rows x 1 KB (one row per instruction, 64 lanes x 16 B
-// along K), parks them in a wave-private LDS buffer and reads them back in operand order
-// (lane (j,g): row j, 16-byte piece 4u+g); rows are padded to 1040 B so both directions are
-// free of bank conflicts.  No workgroup barrier is involved.
-// Each wave owns a fixed K range of ur*32 positions (ur <= 16) for the whole kernel, so its
-// A operands are loaded once into 16 registers-quads and reused for every row tile: the A
-// traffic is 1/(ROWS*T) of the weight traffic instead of 1/1.  The wave walks T tiles of ROWS
-// rows, next tile's loads in flight during the current tile's LDS round trip and MFMAs; the
-// 4 waves of a workgroup (adjacent K ranges) meet in LDS at the end, the gridDim.z workgroups
-// of a tile in the split-K workspace.  ROWS = 8 leaves half of each MFMA idle (it is nowhere
-// near the limit) in exchange for half as many rows in flight.
-// ---------------------------------------------------------------------------------------
-template <int ROWS, int T, bool FULL, bool STREAM>
-__global__ __launch_bounds__(256) void nk_mfma_t_kernel(const half_t* __restrict__ A,
-                                                        const half_t* __restrict__ W,
-                                                        half_t* __restrict__ C,
-                                                        float* __restrict__ ws, int* counters, int M,
-                                                        int N, int K, int flags, int ur, const void* bias) {
-  // FULL: every wave range is complete (ur == 16 and K a multiple of 2048), no K masks needed.
-  constexpr int RS = 1040;  // LDS bytes per staged row: 1 KB + 16 B
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
-  const int j = lane & 15, g = lane >> 4;
-  const int n0 = blockIdx.x * (ROWS * T);
-  const int m0 = blockIdx.y * 16;
-  const int nunits = K >> 5;
-  if (FULL) ur = 16;
-  const int u_lo = (blockIdx.z * 4 + wave) * ur;  // first 32-wide K unit of this wave
-  unsigned char* wb = smem + wave * (ROWS * RS);
-  const u32x4 zero = {0u, 0u, 0u, 0u};
-
-  // lane l streams the 16-byte piece l of the wave's K range, for every row; first tile first
-  const bool lane_ok = FULL || (lane < 4 * ur && (u_lo * 4 + lane) < nunits * 4);
-  const half_t* Wp = W + (size_t)n0 * K + (size_t)u_lo * 32 + lane * 8;
-  u32x4 wcur[ROWS], wnxt[ROWS];
-#pragma unroll
-  for (int r = 0; r < ROWS; ++r) wcur[r] = lane_ok ? load16<STREAM>(Wp + (size_t)r * K) : zero;
-
-  // A operands of the whole K range: a[u] = A[m0+j][32*(u_lo+u) + 8g .. +7], zero where the
-  // row or the unit does not exist (the staged weights of such units are zero as well)
-  u32x4 a[16];
-  const bool arow = (m0 + j) < M;
-  const half_t* Ap = A + (size_t)(m0 + (arow ? j : 0)) * K + (size_t)u_lo * 32 + g * 8;
-#pragma unroll
-  for (int u = 0; u < 16; ++u)
-    a[u] = (arow && (FULL || (u < ur && (u_lo + u) < nunits))) ? load16<false>(Ap + u * 32) : zero;
-
-  float4_t acc[T];
-#pragma unroll
-  for (int t = 0; t < T; ++t) {
-    acc[t] = float4_t{0.f, 0.f, 0.f, 0.f};
-    if (t + 1 < T) {
-#pragma unroll
-      for (int r = 0; r < ROWS; ++r)
-        wnxt[r] = lane_ok ? load16<STREAM>(Wp + (size_t)((t + 1) * ROWS + r) * K) : zero;
-    }
-#pragma unroll
-    for (int r = 0; r < ROWS; ++r) *reinterpret_cast<u32x4*>(wb + r * RS + lane * 16) = wcur[r];
-    wave_lds_sync();
-    u32x4 b[16];
-#pragma unroll
-    for (int u = 0; u < 16; ++u) {
-      b[u] = zero;
-      if (ROWS == 16 || j < ROWS) b[u] = *reinterpret_cast<const u32x4*>(wb + j * RS + (4 * u + g) * 16);
-    }
-#pragma unroll
-    for (int u = 0; u < 16; ++u)
-      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(a[u]), as_half8(b[u]), acc[t], 0, 0, 0);
-    wave_lds_sync();
-    if (t + 1 < T) {
-#pragma unroll
-      for (int r = 0; r < ROWS; ++r) wcur[r] = wnxt[r];
-    }
-  }
-
-  // acc[t][r] = D[m = 4g + r][row j of tile t]; the 4 waves' partials meet in LDS
-  __syncthreads();
-  float(*red)[T][16 * ROWS] = reinterpret_cast<float(*)[T][16 * ROWS]>(smem);
-  if (j < ROWS) {
-#pragma unroll
-    for (int t = 0; t < T; ++t)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) red[wave][t][(4 * g + r) * ROWS + j] = acc[t][r];
-  }
-  __syncthreads();
-  for (int e = threadIdx.x; e < T * 16 * ROWS; e += 256) {
-    const int m = e / (T * ROWS), c = e % (T * ROWS), t = c / ROWS, jj = c % ROWS;
-    float sum = red[0][t][m * ROWS + jj] + red[1][t][m * ROWS + jj] + red[2][t][m * ROWS + jj] +
-                red[3][t][m * ROWS + jj];
-    const int mg = m0 + m, n = n0 + c;
-    if (mg < M) {
-      if (gridDim.z == 1) {
-        half_t* cp = C + (size_t)mg * N + n;
-        *cp = finish_value(sum, cp, n, bias, flags);
-      } else {
-        store_partial(ws + ((size_t)blockIdx.z * M + mg) * N + n, sum, counters != nullptr);
-      }
-    }
-  }
-  finish_splitk<16, ROWS * T>(ws, counters, C, M, N, m0, n0, flags, bias);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -535,7 +349,7 @@ __global__ __launch_bounds__(64 * NW) void nk_mfma_r_kernel(const half_t* __rest
         half_t* cp = C + (size_t)mg * N + n;
         *cp = finish_value(sum, cp, n, bias, flags);
       } else {
-        store_partial(ws + ((size_t)blockIdx.z * M + mg) * N + n, sum, counters != nullptr);
+        publish_partial(ws, counters, C, M, N, mg, n, sum, flags, bias);
       }
     }
   }
@@ -556,10 +370,6 @@ bool nk_dot2_supported(int mb, int rn, int u) {
   const bool rn_ok = rn == 4 || rn == 8 || rn == 16;
   const bool u_ok = u == 1 || u == 2 || u == 4;
   return mb_ok && rn_ok && u_ok && mb * rn <= 64 && rn * u <= 32;
-}
-
-bool nk_mfma_supported(int tile_n, int u) {
-  return (tile_n == 16 || tile_n == 32) && (u == 1 || u == 2 || u == 4 || u == 8);
 }
 
 template <int MB, int RN, int U>
@@ -602,31 +412,6 @@ bool launch_nk_dot2(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
     case 2: return nk_dot2_rn<2>(p, a, s);
     case 4: return nk_dot2_rn<4>(p, a, s);
     case 8: return nk_dot2_rn<8>(p, a, s);
-    default: return false;
-  }
-}
-
-template <int TNW, int U>
-static void nk_mfma_go(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
-  if (p.stream_w) FG_LAUNCH((nk_mfma_kernel<TNW, U, true>), p, a, s);
-  else FG_LAUNCH((nk_mfma_kernel<TNW, U, false>), p, a, s);
-}
-
-template <int TNW>
-static bool nk_mfma_u(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
-  switch (p.unroll) {
-    case 1: nk_mfma_go<TNW, 1>(p, a, s); return true;
-    case 2: nk_mfma_go<TNW, 2>(p, a, s); return true;
-    case 4: nk_mfma_go<TNW, 4>(p, a, s); return true;
-    case 8: nk_mfma_go<TNW, 8>(p, a, s); return true;
-    default: return false;
-  }
-}
-
-bool launch_nk_mfma(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
-  switch (p.tile_n) {
-    case 16: return nk_mfma_u<1>(p, a, s);
-    case 32: return nk_mfma_u<2>(p, a, s);
     default: return false;
   }
 }
@@ -686,63 +471,6 @@ bool launch_nk_mfma4(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
 }
 
 // Transposing variant: unroll = rows per tile (8 or 16), tile_n = rows * T with T in {2,4,8}.
-bool nk_mfma_t_supported(int rows, int tile_n) {
-  if (rows != 8 && rows != 16) return false;
-  const int t = tile_n / rows;
-  return tile_n % rows == 0 && (t == 2 || t == 4 || t == 8);
-}
-
-int nk_mfma_t_slices(int K) { return ((K >> 5) + 63) / 64; }  // workgroups along K (4 waves x <=16 units)
-
-template <int ROWS, int T, bool FULL, bool STREAM>
-static void nk_mfma_t_launch(const fg_plan_t& p, const GemmArgs& a, hipStream_t s, int ur) {
-  constexpr unsigned lds = 4 * ROWS * 1040;
-  static bool raised = false;  // more than 64 KB of LDS per workgroup has to be asked for once
-  if (!raised) {
-    (void)hipFuncSetAttribute(
-        reinterpret_cast<const void*>(&nk_mfma_t_kernel<ROWS, T, FULL, STREAM>),
-        hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-    raised = true;
-  }
-  hipLaunchKernelGGL((nk_mfma_t_kernel<ROWS, T, FULL, STREAM>),
-                     dim3(p.grid_x, p.grid_y, p.grid_z), dim3(256), lds, s,
-                     static_cast<const half_t*>(a.A), static_cast<const half_t*>(a.W),
-                     static_cast<half_t*>(a.C), a.ws, a.counters, a.M, a.N, a.K, a.accumulate, ur, a.bias);
-}
-
-template <int ROWS, int T>
-static void nk_mfma_t_go(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
-  const int nunits = a.K >> 5;
-  const int ur = (nunits + 4 * p.grid_z - 1) / (4 * p.grid_z);  // K units per wave, <= 16
-  const bool full = ur == 16 && nunits == 64 * p.grid_z;
-  if (full) {
-    if (p.stream_w) nk_mfma_t_launch<ROWS, T, true, true>(p, a, s, ur);
-    else nk_mfma_t_launch<ROWS, T, true, false>(p, a, s, ur);
-  } else {
-    if (p.stream_w) nk_mfma_t_launch<ROWS, T, false, true>(p, a, s, ur);
-    else nk_mfma_t_launch<ROWS, T, false, false>(p, a, s, ur);
-  }
-}
-
-template <int ROWS>
-static bool nk_mfma_t_t(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
-  switch (p.tile_n / ROWS) {
-    case 2: nk_mfma_t_go<ROWS, 2>(p, a, s); return true;
-    case 4: nk_mfma_t_go<ROWS, 4>(p, a, s); return true;
-    case 8: nk_mfma_t_go<ROWS, 8>(p, a, s); return true;
-    default: return false;
-  }
-}
-
-bool launch_nk_mfma_t(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
-  if (p.block != 256 || p.grid_z != nk_mfma_t_slices(a.K)) return false;
-  switch (p.unroll) {
-    case 8: return nk_mfma_t_t<8>(p, a, s);
-    case 16: return nk_mfma_t_t<16>(p, a, s);
-    default: return false;
-  }
-}
-
 template <int AROWS, int BAND, int CB>
 static void nk_mfma_r_go(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
   const int slots = p.waves * p.grid_z;

@@ -50,13 +50,9 @@ enum { FG_W_KN = 0, FG_W_NK = 1 };
 enum {
   FG_KERNEL_AUTO = 0,
   FG_KERNEL_NK_DOT2 = 1, /* [N,K] weights, lanes along K, v_dot2_f32_f16                */
-  FG_KERNEL_NK_MFMA = 2, /* [N,K] weights, v_mfma_f32_16x16x32_f16, 16 rows of A a block */
   FG_KERNEL_KN_DOT2 = 3, /* [K,N] weights, 8x8 register transpose + v_dot2_f32_f16       */
   FG_KERNEL_KN_MFMA = 4, /* [K,N] weights, 8x8 register transpose + MFMA                 */
   FG_KERNEL_NK_MFMA4 = 5, /* [N,K] weights, v_mfma_f32_4x4x4_16B_f16: 4 rows x 256 B a load */
-  FG_KERNEL_NK_MFMA_T = 7, /* [N,K] weights, 16x16x32 MFMA fed through a wave-private LDS
-                              transpose: loads are `unroll` (8/16) rows x 1 KB, every wave keeps
-                              the A operands of its fixed K range in registers               */
   FG_KERNEL_NK_MFMA_R = 8  /* [N,K] weights, 16x16x32 MFMA, 16- to 64-column tiles, weights AND
                               activations loaded as contiguous row pieces and transposed in
                               wave-private LDS; fills the chip without split-K                */
@@ -72,9 +68,15 @@ typedef struct fg_plan_t {
   int splitk;   /* S >= 1: K is divided over S workgroups per output tile; S > 1 writes
                    fp32 partials [S,M,N] to the workspace; they are summed in ascending
                    order of S, so results are reproducible (no data atomics)          */
-  int fused;    /* with S > 1: 1 = the workgroup that finishes a tile last sums the
-                   partials in the same launch (one counter atomic per workgroup),
-                   0 = a second kernel does                                            */
+  int fused;    /* with S > 1, how the split completes: 0 = a second kernel sums the partials;
+                   1 = the workgroup that finishes a tile last sums them in the same launch
+                   (one counter atomic per workgroup); 2 = every workgroup adds its partial,
+                   in 2^-28 fixed point, to the element's 64-bit word of the workspace header
+                   with one atomic, and the arrival that completes an element writes it (no
+                   partials in memory; S <= 31, M*N <= 262144; a partial that is not finite
+                   or beyond +-2^20 counts as overflow of its sign).  0 and 1 sum in ascending
+                   order of S in fp32, 2 sums exactly: each is reproducible run to run, the
+                   two families may differ in the last bit                             */
   int tile_n;   /* output columns per workgroup; FG_KERNEL_NK_MFMA_R takes 16, 32, 48, 64 or,
                    with band = 128, 8 waves and no split, any divisor of N from 17 to 47  */
   int m_block;  /* rows of A per workgroup (grid.y = ceil(M / m_block))               */
@@ -98,8 +100,9 @@ typedef struct fg_plan_t {
  *           no (or too small a) workspace the call runs unsplit instead of failing; a forced
  *           S > 1 without workspace is FG_ERR_WORKSPACE.
  *   ws      device scratch of at least fg_workspace_bytes() bytes when the plan's
- *           splitk > 1, else may be NULL.  Its first fg_workspace_header_bytes() bytes hold
- *           arrival counters: zero them once with fg_workspace_init() (or allocate zeroed
+ *           splitk > 1, else may be NULL.  Its first fg_workspace_header_bytes() bytes (64 KiB of
+ *           arrival counters, then 3 MiB of per-element accumulator words) must be zero before
+ *           the first call: zero them once with fg_workspace_init() (or allocate zeroed
  *           memory); every call leaves them zero again.  Calls that share a workspace must
  *           be ordered on one stream.
  * Services, with w_layout = FG_W_KN: edgemm_m8n128k64x4 (backend/cuda/hk/edgemm.cu:102-156),
@@ -119,9 +122,9 @@ int fg_gemm_f16(const void* A, const void* W, void* C, int M, int N, int K, int 
 /*
  * fg_gemm_f16 without the workspace arguments, for callers that cannot allocate: code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the
- * reference.  The split-K workspace is a static device array of FG_STATIC_SCRATCH_BYTES (a 64 KiB
- * counter header + 8 MiB of fp32 partials, twice what the library's own plans need for up to 16
- * rows) that every GPU the library runs on holds until the process ends; the call allocates and
+ * reference.  The split-K workspace is a static device array of FG_STATIC_SCRATCH_BYTES (the
+ * workspace header of fg_workspace_header_bytes() + 8 MiB of fp32 partials, twice what the
+ * library's own plans need for up to 16 rows) that every GPU the library runs on holds until the process ends; the call allocates and
  * frees nothing.  A plan that needs more (S*M*N*4 bytes of partials > 8 MiB, e.g. a forced
  * 16-way split of 16 x 16384 outputs) is rejected with FG_ERR_SCRATCH_LIMIT; plans that do not
  * split have no limit.  `splitk` as in fg_gemm_f16.  Results are those of fg_gemm_f16, bit for bit.  All calls on one GPU share that GPU's array: calls that overlap in time on one
@@ -129,7 +132,7 @@ int fg_gemm_f16(const void* A, const void* W, void* C, int M, int N, int K, int 
  * looks the array's address up and clears its counter header; make that call outside graph
  * capture, with the device of `stream` current.
  */
-#define FG_STATIC_SCRATCH_BYTES (65536 + (8 << 20))
+#define FG_STATIC_SCRATCH_BYTES (65536 + 3145728 + (8 << 20))
 int fg_gemm_f16_static(const void* A, const void* W, void* C, int M, int N, int K, int w_layout,
                        int accumulate, int splitk, void* stream);
 

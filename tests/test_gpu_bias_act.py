@@ -38,9 +38,7 @@ def _bias_act(A, W, bias, act, layout, device, plan=None, splitk=0):
 def _plans():
     return [
         ("nk_dot2", NK, dict(kernel=capi.FG_KERNEL_NK_DOT2, tile_n=4, m_block=2, unroll=2)),
-        ("nk_mfma", NK, dict(kernel=capi.FG_KERNEL_NK_MFMA, tile_n=32, unroll=2)),
         ("nk_mfma4", NK, dict(kernel=capi.FG_KERNEL_NK_MFMA4, tile_n=16, m_block=8, unroll=1)),
-        ("nk_mfma_t", NK, dict(kernel=capi.FG_KERNEL_NK_MFMA_T, tile_n=64, unroll=16)),
         ("nk_mfma_r", NK, dict(kernel=capi.FG_KERNEL_NK_MFMA_R, tile_n=16, unroll=1, waves=8)),
         ("kn_dot2", KN, dict(kernel=capi.FG_KERNEL_KN_DOT2, m_block=2, unroll=2)),
         ("kn_mfma", KN, dict(kernel=capi.FG_KERNEL_KN_MFMA, unroll=1)),
@@ -48,7 +46,7 @@ def _plans():
 
 
 @pytest.mark.parametrize("name,layout,kw", _plans(), ids=[p[0] for p in _plans()])
-@pytest.mark.parametrize("splitk,fused", [(1, 0), (3, 1), (2, 0)])
+@pytest.mark.parametrize("splitk,fused", [(1, 0), (3, 1), (2, 0), (3, 2)])
 def test_every_kernel_family(device, name, layout, kw, splitk, fused):
     K, N = 1152, 384
     for M in (1, 7, 16, 19):
@@ -60,10 +58,7 @@ def test_every_kernel_family(device, name, layout, kw, splitk, fused):
             b = None if (i + M) % 3 == 0 else bias
             ref = oracle.gemm_bias_act(A.numpy(), W.numpy(), layout, None if b is None else b.numpy(), act)
             kwargs = dict(kw)
-            if name != "nk_mfma_t":     # that kernel derives its split from K
-                kwargs.update(splitk=splitk, fused=fused)
-            else:
-                kwargs.update(fused=fused)
+            kwargs.update(splitk=splitk, fused=fused)
             got = _bias_act(A, W, b, act, layout, device, plan=make_plan(**kwargs))
             assert_close_f16(got, ref, "%s M=%d act=%s bias=%s S=%d fused=%d" % (name, M, act, b is not None, splitk, fused))
 

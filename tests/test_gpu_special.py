@@ -145,10 +145,12 @@ def test_pitched_entry_point_rejects_bad_pitches(device):
 @pytest.mark.parametrize("layout,M,N,K", [(KN, 9, 7168, 2048), (KN, 1, 11008, 8192), (KN, 16, 4096, 4096),
                                           (NK, 16, 3072, 12288)])
 def test_in_launch_split_k_repeats_bit_for_bit(device, layout, M, N, K):
-    """Every wave's partial has to be in memory before its workgroup arrives at the tile counter;
-    an arrival that overtakes a store shows as a rare wrong sum.  Several hundred back-to-back
-    calls on rotating weights must all give the bits of the two-pass completion (a second kernel
-    sums the same partials in the same order)."""
+    """A completion that races shows as a rare wrong sum.  Several hundred back-to-back calls on
+    rotating weights must all give the same bits.  With the counter protocol (every wave's partial
+    has to be in memory before its workgroup arrives at the tile counter) those are the bits of
+    the two-pass completion, where a second kernel sums the same partials in the same order; the
+    atomic protocol sums in fixed point, so it is held to its own first result, and that result to
+    the two-pass one within one fp16 ulp."""
     L = capi.lib()
     p = capi.plan(M, N, K, layout, 0)
     if p.splitk < 2 or not p.fused:
@@ -168,10 +170,30 @@ def test_in_launch_split_k_repeats_bit_for_bit(device, layout, M, N, K):
         refs.append(C)
     assert_close_f16(refs[0].cpu().numpy(), (A.float() @ (Ws[0].float() if layout == KN else Ws[0].float().t())).cpu().numpy(),
                      "two-pass reference")
+    for protocol in sorted({1, p.fused}):
+        q = capi.plan(M, N, K, layout, 0)
+        q.fused = protocol
+        want = refs
+        if protocol == 2:
+            want = []
+            for i, W in enumerate(Ws):
+                C = torch.empty((M, N), dtype=torch.half, device=device)
+                capi.check(L.fg_gemm_f16_planned(ptr(A), ptr(W), ptr(C), M, N, K, layout, 0, ctypes.byref(q),
+                                                 ptr(ws), ws.numel(), stream_ptr()), "atomic")
+                want.append(C)
+                a = C.cpu().numpy().view(np.int16).astype(np.int32)
+                b = refs[i].cpu().numpy().view(np.int16).astype(np.int32)
+                far = (np.abs(a - b) > 1) & ((C.float() - refs[i].float()).abs().cpu().numpy() > 2e-6)
+                assert not far.any()                # neighbouring fp16 values, except next to zero
+        C = torch.empty((M, N), dtype=torch.half, device=device)
+        bad = torch.zeros((), dtype=torch.int64, device=device)
+        for i in range(400):
+            capi.check(L.fg_gemm_f16_planned(ptr(A), ptr(Ws[i % 4]), ptr(C), M, N, K, layout, 0, ctypes.byref(q),
+                                             ptr(ws), ws.numel(), stream_ptr()), "in-launch")
+            bad += (C.view(torch.int16) != want[i % 4].view(torch.int16)).sum()
+        assert int(bad.item()) == 0, protocol
+    # and through the entry point that plans by itself
     C = torch.empty((M, N), dtype=torch.half, device=device)
-    bad = torch.zeros((), dtype=torch.int64, device=device)
-    for i in range(400):
-        capi.check(L.fg_gemm_f16(ptr(A), ptr(Ws[i % 4]), ptr(C), M, N, K, layout, 0, 0, ptr(ws), ws.numel(),
-                                 stream_ptr()), "in-launch")
-        bad += (C.view(torch.int16) != refs[i % 4].view(torch.int16)).sum()
-    assert int(bad.item()) == 0
+    capi.check(L.fg_gemm_f16(ptr(A), ptr(Ws[0]), ptr(C), M, N, K, layout, 0, 0, ptr(ws), ws.numel(),
+                             stream_ptr()), "planned by the library")
+    assert torch.equal(C, want[0] if p.fused == 2 else refs[0])

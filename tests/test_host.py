@@ -49,8 +49,7 @@ def test_plan_is_consistent(layout, M, N, K):
     p = capi.plan(M, N, K, layout)
     d = p.as_dict()
     assert p.kernel in ((capi.FG_KERNEL_KN_DOT2, capi.FG_KERNEL_KN_MFMA) if layout == KN
-                        else (capi.FG_KERNEL_NK_DOT2, capi.FG_KERNEL_NK_MFMA, capi.FG_KERNEL_NK_MFMA4,
-                              capi.FG_KERNEL_NK_MFMA_T, capi.FG_KERNEL_NK_MFMA_R)), d
+                        else (capi.FG_KERNEL_NK_DOT2, capi.FG_KERNEL_NK_MFMA4, capi.FG_KERNEL_NK_MFMA_R)), d
     assert N % p.tile_n == 0 and p.grid_x == N // p.tile_n, d
     assert p.grid_y == -(-M // p.m_block) and p.grid_z == p.splitk >= 1, d
     assert p.block == 64 * p.waves and p.waves in (1, 2, 4, 8), d
@@ -64,8 +63,6 @@ def test_plan_is_consistent(layout, M, N, K):
         assert p.kernel in (capi.FG_KERNEL_KN_DOT2, capi.FG_KERNEL_NK_DOT2), d
     if p.kernel == capi.FG_KERNEL_NK_MFMA_R:
         assert p.tile_n in (16, 32, 48, 64) and p.m_block == (32 if M > 16 else 16), d
-    if p.kernel == capi.FG_KERNEL_NK_MFMA_T:
-        assert p.splitk == -(-(K // 32) // 64) and p.waves == 4 and p.tile_n % p.unroll == 0, d
     # a forced split is honoured
     for s in (1, 2, 7):
         q = capi.plan(M, N, K, layout, s)
