@@ -88,6 +88,29 @@ __device__ __forceinline__ int stagger_start(int nsteps, int flags) {
   return (int)(((flags & 2) ? lid : (lid >> 3)) % (unsigned)nsteps);
 }
 
+// Σ_{p < np} base[p * stride], p ascending, with all MAXP reads issued before the first add.  A loop
+// to a run-time bound compiles to read, wait, add per term: up to 32 dependent LDS round trips at
+// the end of every workgroup.  Terms past np re-read term 0 and add +0.
+template <int MAXP>
+__device__ __forceinline__ float lds_sum(const float* base, int stride, int np) {
+  float v[MAXP];
+#pragma unroll
+  for (int p = 0; p < MAXP; ++p) v[p] = base[(p < np ? p : 0) * stride];
+  float s = 0.f;
+#pragma unroll
+  for (int p = 0; p < MAXP; ++p) s += p < np ? v[p] : 0.f;
+  return s;
+}
+__device__ __forceinline__ int lds_sum_i32(const int* base, int stride, int np) {
+  int v[16];
+#pragma unroll
+  for (int p = 0; p < 16; ++p) v[p] = base[(p < np ? p : 0) * stride];
+  int s = 0;
+#pragma unroll
+  for (int p = 0; p < 16; ++p) s += p < np ? v[p] : 0;
+  return s;
+}
+
 // Orders LDS traffic among the lanes of one wavefront (data handed from lane to lane through
 // a wave-private LDS region).  The LDS unit serves a wave's requests in order; this only keeps
 // the compiler from moving the accesses across the hand-over point.  No s_barrier is issued.

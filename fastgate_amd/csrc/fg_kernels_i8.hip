@@ -130,11 +130,8 @@ __global__ __launch_bounds__(512) void w8a16_kernel(const int8_t* __restrict__ W
   __syncthreads();
   for (int t = threadIdx.x; t < RN * MB; t += blockDim.x) {
     const int m = t / RN, r = t % RN;
-    float sum = 0.f, xs = 0.f;
-    for (int p = 0; p < nw * 4; ++p) {
-      sum += red[p][r * MB + m];
-      xs += redx[p][m];
-    }
+    const float sum = lds_sum<32>(&red[0][r * MB + m], RN * MB, nw * 4);
+    const float xs = lds_sum<32>(&redx[0][m], MB, nw * 4);
     const int n = n0 + r;
     if (m < M)
       Y[(size_t)m * N + n] =
@@ -240,11 +237,8 @@ __global__ __launch_bounds__(256) void w8a16_m1_kernel(const int8_t* __restrict_
   __syncthreads();
   if (threadIdx.x < RN) {
     const int r = threadIdx.x;
-    float sum = 0.f, xs = 0.f;
-    for (int p = 0; p < nw * 4; ++p) {
-      sum += red[p][r];
-      xs += redx[p];
-    }
+    const float sum = lds_sum<16>(&red[0][r], RN, nw * 4);
+    const float xs = lds_sum<16>(&redx[0], 1, nw * 4);
     Y[n0 + r] = static_cast<half_t>((sum - zero_point * xs) * (scalar_scale * scale_value(scale_raw)));
   }
 }
@@ -307,8 +301,7 @@ __global__ __launch_bounds__(256) void i8i8_kernel(const int8_t* __restrict__ Wq
   __syncthreads();
   for (int t = threadIdx.x; t < RN * MB; t += blockDim.x) {
     const int m = t / RN, r = t % RN;
-    int sum = 0;
-    for (int p = 0; p < nw * 4; ++p) sum += red[p][r * MB + m];
+    const int sum = lds_sum_i32(&red[0][r * MB + m], RN * MB, nw * 4);
     if (m < M) out[(size_t)m * N + n0 + r] = sum;
   }
 }
@@ -440,12 +433,9 @@ __global__ __launch_bounds__(256) void w4a16_kernel(const uint8_t* __restrict__ 
   __syncthreads();
   for (int t = threadIdx.x; t < RN * MB; t += blockDim.x) {
     const int m = t / RN, r = t % RN;
-    float sum = 0.f, xe = 0.f, xo = 0.f;
-    for (int p = 0; p < nw * 4; ++p) {
-      sum += red[p][r * MB + m];
-      xe += redx[p][m];
-      xo += redo[p][m];
-    }
+    const float sum = lds_sum<16>(&red[0][r * MB + m], RN * MB, nw * 4);
+    const float xe = lds_sum<16>(&redx[0][m], MB, nw * 4);
+    const float xo = lds_sum<16>(&redo[0][m], MB, nw * 4);
     const int n = n0 + r;
     if (m < M)
       Y[(size_t)m * N + n] = static_cast<half_t>((sum - 64.f * xo - zero_point * (xe + xo)) *
@@ -586,11 +576,8 @@ __global__ __launch_bounds__(64 * NW) void w8a16_r_kernel(const int8_t* __restri
   for (int e = threadIdx.x; e < 16 * TN; e += blockDim.x) {
     const int m = e / TN, n = n0 + e % TN;
     if (m < M) {
-      float sum = 0.f, xs = 0.f;
-      for (int wv = 0; wv < nw; ++wv) {
-        sum += red[wv][0][e];
-        xs += red[wv][1][m * 16 + (e & 15)];
-      }
+      const float sum = lds_sum<NW>(&red[0][0][e], 2 * 16 * TN, nw);
+      const float xs = lds_sum<NW>(&red[0][1][m * 16 + (e & 15)], 2 * 16 * TN, nw);
       Y[(size_t)m * N + n] =
           static_cast<half_t>((sum - zero_point * xs) * (scalar_scale * scale_value(scale_raw)));
     }
@@ -712,11 +699,8 @@ __global__ __launch_bounds__(512) void w4a16_r_kernel(const uint8_t* __restrict_
   for (int e = threadIdx.x; e < 256; e += blockDim.x) {
     const int m = e >> 4, n = n0 + (e & 15);
     if (m < M) {
-      float sum = 0.f, xs = 0.f;
-      for (int wv = 0; wv < nw; ++wv) {
-        sum += red[wv][0][e];
-        xs += red[wv][1][e];
-      }
+      const float sum = lds_sum<NW>(&red[0][0][e], 512, nw);
+      const float xs = lds_sum<NW>(&red[0][1][e], 512, nw);
       Y[(size_t)m * N + n] =
           static_cast<half_t>((sum - zero_point * xs) * (scalar_scale * scale_value(scale_raw)));
     }

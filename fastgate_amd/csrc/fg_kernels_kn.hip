@@ -120,9 +120,7 @@ __global__ __launch_bounds__(64 * NW) void kn_mfma_kernel(const half_t* __restri
         const int e = base + i * (int)blockDim.x + (int)threadIdx.x;
         valid[i] = e < rows * 128;
         const int m = valid[i] ? e >> 7 : 0, c = e & 127;
-        float sum = 0.f;
-        for (int w = 0; w < nw; ++w) sum += red[w][m][c];
-        part[i] = sum;
+        part[i] = lds_sum<NW>(&red[0][m][c], 16 * 128, nw);
         idx[i] = (size_t)(m0 + m) * N + n0 + c;
       }
       fix_arrive<NB>(facc, fcls, idx, part, valid, gridDim.z, C, N, bias, flags);
@@ -134,12 +132,24 @@ __global__ __launch_bounds__(64 * NW) void kn_mfma_kernel(const half_t* __restri
     const int m = e >> 4, c0 = (e & 15) * 8;
     const int mg = m0 + m;
     if (mg < M) {
+      // the reads of all waves in flight before the first add
+      float4_t lo[NW], hi[NW];
+#pragma unroll
+      for (int w = 0; w < NW; ++w) {
+        const float4_t* src = reinterpret_cast<const float4_t*>(&red[w < nw ? w : 0][m][c0]);
+        lo[w] = src[0];
+        hi[w] = src[1];
+      }
       float sum[8];
 #pragma unroll
       for (int i = 0; i < 8; ++i) sum[i] = 0.f;
-      for (int w = 0; w < nw; ++w)
 #pragma unroll
-        for (int i = 0; i < 8; ++i) sum[i] += red[w][m][c0 + i];
+      for (int w = 0; w < NW; ++w)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          sum[i] += w < nw ? lo[w][i] : 0.f;
+          sum[4 + i] += w < nw ? hi[w][i] : 0.f;
+        }
       if (gridDim.z == 1) {
         half_t* c = C + (size_t)mg * N + n0 + c0;
         half8_t out;
@@ -239,9 +249,7 @@ __global__ __launch_bounds__(64 * NW) void kn_dot2_kernel(const half_t* __restri
         const int e = base + i * (int)blockDim.x + (int)threadIdx.x;
         valid[i] = e < rows * 128;
         const int m = valid[i] ? e >> 7 : 0, nn = e & 127;
-        float sum = 0.f;
-        for (int p = 0; p < nw * 4; ++p) sum += red[p][m][nn];
-        part[i] = sum;
+        part[i] = lds_sum<4 * NW>(&red[0][m][nn], MB * 128, nw * 4);
         idx[i] = (size_t)(m0 + m) * N + n0 + nn;
       }
       fix_arrive<NB>(facc, fcls, idx, part, valid, gridDim.z, C, N, bias, flags);
@@ -250,8 +258,7 @@ __global__ __launch_bounds__(64 * NW) void kn_dot2_kernel(const half_t* __restri
   }
   for (int e = threadIdx.x; e < MB * 128; e += blockDim.x) {
     const int m = e >> 7, nn = e & 127;
-    float sum = 0.f;
-    for (int p = 0; p < nw * 4; ++p) sum += red[p][m][nn];
+    const float sum = lds_sum<4 * NW>(&red[0][m][nn], MB * 128, nw * 4);
     const int mg = m0 + m, n = n0 + nn;
     if (mg < M) {
       if (gridDim.z == 1) {

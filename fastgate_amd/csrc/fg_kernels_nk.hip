@@ -83,8 +83,7 @@ __global__ __launch_bounds__(256) void nk_dot2_kernel(const half_t* __restrict__
   __syncthreads();
   for (int t = threadIdx.x; t < RN * MB; t += blockDim.x) {
     const int m = t / RN, r = t % RN;
-    float sum = 0.f;
-    for (int p = 0; p < nw * 4; ++p) sum += red[p][r * MB + m];
+    const float sum = lds_sum<16>(&red[0][r * MB + m], RN * MB, nw * 4);
     const int mg = m0 + m, n = n0 + r;
     if (mg < M) {
       if (gridDim.z == 1) {
@@ -190,8 +189,7 @@ __global__ __launch_bounds__(256) void nk_mfma4_kernel(const half_t* __restrict_
   for (int e = threadIdx.x; e < R4 * MG * 16; e += blockDim.x) {
     // e = ((g*4 + i) * R4 + r) * 4 + jj : consecutive threads write consecutive columns
     const int jj = e & 3, r = (e >> 2) % R4, gi = (e >> 2) / R4, g = gi >> 2, i = gi & 3;
-    float sum = 0.f;
-    for (int p = 0; p < nw * 4; ++p) sum += red[p][((r * MG + g) * 4 + i) * 4 + jj];
+    const float sum = lds_sum<16>(&red[0][((r * MG + g) * 4 + i) * 4 + jj], R4 * MG * 16, nw * 4);
     const int mg = m0 + 4 * g + i, n = n0 + 4 * r + jj;
     if (mg < M) {
       if (gridDim.z == 1) {
@@ -341,8 +339,7 @@ __global__ __launch_bounds__(64 * NW) void nk_mfma_r_kernel(const half_t* __rest
       for (int r = 0; r < 4; ++r) red[wave][(16 * mb + 4 * g + r) * TN + 16 * b + j] = acc[b][mb][r];
   __syncthreads();
   for (int e = threadIdx.x; e < TM * TN; e += blockDim.x) {
-    float sum = 0.f;
-    for (int wv = 0; wv < nw; ++wv) sum += red[wv][e];
+    const float sum = lds_sum<NW>(&red[0][e], TM * TN, nw);
     const int mg = m0 + e / TN, n = n0 + e % TN;
     if (e / TN < AROWS && mg < M && (!RAGGED || e % TN < tw)) {
       if (gridDim.z == 1) {
