@@ -33,6 +33,9 @@ HIP_SOURCES = [
     "fg_capi.hip",
 ]
 
+# plain C++ units of the library (no HIP): the launch planner
+HOST_SOURCES = ["fg_planner.cpp"]
+
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",
     "-O3",
@@ -75,8 +78,15 @@ def build_lib(verbose: bool = True) -> Path:
              quiet_pattern="is not a recognized feature")
         return str(obj)
 
-    with ThreadPoolExecutor(max_workers=min(8, len(HIP_SOURCES))) as pool:
-        objs = list(pool.map(compile_one, HIP_SOURCES))
+    def compile_host(src: str) -> str:
+        obj = OBJ / (Path(src).stem + ".o")
+        _run(["g++", "-O2", "-fPIC", "-std=c++17", "-Wall", "-I", str(ROOT / "include"), "-c", str(CSRC / src),
+              "-o", str(obj)])
+        return str(obj)
+
+    with ThreadPoolExecutor(max_workers=min(8, len(HIP_SOURCES) + len(HOST_SOURCES))) as pool:
+        host = [pool.submit(compile_host, s) for s in HOST_SOURCES]
+        objs = list(pool.map(compile_one, HIP_SOURCES)) + [h.result() for h in host]
     out = PKG / LIB_NAME
     _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(out), *objs])
     if verbose:

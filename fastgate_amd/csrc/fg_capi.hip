@@ -10,6 +10,7 @@
 #include <mutex>
 
 #include "fg_internal.h"
+#include "fg_plan.h"
 
 // Split-K scratch of fg_gemm_f16_static: one copy per GPU, held until the process ends.  The name
 // is a host-side stand-in for the symbol, never a device address: host code reaches the memory
@@ -19,524 +20,21 @@ static __device__ __align__(256) unsigned char scratch[FG_STATIC_SCRATCH_BYTES];
 namespace fg {
 namespace {
 
-constexpr int kCUs = 256;  // MI355X compute units
-
-int ceil_div(int a, int b) { return (a + b - 1) / b; }
-
-int pick_waves(int items) { return items >= 4 ? 4 : (items >= 2 ? 2 : 1); }
-
-// Work items = groups of `unroll` K units handed round-robin to waves*S slots.  Returns the
-// fraction of slot-steps that carry real work (1.0 = perfectly even).
-double balance(int items, int slots) {
-  const int per = ceil_div(items, slots);
-  return (double)items / ((double)per * slots);
-}
-
-// Cross-workgroup split-K factor for the K-interleaved kernels.  A split costs S*M*N*8 bytes
-// of fp32 partial traffic and the arrival protocol, so it is only taken when the un-split
-// grid leaves CUs idle.
-int pick_splitk(int tiles, int waves, int items, int M, int N, int K, int target_wgs) {
-  static const int cand[] = {1, 2, 3, 4, 6, 8, 12, 16};
-  int best = 1;
-  double best_score = -1.0;
-  for (int S : cand) {
-    if (S > 1 && items / (waves * S) < 2) continue;  // keep >= 2 steps per wave
-    const double fill = std::min(1.0, (double)tiles * S / target_wgs);
-    const double extra = S > 1 ? (8.0 * S * M * N) / (2.0 * K * N) : 0.0;  // partials vs weights
-    double score = balance(items, waves * S) * fill / (1.0 + extra);
-    if (S > 1) score *= 0.95;
-    if (score > best_score + 1e-9) {
-      best_score = score;
-      best = S;
-    }
-  }
-  return best;
-}
-
-int validate_shape(int M, int N, int K, int w_layout) {
-  if (M <= 0 || N <= 0 || K <= 0) return FG_ERR_INVALID_ARG;
-  if (w_layout != FG_W_KN && w_layout != FG_W_NK) return FG_ERR_INVALID_ARG;
-  if (N % 128 != 0 || K % 128 != 0) return FG_ERR_ALIGN128;
-  return FG_OK;
-}
-
-// Fills grid/block/workspace from the tile fields; rejects tiles that were not built.
-int finish_plan(int M, int N, int K, fg_plan_t* p) {
-  const int max_waves =
-      ((p->kernel == FG_KERNEL_NK_MFMA_R && (p->band ? p->band : 256 * p->unroll) <= 256) ||
-       p->kernel == FG_KERNEL_KN_MFMA ||
-       (p->kernel == FG_KERNEL_KN_DOT2 && p->m_block <= 2))
-          ? 8
-          : 4;
-  if (p->splitk < 1 || p->waves < 1 || p->waves > max_waves || (p->waves & (p->waves - 1))) {
-    return FG_ERR_INVALID_ARG;
-  }
-  switch (p->kernel) {
-    case FG_KERNEL_NK_DOT2:
-      if (!nk_dot2_supported(p->m_block, p->tile_n, p->unroll)) return FG_ERR_UNSUPPORTED;
-      break;
-    case FG_KERNEL_NK_MFMA4:
-      if (!nk_mfma4_supported(p->m_block, p->tile_n, p->unroll)) return FG_ERR_UNSUPPORTED;
-      break;
-    case FG_KERNEL_NK_MFMA_R:
-      // 16, 32, 48, 64, or any width from 17 to 47 that divides N (one partly filled column
-      // block; 128-byte bands, 8 waves, no split-K)
-      if (p->tile_n != 32 && p->tile_n != 48 && p->tile_n != 64 &&
-          !(p->tile_n > 16 && p->tile_n < 48 && N % p->tile_n == 0)) {
-        p->tile_n = 16;
-      }
-      if (p->tile_n % 16 != 0 && (p->splitk != 1 || p->waves != 8)) return FG_ERR_UNSUPPORTED;
-      p->m_block = p->m_block == 32 ? 32 : 16;  // 32: two row blocks per workgroup (128-byte bands)
-      if (p->band == 0) {
-        if (p->unroll != 1 && p->unroll != 2) return FG_ERR_UNSUPPORTED;
-        p->band = 256 * p->unroll;
-      }
-      if (p->band != 128 && p->band != 256 && p->band != 512) return FG_ERR_UNSUPPORTED;
-      if ((p->tile_n > 32 || p->tile_n % 16 != 0 || p->m_block == 32) && p->band != 128) return FG_ERR_UNSUPPORTED;
-      if (p->m_block == 32 && (p->tile_n % 16 != 0 || p->tile_n > 48)) return FG_ERR_UNSUPPORTED;
-      p->unroll = p->band == 512 ? 2 : 1;
-      break;
-    case FG_KERNEL_KN_DOT2:
-      p->tile_n = 128;
-      if (!kn_dot2_supported(p->m_block, p->unroll)) return FG_ERR_UNSUPPORTED;
-      break;
-    case FG_KERNEL_KN_MFMA:
-      p->tile_n = 128;
-      p->m_block = 16;
-      if (!kn_mfma_supported(p->unroll)) return FG_ERR_UNSUPPORTED;
-      break;
-    default:
-      return FG_ERR_UNSUPPORTED;
-  }
-  if (N % p->tile_n != 0) return FG_ERR_UNSUPPORTED;
-  if (p->splitk > 65535) return FG_ERR_INVALID_ARG;
-  p->grid_x = N / p->tile_n;
-  p->grid_y = ceil_div(M, p->m_block);
-  if (p->grid_y > 65535) return FG_ERR_INVALID_ARG;  // HIP's limit on grid.y
-  p->grid_z = p->splitk;
-  p->block = 64 * p->waves;
-  if (p->splitk > 1) {
-    if ((long long)p->grid_x * p->grid_y > kWsMaxTiles) p->fused = 0;
-    // the in-launch completion addresses the partials with 32-bit byte offsets
-    if ((unsigned long long)p->splitk * M * N * sizeof(float) > 0x7fffffffull) p->fused = 0;
-    p->workspace_bytes = kWsHeaderBytes + (size_t)p->splitk * M * N * sizeof(float);
-  } else {
-    p->workspace_bytes = 0;
-  }
-  return FG_OK;
-}
-
-// Wider tiles of the row-load kernel on 128-byte bands.  Two, three or a ragged number of column
-// blocks share a staged band of activations and a band carries half the activation bytes, so the
-// L2 traffic for A drops to a quarter or less of the 16-column / 256-byte form -- but the grid
-// shrinks with the tile, so it has to land on whole CUs: 192..256 workgroups of 8 waves (one a
-// CU) or 448..512 (two a CU).  Candidates, measured against the 16-column form (us):
-//   32 columns            K = N = 8192 M=16 22.8 / 24.7, M=8 22.9 / 23.3; K = N = 6144 M=16 16.6 / 18.9;
-//                         K=2048 N=8192 M=16 7.9 / 9.0; K=4096 N=16384 M=16 22.4 / 24.3 (4 waves)
-//   32 columns, split-K   N=3072 K=12288 M=16 S=2 18.2 / 19.4 (M <= 8: 16.3 / 16.1, so M >= 9 only);
-//                         N=2560 K=10240 M=16 S=3 13.3 / 16.7; N=5120 K=13824 S=3 (two a CU) 24.8 / 27.0
-//   48 columns            N = 12288: K=3072 M=16 14.4 / 15.9, K=12288 47.0 / 52.6; N=3072 K=12288 split 4 ways
-//   64 columns            N = 28672, K = 8192
-//   N/256 or N/512 columns with a partly filled last block (masked loads cost a little):
-//                         N=11008 K=4096 M=16 17.4 / 19.0 (M=8: 17.4 / 17.0); N=10240 K=8192 M=16
-//                         28.4 / 33.0; N = K = 5120 M=8 12.1 / 14.1; N=6144 K=4096 M=16 11.2 / 12.9
-//                         (24 columns, against 32); N=13824 K=5120 M=16 26.1 / 30.3 (27 columns, two a CU)
-// 384 workgroups (N = 12288 at 32 columns) leave half the CUs with one: 46+ us against 45.
-struct WideTile {
-  int tile_n = 0, waves = 0, splitk = 1;
-};
-WideTile pick_wide_tile(int M, int N, int K, int splitk) {
-  WideTile best;
-  double best_fill = 0.0;
-  // a later candidate replaces an earlier one only when it fills the CUs better by `margin`
-  auto offer = [&](int tile, int waves, int S, int wgs, bool allowed, double margin = 0.04) {
-    if (!allowed) return;
-    const double fill = (double)wgs / (double)(ceil_div(wgs, kCUs) * kCUs);
-    if (fill > best_fill + margin) {
-      best_fill = fill;
-      best = WideTile{tile, waves, S};
-    }
-  };
-  const bool auto_split = splitk == 0;
-  // Rows that do not start on a 2 KB boundary (K not a multiple of 1024) cost the 128-byte-band
-  // tiles their lead: N=12288 K=11008 M=8 48 columns 49.6 us against 42.4 for 16 columns on 256-byte
-  // bands, K=10752 46.4 / 41.9, while K=10240 and K=11264 are 40.2 and 42.6 with 48 columns;
-  // N=8192 K=11008 M=8 32 columns 31.1 / 29.8, N=16384 59.0 / 55.6.  With 9..16 rows the 32-column
-  // forms stay level.
-  const bool odd_pitch = K % 1024 != 0 && K > 4096;
-  if (N % 32 == 0) {
-    const int t32 = N / 32;
-    // not at K = 4096, where rows 8 KB apart make this form 8-15 % slower than 16-column tiles
-    // (N=8192 M=8 14.6 us against 12.5; K = 3840 and 4352 are unaffected)
-    offer(32, 8, 1, t32, t32 <= kCUs && 4 * t32 >= 3 * kCUs && (M >= 4 || t32 < kCUs) && K != 4096 &&
-                             (!odd_pitch || M >= 9 || 8 * t32 < 7 * kCUs));
-    // short rows of very wide outputs: two 8-wave workgroups of 32 columns on every CU
-    // (K=2048: N=14336 M=8 12.1 -> 11.3 us, N=16384 M=16 13.7 -> 12.7)
-    offer(32, 8, 1, t32, K > 1024 && K <= 2048 && M >= 4 && t32 <= 2 * kCUs && 8 * t32 >= 13 * kCUs);
-    // 64 columns on 13/16 of the CUs or more beat two 4-wave workgroups of 32 on each
-    // (N=14336 K=4096: M=8 21.0 -> 20.0 us, M=16 21.9 -> 20.8; N=13824 K=5120 M=8 25.8 -> 24.7)
-    if (N % 64 == 0) {
-      const int t64 = N / 64;
-      offer(64, 8, 1, t64, M >= 5 && K >= 2048 && t64 < kCUs && 16 * t64 >= 13 * kCUs);
-      // ... and one 64-column workgroup on every CU for 12 rows and more (N=16384 M=16: K=5120
-      // 30.1 -> 28.0 us, K=14336 73.4 -> 70.5)
-      offer(64, 8, 1, t64, M >= 12 && K >= 5120 && t64 == kCUs);
-    }
-    offer(32, 4, 1, t32, 8 * t32 >= 7 * 2 * kCUs && t32 <= 2 * kCUs && (t32 == 2 * kCUs ? M >= 5 : M >= 9) &&
-                             (!odd_pitch || M >= 9));
-  }
-  if (N % 48 == 0) {
-    const int t48 = N / 48;
-    // (one a CU from four rows on: N=9216 M=4 K=4096 14.9 -> 14.2 us, K=8192 27.7 -> 25.5)
-    offer(48, 8, 1, t48, !odd_pitch && ((M >= (t48 < kCUs ? 3 : 8) && t48 <= kCUs && 4 * t48 >= 3 * kCUs) ||
-                                        (t48 == 2 * kCUs && M >= 9)));
-  }
-  if (N % 64 == 0) {
-    // very wide outputs (N=28672 K=8192 M=16: 64 columns 72.1 us, 32 columns 74.0, 16 columns 81+)
-    const int t64 = N / 64;
-    offer(64, 8, 1, t64, M >= 9 && K >= 8192 && t64 <= 2 * kCUs && 8 * t64 >= 7 * 2 * kCUs);
-  }
-  if (N % 32 == 0 && auto_split && N / 32 < 3 * kCUs / 4) {
-    // split-K keeps at least 3072 k per split (six 128-byte bands for each of eight waves)
-    const int t32 = N / 32;
-    for (int S = 2; S <= 4; ++S) {
-      const int wgs = t32 * S;
-      // (64 tiles or fewer split four ways from 2048 k a split: N=2048 M=16 K=8192 10.2 -> 9.7 us,
-      // K=11008 12.8 -> 11.9; two ways only beyond K = 8192: N=4096 K=8192 M=16 15.0 against 14.3
-      // for 16 columns unsplit)
-      const bool long_k = t32 <= 64 ? K / S >= 2048 : K / S >= 3072 && (S > 2 || K > 8192);
-      offer(32, 8, S, wgs, long_k && M >= 9 && wgs <= kCUs && 4 * wgs >= 3 * kCUs);
-    }
-    if (N % 48 == 0) {
-      // (N=3072 K=12288 M=16: 48 columns split 4 ways 16.4 us, 32 columns split 2 ways 17.9)
-      const int t48 = N / 48;
-      for (int S = 2; S <= 4; ++S) {
-        const int wgs = t48 * S;
-        // (64 tiles: from 1536 k a split, N=3072 K=6144 M=16 11.3 -> 10.6 us; 8 rows only with long
-        // K, K=14336 18.1 -> 17.3 but K=6144 9.4 -> 10.1)
-        const bool ok48 = (t48 <= 64 && S == 4) ? K / S >= 1536 && (M >= 9 || (M == 8 && K >= 12288))
-                                               : K / S >= 3072 && M >= 9;
-        offer(48, 8, S, wgs, ok48 && wgs <= kCUs && 4 * wgs >= 3 * kCUs);
-      }
-    }
-    // two workgroups a CU, only where no split lands on one a CU
-    bool one_a_cu = false;
-    for (int S = 1; S <= 4; ++S) one_a_cu |= t32 * S <= kCUs && 4 * t32 * S >= 3 * kCUs;
-    for (int S = 2; S <= 4 && !one_a_cu; ++S) {
-      const int wgs = t32 * S;
-      offer(32, 8, S, wgs, K / S >= 3072 && M >= 4 && wgs <= 2 * kCUs && 8 * wgs >= 7 * 2 * kCUs);
-    }
-  }
-  // Ragged tiles pay for their masked loads and empty operand slots: they need a clearly better
-  // fill (N = 7168, M = 9: 28 columns 19.4 us, 32 columns 18.2), three column blocks (33..47 columns) against 48 columns too (N = 9216:
-  // 36 columns 17.3 us, 48 columns 15.5), and two ragged workgroups a CU lose to 448 workgroups of
-  // 32 columns (N=14336 K=4096 M=16: 23.9 / 22.0).
-  if (K >= 1024 && N % kCUs == 0) {
-    const int tw = N / kCUs;
-    const bool thin16 = N / 16 < 3 * kCUs / 2;  // 16-column tiles would leave CUs with one workgroup
-    // (K = 4096 again, two nearly full column blocks: N=7168 M=9 28 columns 14.4 us against 13.0 for
-    // 16; N=6144 24 columns 10.9 / 11.6 and N=11008 43 columns 17.0 / 18.4 are unaffected)
-    offer(tw, 8, 1, kCUs,
-          tw >= 20 && tw < 48 && tw % 16 != 0 && (M >= 9 || (thin16 && M >= 3)) && !(K == 4096 && tw > 24 && tw < 32),
-          tw > 32 ? 0.3 : 0.15);
-  }
-  if (K >= 1024 && N % (2 * kCUs) == 0) {
-    const int tw = N / (2 * kCUs);
-    offer(tw, 8, 1, 2 * kCUs, tw >= 20 && tw < 48 && tw % 16 != 0 && M >= 9, 0.15);
-  }
-  return best;
-}
-
-int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
-  std::memset(p, 0, sizeof(*p));
-  p->stream_w = 1;
-  // Split-K can finish inside the launch (the last workgroup of a tile sums the partials) or
-  // in a second kernel.  Measured at K = N = 8192, S = 4 (us per call, second kernel / in-launch):
-  // [K,N] M=1 26.4 / 25.0, M=8 26.2 / 25.2, M=16 26.5 / 25.9.  Beyond one block of 16 rows the
-  // second kernel takes over.
-  p->fused = M <= 16;
-  int items = 1;
-  bool row_tiles = false;   // the 16-column row-load kernel picks its own split
-  bool wide_tiles = false;  // ... in its 32-column form
-  int wide_band_waves = 0, wide_band_split = 0;  // ... on 128-byte bands: waves and split are fixed
-  if (w_layout == FG_W_NK) {
-    // Measured on MI355X at K = N = 8192 (us per call): M=1 dot2 tile 4: 21.6-22.4; M=4 dot2
-    // 24.3 / mfma4 22.3; M=8 dot2 27.8 / mfma4 25.6 / row-load 23.3; M=16 mfma4 36 / direct
-    // 16x16x32 31.7 / transposing 27.3 / row-load 24.6.  Every rule below is the measured winner of
-    // a sweep over K = N in 1024..16384 and the LLaMA / DiT projection shapes for its range.
-    const bool huge = K >= 16384 && N >= 16384;  // the 4x4x4 MFMA kernel's zone, also for M <= 2
-    if ((M <= 2 && !huge) || (M <= 4 && N <= 2048 && K >= 8192)) {
-      // (few, long rows at M = 3..4: v_dot2 8.8-9.3 us against 9.4-9.5 for N = 2048, K = 8192)
-      p->kernel = FG_KERNEL_NK_DOT2;
-      p->m_block = M <= 2 ? M : 4;
-      p->tile_n = 4;
-      // two load groups in flight beyond K = 8192 (K=11008 N=4096 M=1 16.7 -> 15.8 us, K=14336
-      // 20.0 -> 19.0); start steps by workgroup id below K = 8192 and between 8192 and 16384, by
-      // workgroup id / 8 at 8192 (22.0 -> 21.8) and from 16384 on (N=4096 23.2 -> 21.6, N=8192
-      // 42.5 -> 40.2, N=14336 71.5 -> 68.8)
-      p->unroll = (K > 8192 || M > 2) ? 2 : 1;
-      items = ceil_div(K / 8, 64 * p->unroll);
-      p->stagger = M <= 2 ? (K < 8192 || (K > 8192 && K < 16384)) : items <= 16;
-    } else if (M <= 8 && huge) {
-      // (K = N = 16384: M = 1 79.8 us against 82.1 for v_dot2, M = 2 79.1 / 81.5, M = 4 78.7 against
-      // 79.9 for the row-load kernel, M = 8 77.5 / 78.9; at
-      // N = 8192, K = 28672 the row-load kernel is ahead, M = 8 69.8 / 78.3)
-      p->kernel = FG_KERNEL_NK_MFMA4;
-      p->m_block = M <= 4 ? 4 : 8;
-      if (K >= 16384) {
-        p->tile_n = 32, p->unroll = 1;
-      } else if (K == 8192 || N <= 4096) {
-        // two chunks per wave and step: 8 steps at K = 8192, one K band per XCD
-        p->tile_n = N <= 4096 ? 8 : 16, p->unroll = K >= 256 ? 2 : 1, p->stagger = K <= 8192;
-      } else {
-        p->tile_n = 16, p->unroll = 1;
-      }
-      items = ceil_div(K / 128, p->unroll);
-    } else {
-      // M >= 3: 16-column tiles, weights and activations as contiguous row pieces through LDS,
-      // 8 waves on 256-byte bands.  Measured against the best of the other [N,K] kernels (us):
-      // K = N = 8192 M=8 23.2 / 25.6, M=16 24.6 / 27.3; K=3072 N=12288 M=16 15.6 / 21.0;
-      // K=12288 N=3072 M=16 19.1 / 20.3; K = N = 4096 M=8 7.8 / 9.5; K=4096 N=11008 M=8 16.5 / 20.1.
-      // At K = 16384 four waves on 512-byte bands are level or slightly ahead (M=16 84.3 / 85.8).
-      // M = 3..4 against the 4x4x4 kernel: K = N = 4096 8.7-8.9 / 9.2-9.5, K = N = 8192 22.9 / 22.3-24.0,
-      // K=12288 N=3072 14.6 / 15.2-16.0, K=4096 N=11008 15.8 / 16.6-16.9.
-      p->kernel = FG_KERNEL_NK_MFMA_R;
-      p->m_block = 16;
-      p->tile_n = 16;
-      p->unroll = (K >= 16384 && N >= 8192) ? 2 : 1;
-      items = ceil_div(K, 128 * p->unroll);
-      row_tiles = true;
-      if (M > 16) {
-        // 32 rows of A per workgroup (two MFMA row blocks on 128-byte bands): 17..32 rows read the
-        // weights once instead of twice
-        p->m_block = 32;
-        p->unroll = 1;
-        p->band = 128;
-        items = ceil_div(K, 64);
-      }
-      if (!wide_tiles && M <= 32 && splitk <= 1) {
-        WideTile wt = pick_wide_tile(M < 16 ? M : 16, N, K, splitk);
-        if (M > 16 && (wt.tile_n % 16 != 0 || wt.tile_n > 48)) wt = WideTile{};  // no ragged or 64-column form
-        if (wt.tile_n) {
-          p->tile_n = wt.tile_n;
-          p->unroll = 1;
-          p->band = 128;
-          wide_tiles = true;
-          wide_band_waves = wt.waves;
-          wide_band_split = wt.splitk;
-        }
-      }
-    }
-  } else {
-    const size_t weights = (size_t)N * K;
-    const bool dot2_m1 = weights < ((size_t)1 << 27) || (weights < ((size_t)1 << 28) && N >= 25600);
-    if (M == 1 ? dot2_m1 : (M == 2 && weights < ((size_t)1 << 27))) {
-      // (at K = N = 16384 the MFMA kernel streams better even for M = 1: 80 us against 90; two rows
-      // from 2^27 weights on: K=8192 N=16384 43.7 / 46.0, K=28672 N=8192 76.5 / 78.4, K=8192 N=28672
-      // 73.9 / 75.3; one row too where such weights still need a split: K=11008 N=16384 56.7 / 59.9,
-      // K=14336 N=16384 71.7 / 77.2, while K=8192 N=28672, unsplit, is 74.9 / 73.8)
-      p->kernel = FG_KERNEL_KN_DOT2;
-      p->m_block = M;
-    } else {
-      p->kernel = FG_KERNEL_KN_MFMA;  // 26.3 us against 29.8 for v_dot2 at M = 4, K = N = 8192
-      p->m_block = 16;
-    }
-    p->tile_n = 128;
-    // one 32-row unit in flight per wave and step: with the split-K tail no longer waiting on
-    // each partial in turn, deeper splits of shorter steps win (v_dot2, M = 1, two units / one:
-    // K = N = 4096 10.5 / 9.7 us, K=3072 N=12288 16.7 / 15.5, K=4096 N=11008 18.5 / 17.3)
-    p->unroll = 1;
-    items = ceil_div(K / 32, p->unroll);
-  }
-  {
-    p->waves = (row_tiles && !wide_tiles && p->unroll == 1 && items >= 16) ? 8 : pick_waves(items);
-    if (wide_band_waves) {
-      p->waves = wide_band_waves;
-      while (p->waves > 1 && p->waves > K / 64) p->waves >>= 1;  // one 128-byte band per wave at least
-    }
-    const int tiles = (N / p->tile_n) * ceil_div(M, p->m_block);
-    if (splitk > 0) {
-      p->splitk = splitk;
-    } else if (w_layout == FG_W_KN) {
-      // [K,N] tiles are 128 columns wide, so the grid needs split-K to cover the chip: the
-      // factor that brings tiles*S closest to one workgroup per CU.
-      int best = 1;
-      bool half_filled = false;  // fewer workgroups than CUs on purpose
-      if ((size_t)N * K < ((size_t)1 << 26) && items >= 16 && M <= 16) {
-        // Below 8192 x 8192 the call is latency-bound: 8 waves per workgroup and half the split
-        // (about 192 workgroups) shorten every wave's chain of dependent loads.  Measured (us,
-        // 4 waves / 8 waves, M = 4): K=N=4096 12.3 / 11.2, K=4096 N=11008 20.1 / 18.1,
-        // K=3072 N=12288 17.2 / 15.9, K=12288 N=3072 20.5 / 17.8, K=N=2048 12.3 / 8.8.
-        // Here the in-launch reduction also wins for 9..16 rows (M = 16: K=3072 N=12288 17.2 us
-        // against 17.9 with the second kernel, K=12288 N=3072 18.9 / 20.0, K=4096 N=11008 19.3 /
-        // 20.3); at 8192 x 8192 the second kernel stays 0.6 us ahead for them.
-        // Sixteen tiles or fewer with K <= 8192 leave each wave one or two units at 192 workgroups:
-        // aim at 128 there (N=2048: K=4096 M=1 9.7 -> 8.1 us, M=16 10.8 -> 9.0; K=8192 12.0 -> 10.6).
-        // Eight tiles with long K take a 24-way split (N=1024 K=28672: M=1 15.3 -> 13.8, M=16 17.9
-        // -> 16.2) as long as every wave keeps two units.
-        p->waves = 8;
-        p->fused = 1;
-        half_filled = tiles <= 16 && K <= 8192;
-        const double target = half_filled ? 128.0 : 192.0;
-        double best_dist = 1e30;
-        static const int kSplits[] = {1, 2, 4, 8, 16, 24};
-        for (int S : kSplits) {
-          if (items / (p->waves * S) < 1) break;
-          if (S > 16 && (tiles > 8 || items / (p->waves * S) < 2)) break;
-          // 9..16 rows: the partials of a split that leaves a wave one unit cost more than the
-          // idle CUs once there are more than 192 workgroups (N=4096 K=2048 M=12: 8 ways 10.3 us,
-          // 4 ways 8.3; N=2048 K=2048 M=16: 8 ways 7.4, 4 ways 7.9)
-          if (M > 8 && S > 1 && items / (p->waves * S) < 2 && tiles * S > 192) break;
-          const double dist = std::fabs(std::log2((double)tiles * S / target));
-          if (dist < best_dist - 1e-9) {
-            best_dist = dist;
-            best = S;
-          }
-        }
-      } else if ((size_t)N * K >= ((size_t)1 << 18)) {  // 1024 x 1024: 7.7 us with S = 8 against 9.0 without
-        // up to eight rows the partials are small enough for two workgroups per CU to pay, the more
-        // so as the two take neighbouring column bands (K = N = 8192, S = 8 / S = 4: M=1 23.1 / 24.3
-        // us, M=4 23.9 / 25.4, M=8 24.7 / 24.9; K=4096 N=16384 M=1 S = 4 / 2: 23.3 / 24.5)
-        const bool two_a_cu = (size_t)N * K <= ((size_t)1 << 26) && ((M <= 8 && tiles <= 64) || (M <= 2 && tiles <= 128));
-        const int target = two_a_cu ? 2 * kCUs : kCUs;
-        double best_ratio = 1e30;
-        for (int S = 1; S <= 16; S *= 2) {
-          if (items / (p->waves * S) < 1) break;
-          const double r = (double)tiles * S / target;
-          const double ratio = r > 1.0 ? r : 1.0 / (r * r);  // idle CUs cost more than a deeper split
-          if (ratio < best_ratio - 1e-9) {
-            best_ratio = ratio;
-            best = S;
-          }
-        }
-      }
-      p->splitk = best;
-      // the v_dot2 kernel wants eight waves on every CU: K=4096 N=16384, M = 1, S = 2:
-      // 26.9 us with four waves a workgroup, 24.3 with eight
-      if (p->kernel == FG_KERNEL_KN_DOT2 && p->waves == 4 && tiles * best < 2 * kCUs &&
-          items / (8 * best) >= 2) {
-        p->waves = 8;
-      }
-      // 9..16 rows at 8192 x 8192: 26.0 us with eight waves against 26.5 with four (at 16384 x 16384
-      // four stay ahead, 82.3 against 89)
-      if (p->kernel == FG_KERNEL_KN_MFMA && M > 8 && p->waves == 4 &&
-          (size_t)N * K <= ((size_t)1 << 26) && items / (8 * best) >= 2) {
-        p->waves = 8;
-      }
-      // The rules above only try powers of two.  When their choice leaves the CUs unevenly loaded
-      // (tiles * S just over a multiple of 256: 80 tiles x 4 = 320 workgroups take 36 us where
-      // 80 x 3 = 240 take 29), search every S with either one 8-wave workgroup per CU or two
-      // 4-wave ones, scored by how evenly the CUs are filled, how evenly K divides over the wave
-      // slots, the partial traffic and the length of each wave's chain of loads.  Fitted to
-      // sweeps over N in {5120, 6144, 9216, 10240, 11008, 12288, 13824, 14336} x K in {3072..13824}.
-      {
-        auto score = [&](int S, int w) {
-          const int n = tiles * S;
-          const int per_cu = ceil_div(n, kCUs);
-          const double fill = (double)n / ((double)per_cu * kCUs);
-          const double per_wave = (double)items / (w * S);
-          const double chain = per_wave >= 8.0 ? 1.0 : std::sqrt(per_wave / 8.0);
-          const double partials = 1.0 / (1.0 + 4.0 * S * M / K);
-          // 9..16 rows: two 4-wave workgroups a CU write twice the partials of one 8-wave workgroup
-          // for the same K range and lose to it at equal fill (N=5120 K=8192 M=16: 11 splits of 4
-          // waves 20.4 us, 5 of 8 waves 19.2; N=9216 K=4096 18.2 / 17.6)
-          const double two_a_cu = (M > 8 && w == 4) ? 0.88 : 1.0;
-          return fill * balance(items, w * S) * partials * chain * two_a_cu;
-        };
-        const int n0 = tiles * p->splitk;
-        const double fill0 = (double)n0 / ((double)ceil_div(n0, kCUs) * kCUs);
-        if (fill0 < 0.85 && !half_filled && M <= 16 && (size_t)N * K >= ((size_t)1 << 22)) {
-          double best_score = score(p->splitk, p->waves) * 1.05;  // switch for a clear win only
-          int best_s = 0, best_w = 0;
-          for (int S = 1; S <= 16; ++S) {
-            const int per_cu = ceil_div(tiles * S, kCUs);
-            if (per_cu > 2) break;
-            const int w = per_cu == 1 ? 8 : 4;
-            if (items / (w * S) < 2) break;
-            const double sc = score(S, w);
-            if (sc > best_score + 1e-9) {
-              best_score = sc;
-              best_s = S;
-              best_w = w;
-            }
-          }
-          if (best_s) {
-            p->splitk = best_s;
-            p->waves = best_w;
-          }
-        }
-      }
-      // 9..16 rows, four splits of 64 tiles (one workgroup on every CU) and at least eight units a
-      // wave: eight waves with two units in flight (K = N = 8192 M=16 26.2 -> 25.7 us, K=14336
-      // 42.0 -> 41.2; not with rows off 2 KB boundaries, and not with other splits: K=4096 N=12288
-      // 21.1 -> 21.6)
-      if (p->kernel == FG_KERNEL_KN_MFMA && M > 8 && M <= 16 && tiles == 64 && p->splitk == 4 &&
-          K % 1024 == 0 && items / (8 * 4) >= 8 && (size_t)N * K <= ((size_t)1 << 27)) {
-        p->waves = 8;
-        p->unroll = 2;
-      }
-      // One or two rows: two 4-wave workgroups a CU on neighbouring column bands instead of one
-      // 8-wave workgroup, where that lands on 448..512 workgroups and leaves every wave four units
-      // (M=1, twice the split with 4 waves / 8 waves: K=14336 N=8192 37.3 / 40.6 us, K=11008 N=8192
-      // 30.4 / 32.4, K=5120 N=16384 28.2 / 29.8; M=2: K=11008 N=4096 17.6 / 18.5, K=4096 N=8192
-      // 14.1 / 14.7)
-      {
-        const int twice = 2 * tiles * p->splitk;
-        if (splitk == 0 && M <= 2 && p->kernel == FG_KERNEL_KN_DOT2 && p->waves == 8 &&
-            p->splitk <= 8 && twice >= 448 && twice <= 2 * kCUs && items / (4 * 2 * p->splitk) >= 4) {
-          p->splitk *= 2;
-          p->waves = 4;
-        }
-      }
-    } else if (wide_band_split) {
-      p->splitk = wide_band_split;
-      p->fused = 1;
-    } else if (row_tiles) {
-      // 192 tiles still run best unsplit (K=12288 N=3072 M=8: 16.0 us against 17.4 with S = 4);
-      // 128 tiles or fewer want two workgroups per CU once K is long (N=2048: K=8192 M=16
-      // 10.5 us with S = 2 against 12.4, K=16384 15.7 against 21.7).  The partials of a 16-column
-      // tile are small, so the split always completes inside the launch.
-      // (from K = 5120 on for 8 rows and more: N=1024 K=6144 M=16 10.2 -> 7.9 us, N=2048 K=6144
-      // M=8 9.0 -> 8.0)
-      int S = (tiles > kCUs / 2 || K < (M >= 8 ? 5120 : 8192)) ? 1 : ceil_div(kCUs, tiles);
-      while (S > 1 && items / (p->waves * S) < 2) --S;  // keep two bands per wave
-      p->splitk = S;
-      p->fused = 1;
-      // with only two 256-byte bands left per wave, four of 128 bytes pipeline better
-      // (N=1024 K=8192 S=4: M=8 7.8 us against 8.9, M=16 8.0 / 9.4)
-      if (S > 1 && p->unroll == 1 && items / (p->waves * S) <= 2) p->band = 128;
-      // the same for short rows of wide outputs (K=2048 M=8: N=10240 10.6 -> 9.4 us, N=12288 M=4
-      // 11.1 -> 10.0; K=1024 N=13824 M=8 8.0 -> 7.7; K=4096 N=12288 M=6 18.5 -> 16.8)
-      if (S == 1 && p->unroll == 1 && K >= 1024 && (K <= 2048 ? N >= 8192 : (K <= 4096 && N >= 12288))) {
-        p->band = 128;
-        p->waves = 8;
-      }
-    } else {
-      p->splitk = pick_splitk(tiles, p->waves, items, M, N, K, kCUs);
-    }
-  }
-  const int st = finish_plan(M, N, K, p);
-  if (st != FG_OK) return st;
-  // In-launch completion through one fixed-point atomic per output element (fused = 2) instead of
-  // partials + arrival counter (fused = 1): one memory round trip after the K loop instead of
-  // three, but S * M * N atomics.  Measured over 11 N x 7 K x 6 M on both layouts (us gained over
-  // the counter protocol): every v_dot2 split 0.5 .. 2.5, every [N,K] split 0.3 .. 1.9; the [K,N]
-  // MFMA kernel with eight waves 0.1 .. 1.7 below 2^18 atomics or from eight splits on (up to 0.9
-  // lost otherwise), with four waves 0.8 .. 2.5 only for deep splits of few elements (1 .. 2.5 lost
-  // otherwise: K = 8192 N = 12288 M = 16, five splits, 38.4 -> 40.5).
-  if (p->splitk > 1 && p->fused == 1 && p->splitk <= kFixMaxSplit && (size_t)M * N <= kWsAccElems) {
-    const size_t atomics = (size_t)p->splitk * M * N;
-    bool atomic = true;
-    if (p->kernel == FG_KERNEL_KN_MFMA) {
-      atomic = p->waves >= 8 ? (atomics < ((size_t)1 << 18) || p->splitk >= 8)
-                             : (atomics < ((size_t)1 << 17) && p->splitk >= 8);
-    }
-    if (atomic) p->fused = 2;
-  }
-  return FG_OK;
-}
-
 int check_launch() { return hipGetLastError() == hipSuccess ? FG_OK : FG_ERR_LAUNCH; }
+
+// The planner's rules and the [K,N] kernels' band spreading count compute units: read the current
+// device's once.  Without a device (host-only planning) the count stays at MI355X's 256.
+void read_compute_units() {
+  static std::once_flag once;
+  std::call_once(once, [] {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) {
+      set_compute_units(n);
+    }
+    (void)hipGetLastError();
+  });
+}
 
 // `tail`: bias and activation bits of the kernels' flag word (0 for a plain product).
 int run_gemm(const void* A, const void* W, void* C, int M, int N, int K, int accumulate,
@@ -551,7 +49,8 @@ int run_gemm(const void* A, const void* W, void* C, int M, int N, int K, int acc
   if (ldw == 0) ldw = kn ? N : K;
   if (ldw != (kn ? N : K) && (!kn || ldw < N || ldw % 8 != 0)) return FG_ERR_INVALID_ARG;
   GemmArgs a{A, W, C, nullptr, nullptr, M, N, K,
-             (accumulate ? kFlagAccumulate : 0) | (p.stagger ? kFlagStagger : 0) | tail, bias, ldw};
+             (accumulate ? kFlagAccumulate : 0) | (p.stagger ? kFlagStagger : 0) | tail, bias, ldw,
+             compute_units()};
   if (p.splitk > 1) {
     a.ws = reinterpret_cast<float*>(static_cast<unsigned char*>(ws) + kWsHeaderBytes);
     a.counters = p.fused ? static_cast<int*>(ws) : nullptr;
@@ -632,9 +131,10 @@ const char* fg_strerror(int status) {
 
 int fg_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* out) {
   if (out == nullptr || splitk < 0) return FG_ERR_INVALID_ARG;
-  const int st = fg::validate_shape(M, N, K, w_layout);
+  fg::read_compute_units();
+  const int st = fg::plan_validate_shape(M, N, K, w_layout);
   if (st != FG_OK) return st;
-  return fg::make_plan(M, N, K, w_layout, splitk, out);
+  return fg::plan_make(M, N, K, w_layout, splitk, out);
 }
 
 size_t fg_workspace_bytes(int M, int N, int K, int w_layout, int splitk) {
@@ -704,13 +204,13 @@ int fg_gemm_f16_pitched(const void* A, const void* W, void* C, int M, int N, int
 int fg_gemm_f16_planned(const void* A, const void* W, void* C, int M, int N, int K, int w_layout,
                         int accumulate, fg_plan_t* plan, void* ws, size_t ws_bytes, void* stream) {
   if (A == nullptr || W == nullptr || C == nullptr || plan == nullptr) return FG_ERR_INVALID_ARG;
-  int st = fg::validate_shape(M, N, K, w_layout);
+  int st = fg::plan_validate_shape(M, N, K, w_layout);
   if (st != FG_OK) return st;
   if ((w_layout == FG_W_NK && !fg::is_nk(plan->kernel)) ||
       (w_layout == FG_W_KN && !fg::is_kn(plan->kernel))) {
     return FG_ERR_UNSUPPORTED;
   }
-  st = fg::finish_plan(M, N, K, plan);
+  st = fg::plan_finish(M, N, K, plan);
   if (st != FG_OK) return st;
   return fg::run_gemm(A, W, C, M, N, K, accumulate, *plan, ws, ws_bytes,
                       static_cast<hipStream_t>(stream));
@@ -730,13 +230,13 @@ int fg_gemm_f16_bias_act(const void* A, const void* W, const void* bias, int act
     if (st != FG_OK) return st;
     plan = &p;
   } else {
-    st = fg::validate_shape(M, N, K, w_layout);
+    st = fg::plan_validate_shape(M, N, K, w_layout);
     if (st != FG_OK) return st;
     if ((w_layout == FG_W_NK && !fg::is_nk(plan->kernel)) ||
         (w_layout == FG_W_KN && !fg::is_kn(plan->kernel))) {
       return FG_ERR_UNSUPPORTED;
     }
-    st = fg::finish_plan(M, N, K, plan);
+    st = fg::plan_finish(M, N, K, plan);
     if (st != FG_OK) return st;
   }
   return fg::run_gemm(A, W, C, M, N, K, 0, *plan, ws, ws_bytes, static_cast<hipStream_t>(stream),

@@ -8,6 +8,7 @@
 #include <stdint.h>
 
 #include "fg_flags.h"
+#include "fg_plan.h"
 
 namespace fg {
 
@@ -22,13 +23,10 @@ struct GemmArgs {
                    // steps); bit 4 add bias; bits 5-7 activation (FG_ACT_*)
   const void* bias;  // fp16 [N] when bit 4 is set
   int ldw;           // elements between consecutive rows of W; [K,N] kernels only (else N or K)
+  int cus;           // compute units of the device ([K,N] kernels spread column bands over them)
 };
 
 // Tile sets that exist as instantiations (the planner and the validators share these).
-bool nk_dot2_supported(int m_block, int tile_n, int unroll);
-bool nk_mfma4_supported(int m_block, int tile_n, int unroll);
-bool kn_dot2_supported(int m_block, int unroll);
-bool kn_mfma_supported(int unroll);
 
 bool launch_nk_dot2(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
 bool launch_nk_mfma4(const fg_plan_t& p, const GemmArgs& a, hipStream_t s);
@@ -57,7 +55,6 @@ void launch_dequant_i32_f16(const int32_t* acc, const void* scale, float x_scale
                             int N, hipStream_t s);
 
 // Split-K workspace: a header of arrival counters (zero between calls), then the partials.
-constexpr int kWsMaxTiles = (int)(kWsCounterBytes / sizeof(int));
 void launch_fill_zero(void* p, size_t bytes, hipStream_t s);
 
 constexpr int kStreamReadBlocks = 2048;

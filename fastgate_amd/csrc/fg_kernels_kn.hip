@@ -39,8 +39,8 @@ __device__ __forceinline__ void transpose8x8(const u32x4 (&rows)[8], u32x4 (&bt)
 // plane (x fastest), so every z plane is shifted by the number of full rounds of 256 workgroups
 // dispatched before it.  Each plane still covers every tile once, so a tile keeps one workgroup
 // per z.  K = N = 8192, M = 1 (512 workgroups): 24.2 -> 23.1 us; one workgroup a CU: unchanged.
-__device__ __forceinline__ int kn_tile(int x, int z, int gx) {
-  const int round = (int)((z * gx * gridDim.y) / 256);
+__device__ __forceinline__ int kn_tile(int x, int z, int gx, int cus) {
+  const int round = (int)((z * gx * gridDim.y) / cus);
   return (x + round) % gx;
 }
 
@@ -54,13 +54,13 @@ __global__ __launch_bounds__(64 * NW) void kn_mfma_kernel(const half_t* __restri
                                                       const half_t* __restrict__ W,
                                                       half_t* __restrict__ C,
                                                       float* __restrict__ ws, int* counters, int M, int N,
-                                                      int K, int flags, const void* bias, int ldw) {
+                                                      int K, int flags, const void* bias, int ldw, int cus) {
   __shared__ float red[NW][16][128];  // NW = most waves per workgroup
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int nw = blockDim.x >> 6;
   const int j = lane & 15, g = lane >> 4;
-  const int tile_x = kn_tile(blockIdx.x, blockIdx.z, gridDim.x);
+  const int tile_x = kn_tile(blockIdx.x, blockIdx.z, gridDim.x, cus);
   const int n0 = tile_x * 128;
   const int m0 = blockIdx.y * 16;
   const int slots = nw * gridDim.z;
@@ -181,13 +181,13 @@ __global__ __launch_bounds__(64 * NW) void kn_dot2_kernel(const half_t* __restri
                                                       const half_t* __restrict__ W,
                                                       half_t* __restrict__ C,
                                                       float* __restrict__ ws, int* counters, int M, int N,
-                                                      int K, int flags, const void* bias, int ldw) {
+                                                      int K, int flags, const void* bias, int ldw, int cus) {
   __shared__ float red[4 * NW][MB][128];  // NW = most waves per workgroup
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int nw = blockDim.x >> 6;
   const int j = lane & 15, g = lane >> 4;
-  const int tile_x = kn_tile(blockIdx.x, blockIdx.z, gridDim.x);
+  const int tile_x = kn_tile(blockIdx.x, blockIdx.z, gridDim.x, cus);
   const int n0 = tile_x * 128;
   const int m0 = blockIdx.y * MB;
   const int slots = nw * gridDim.z;
@@ -275,12 +275,6 @@ __global__ __launch_bounds__(64 * NW) void kn_dot2_kernel(const half_t* __restri
 // ---------------------------------------------------------------------------------------
 // Host launchers
 // ---------------------------------------------------------------------------------------
-bool kn_dot2_supported(int mb, int u) {
-  return (mb == 1 || mb == 2 || mb == 4 || mb == 8) && (u == 1 || u == 2 || u == 4) &&
-         !(mb == 8 && u == 4);
-}
-bool kn_mfma_supported(int u) { return u == 1 || u == 2 || u == 4; }
-
 template <int MB, int U>
 static void kn_dot2_go(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
   const dim3 grid(p.grid_x, p.grid_y, p.grid_z), block(p.block);
@@ -290,16 +284,16 @@ static void kn_dot2_go(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
   if constexpr (MB <= 2) {
     if (p.waves == 8) {
       hipLaunchKernelGGL((kn_dot2_kernel<MB, U, true, 8>), grid, block, 0, s, A, W, C, a.ws, a.counters, a.M,
-                         a.N, a.K, a.accumulate, a.bias, a.ldw);
+                         a.N, a.K, a.accumulate, a.bias, a.ldw, a.cus);
       return;
     }
   }
   if (p.stream_w)
     hipLaunchKernelGGL((kn_dot2_kernel<MB, U, true, 4>), grid, block, 0, s, A, W, C, a.ws, a.counters, a.M, a.N,
-                       a.K, a.accumulate, a.bias, a.ldw);
+                       a.K, a.accumulate, a.bias, a.ldw, a.cus);
   else
     hipLaunchKernelGGL((kn_dot2_kernel<MB, U, false, 4>), grid, block, 0, s, A, W, C, a.ws, a.counters, a.M, a.N,
-                       a.K, a.accumulate, a.bias, a.ldw);
+                       a.K, a.accumulate, a.bias, a.ldw, a.cus);
 }
 
 template <int MB>
@@ -333,13 +327,13 @@ static void kn_mfma_go(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
   auto* C = static_cast<half_t*>(a.C);
   if (p.waves == 8) {
     hipLaunchKernelGGL((kn_mfma_kernel<U, true, 8>), grid, block, 0, s, A, W, C, a.ws, a.counters, a.M, a.N, a.K,
-                       a.accumulate, a.bias, a.ldw);
+                       a.accumulate, a.bias, a.ldw, a.cus);
   } else if (p.stream_w) {
     hipLaunchKernelGGL((kn_mfma_kernel<U, true, 4>), grid, block, 0, s, A, W, C, a.ws, a.counters, a.M, a.N, a.K,
-                       a.accumulate, a.bias, a.ldw);
+                       a.accumulate, a.bias, a.ldw, a.cus);
   } else {
     hipLaunchKernelGGL((kn_mfma_kernel<U, false, 4>), grid, block, 0, s, A, W, C, a.ws, a.counters, a.M, a.N, a.K,
-                       a.accumulate, a.bias, a.ldw);
+                       a.accumulate, a.bias, a.ldw, a.cus);
   }
 }
 

@@ -362,13 +362,6 @@ __global__ __launch_bounds__(64 * NW) void nk_mfma_r_kernel(const half_t* __rest
                      static_cast<half_t*>((a).C), (a).ws, (a).counters, (a).M, (a).N, (a).K,  \
                      (a).accumulate, (a).bias)
 
-bool nk_dot2_supported(int mb, int rn, int u) {
-  const bool mb_ok = mb == 1 || mb == 2 || mb == 4 || mb == 8;
-  const bool rn_ok = rn == 4 || rn == 8 || rn == 16;
-  const bool u_ok = u == 1 || u == 2 || u == 4;
-  return mb_ok && rn_ok && u_ok && mb * rn <= 64 && rn * u <= 32;
-}
-
 template <int MB, int RN, int U>
 static void nk_dot2_go(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
   if (p.stream_w) FG_LAUNCH((nk_dot2_kernel<MB, RN, U, true>), p, a, s);
@@ -411,15 +404,6 @@ bool launch_nk_dot2(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
     case 8: return nk_dot2_rn<8>(p, a, s);
     default: return false;
   }
-}
-
-bool nk_mfma4_supported(int m_block, int tile_n, int u) {
-  const int mg = m_block / 4, r4 = tile_n / 4;
-  if (m_block % 4 || tile_n % 4) return false;
-  const bool mg_ok = mg >= 1 && mg <= 4;
-  const bool r4_ok = r4 == 1 || r4 == 2 || r4 == 4 || r4 == 8;
-  const bool u_ok = u == 1 || u == 2 || u == 4;
-  return mg_ok && r4_ok && u_ok && mg * r4 <= 16 && (mg + r4) * u <= 24;
 }
 
 template <int MG, int R4, int U>

@@ -50,20 +50,62 @@ void check_tensor(const at::Tensor& t, const char* name, at::ScalarType dtype, c
 
 // Split-K scratch, one buffer per (device, stream), grown on demand through the caching
 // allocator so that reuse is ordered on the stream that last used it.  Allocated zeroed: the
-// arrival counters at its start must be zero before the first call and every call leaves
-// them zero.
-at::Tensor workspace(const at::Tensor& like, size_t bytes) {
+// header at its start (arrival counters and accumulator words) must be zero before the first
+// call and every call leaves it zero.  The last buffer a thread used is remembered without a
+// lock; only a change of device or stream, or growth, goes to the shared table.
+struct Workspace {
+  void* ptr = nullptr;
+  size_t bytes = 0;
+};
+Workspace workspace(int device, void* stream, const at::Tensor& like, size_t bytes) {
+  struct Last {
+    int device = -1;
+    void* stream = nullptr;
+    Workspace ws;
+  };
+  static thread_local Last last;
+  if (last.device == device && last.stream == stream && last.ws.bytes >= bytes) return last.ws;
   static std::mutex mu;
   static std::map<std::pair<int, void*>, at::Tensor> cache;
   std::lock_guard<std::mutex> lock(mu);
-  const auto key = std::make_pair((int)like.device().index(), current_stream(like));
+  const auto key = std::make_pair(device, stream);
   auto it = cache.find(key);
   if (it == cache.end() || (size_t)it->second.numel() < bytes) {
-    size_t want = std::max<size_t>(bytes, (size_t)8 << 20);
+    const size_t want = std::max<size_t>(bytes, (size_t)16 << 20);
     cache[key] = at::zeros({(int64_t)want}, like.options().dtype(at::kByte));
     it = cache.find(key);
   }
-  return it->second;
+  last.device = device;
+  last.stream = stream;
+  last.ws = Workspace{it->second.data_ptr(), (size_t)it->second.numel()};
+  return last.ws;
+}
+
+// The library's plan for (M, N, K, layout), remembered per thread: planning walks a few hundred
+// lines of rules, a call of a small shape takes a few microseconds in all.
+const fg_plan_t& cached_plan(int M, int N, int K, int w_layout, int* status) {
+  struct Entry {
+    int M = 0, N = 0, K = 0, layout = -1, status = 0;
+    fg_plan_t plan;
+  };
+  static thread_local Entry table[64];
+  const unsigned h = ((unsigned)M * 2654435761u ^ (unsigned)N * 40503u ^ (unsigned)K * 2246822519u ^
+                      (unsigned)w_layout) >> 7;
+  Entry& e = table[h & 63];
+  if (e.M != M || e.N != N || e.K != K || e.layout != w_layout) {
+    e.status = fg_plan(M, N, K, w_layout, 0, &e.plan);
+    e.M = M, e.N = N, e.K = K, e.layout = w_layout;
+  }
+  *status = e.status;
+  return e.plan;
+}
+
+// Plan of a GEMM operator call.  `bz` is the reference's split-K factor, tuned for another GPU
+// (its scripts pass 1 and 2, which would leave three quarters of this one idle): it is accepted
+// and does not enter the plan.  fg_gemm_f16's own `splitk` argument is the way to force a split.
+const fg_plan_t& call_plan(int M, int N, int K, int w_layout, int bz, int* status) {
+  (void)bz;
+  return cached_plan(M, N, K, w_layout, status);
 }
 
 enum Protocol { kOverwrite = 0, kAccumulate = 1 };
@@ -77,7 +119,7 @@ void gemm(const char* op, const at::Tensor& A, const at::Tensor& W, at::Tensor& 
   const int64_t M = A.size(0), K = A.size(1);
   const int64_t N = w_layout == FG_W_KN ? W.size(1) : W.size(0);
   if (N % 128 || K % 128) throw std::invalid_argument(msg128);
-  TORCH_CHECK(bz >= 0, op, ": bz must be non-negative (0 lets the library choose)");
+  TORCH_CHECK(bz >= 0, op, ": bz must be non-negative");
   check_tensor(A, "A", at::kHalf, op);
   // B[K,N] may be a view of padded weights: rows W.stride(0) >= N elements apart (a multiple of 8),
   // unit stride along N.  The reference's tensors are dense; a pitch of N + 128 is about 9 % faster
@@ -102,14 +144,12 @@ void gemm(const char* op, const at::Tensor& A, const at::Tensor& W, at::Tensor& 
   TORCH_CHECK(M <= INT32_MAX && N <= INT32_MAX && K <= INT32_MAX, op, ": size overflow");
 
   c10::hip::HIPGuardMasqueradingAsCUDA guard(A.device());
-  const size_t ws_bytes = fg_workspace_bytes((int)M, (int)N, (int)K, w_layout, bz);
-  at::Tensor ws;
-  void* ws_ptr = nullptr;
-  if (ws_bytes) {
-    ws = workspace(A, ws_bytes);
-    ws_ptr = ws.data_ptr();
-  }
   int st;
+  fg_plan_t plan = call_plan((int)M, (int)N, (int)K, w_layout, bz, &st);
+  raise_status(st, op);
+  void* stream = current_stream(A);
+  Workspace ws;
+  if (plan.workspace_bytes) ws = workspace((int)A.device().index(), stream, A, plan.workspace_bytes);
   if (tail) {
     const void* bias_ptr = nullptr;
     if (bias.defined()) {
@@ -119,15 +159,13 @@ void gemm(const char* op, const at::Tensor& A, const at::Tensor& W, at::Tensor& 
       bias_ptr = bias.data_ptr();
     }
     st = fg_gemm_f16_bias_act(A.data_ptr(), W.data_ptr(), bias_ptr, act, C.data_ptr(), (int)M,
-                              (int)N, (int)K, w_layout, bz, nullptr, ws_ptr, ws_bytes,
-                              current_stream(A));
+                              (int)N, (int)K, w_layout, 0, &plan, ws.ptr, ws.bytes, stream);
   } else if (pitched) {
     st = fg_gemm_f16_pitched(A.data_ptr(), W.data_ptr(), C.data_ptr(), (int)M, (int)N, (int)K,
-                             (int)W.stride(0), protocol == kAccumulate, bz, ws_ptr, ws_bytes,
-                             current_stream(A));
+                             (int)W.stride(0), protocol == kAccumulate, 0, ws.ptr, ws.bytes, stream);
   } else {
-    st = fg_gemm_f16(A.data_ptr(), W.data_ptr(), C.data_ptr(), (int)M, (int)N, (int)K, w_layout,
-                     protocol == kAccumulate, bz, ws_ptr, ws_bytes, current_stream(A));
+    st = fg_gemm_f16_planned(A.data_ptr(), W.data_ptr(), C.data_ptr(), (int)M, (int)N, (int)K,
+                             w_layout, protocol == kAccumulate, &plan, ws.ptr, ws.bytes, stream);
   }
   raise_status(st, op);
 }
@@ -191,7 +229,7 @@ const OpSpec kOps3[] = {
      "C += A @ B_t.T, B_t[N,K]; C is not zeroed (hk/edgemm_tr.cu:99-116)"},
 };
 
-// (A, B, C, bz) operators: bz is the split-K factor (0 = library heuristic).
+// (A, B, C, bz) operators: bz, the reference's split-K factor, is accepted and not used.
 const OpSpec kOps4[] = {
     {"flat_gemm_m8n128k64x4_bz1", FG_W_KN, kAccumulate, kMsgNK,
      "C += A @ B, B[K,N], split-K bz (hk/flatgemm.cu:13-32)"},
@@ -229,15 +267,14 @@ void gemv_f16(const char* op, const at::Tensor& mat, const at::Tensor& vec, at::
   TORCH_CHECK(mat.device() == vec.device() && mat.device() == res.device(), op,
               ": tensors are on different devices");
   c10::hip::HIPGuardMasqueradingAsCUDA guard(mat.device());
-  const size_t ws_bytes = fg_workspace_bytes((int)M, (int)N, (int)K, FG_W_NK, 0);
-  at::Tensor ws;
-  void* ws_ptr = nullptr;
-  if (ws_bytes) {
-    ws = workspace(mat, ws_bytes);
-    ws_ptr = ws.data_ptr();
-  }
-  raise_status(fg_gemm_f16(vec.data_ptr(), mat.data_ptr(), res.data_ptr(), (int)M, (int)N, (int)K,
-                           FG_W_NK, 0, 0, ws_ptr, ws_bytes, current_stream(mat)),
+  int st;
+  fg_plan_t plan = cached_plan((int)M, (int)N, (int)K, FG_W_NK, &st);
+  raise_status(st, op);
+  void* stream = current_stream(mat);
+  Workspace ws;
+  if (plan.workspace_bytes) ws = workspace((int)mat.device().index(), stream, mat, plan.workspace_bytes);
+  raise_status(fg_gemm_f16_planned(vec.data_ptr(), mat.data_ptr(), res.data_ptr(), (int)M, (int)N, (int)K,
+                                   FG_W_NK, 0, &plan, ws.ptr, ws.bytes, stream),
                op);
 }
 
@@ -364,10 +401,7 @@ void hgemm(at::Tensor A, at::Tensor B, at::Tensor C) { at::matmul_out(C, A, B); 
 void hgemm_tr(at::Tensor A, at::Tensor B, at::Tensor C) { at::matmul_out(C, A, B.t()); }
 void mma(at::Tensor A, at::Tensor B, at::Tensor C) { at::matmul_out(C, A, B.t()); }
 
-py::dict plan(int M, int N, int K, int w_layout, int splitk) {
-  fg_plan_t p;
-  const int st = fg_plan(M, N, K, w_layout, splitk, &p);
-  raise_status(st, "plan");
+py::dict plan_dict(const fg_plan_t& p) {
   py::dict d;
   d["kernel"] = p.kernel;
   d["splitk"] = p.splitk;
@@ -383,6 +417,29 @@ py::dict plan(int M, int N, int K, int w_layout, int splitk) {
   d["block"] = p.block;
   d["workspace_bytes"] = p.workspace_bytes;
   return d;
+}
+
+py::dict plan(int M, int N, int K, int w_layout, int splitk) {
+  fg_plan_t p;
+  const int st = fg_plan(M, N, K, w_layout, splitk, &p);
+  raise_status(st, "plan");
+  return plan_dict(p);
+}
+
+// The plan operator `name` runs for a shape and a `bz` argument (host only).
+py::dict plan_dict(const fg_plan_t& p);
+py::dict plan_for(const std::string& name, int M, int N, int K, int bz) {
+  const OpSpec* spec = nullptr;
+  for (const OpSpec& s : kOps3)
+    if (name == s.name) spec = &s;
+  for (const OpSpec& s : kOps4)
+    if (name == s.name) spec = &s;
+  if (spec == nullptr) throw std::invalid_argument("plan_for: unknown GEMM operator " + name);
+  if (N % 128 || K % 128) throw std::invalid_argument(spec->msg);
+  int st;
+  const fg_plan_t p = call_plan(M, N, K, spec->layout, bz, &st);
+  raise_status(st, "plan_for");
+  return plan_dict(p);
 }
 
 }  // namespace
@@ -463,6 +520,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("mma", &mma, "C = A @ B_t.T through the vendor GEMM (czn/mma.cu:19-88)");
   m.def("plan", &plan, py::arg("M"), py::arg("N"), py::arg("K"), py::arg("w_layout"),
         py::arg("splitk") = 0, "launch plan the library picks for a shape (host only)");
+  m.def("plan_for", &plan_for, py::arg("name"), py::arg("M"), py::arg("N"), py::arg("K"), py::arg("bz") = 0,
+        "launch plan operator `name` uses for a shape; bz is accepted and does not enter (host only)");
   m.attr("W_KN") = (int)FG_W_KN;
   m.attr("W_NK") = (int)FG_W_NK;
 }

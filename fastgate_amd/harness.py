@@ -8,7 +8,10 @@ What is kept, with the line of the reference it follows:
   * timing (:125-137): `warmup` untimed calls, then `iters` calls each bracketed by a device
     synchronize and a host clock; the figure is the mean in milliseconds per call;
   * verdicts: the share of outputs within 100 of torch.matmul (:152-166) and
-    torch.allclose(rtol=1e-1, atol=1e-2) (:236).
+    torch.allclose(rtol=1e-1, atol=1e-2) (:236);
+  * the per-operator check of `iter_func` (:190-250): inputs uniform in [0, 1), the operator called
+    twice on fresh outputs, the two runs compared, the first compared with torch.matmul, then
+    torch and the operator timed with the same loop.
 The vendor column (`hgemm`, cuBLAS in the reference) is this library's `hgemm`, i.e. hipBLASLt
 through ATen.  Nothing here computes on the CPU.
 """
@@ -121,6 +124,41 @@ def run_config(funcs, M: int, K: int, N: int, warmup: int = WARMUP, iters: int =
         entry["ms"] = speed_test(lambda: dispatch_func_btrans(f, A, B_T, C_t, bz), warmup, iters)
         row["ops"][_name(f)] = entry
     return row
+
+
+def iter_func(funcs, configs, warmup: int = WARMUP, iters: int = ITERS, device="cuda", seed: int = 10):
+    """script/standard-test.py:190-250 for every (operator, (M, K, N)): A, B uniform in [0, 1) with
+    columns -4:-2 of B divided by 100; the operator runs twice, on two zeroed outputs; the runs are
+    compared with each other (allclose in the reference; here the bits are compared as well, since
+    the operators are reproducible run to run) and the first with torch.matmul; then torch.matmul
+    and the operator are timed.  The reference calls every operator as func(A, B, C); the calling
+    convention of each name (weight first, transposed weight, trailing bz) is applied here as
+    dispatch_func does.  Returns one dict per (operator, config)."""
+    out = []
+    for f in funcs:
+        for (M, K, N) in configs:
+            g = torch.Generator(device=device).manual_seed(seed)
+            A = torch.rand((M, K), dtype=torch.float16, device=device, generator=g)
+            B = torch.rand((K, N), dtype=torch.float16, device=device, generator=g)
+            B[:, -4:-2] = B[:, -4:-2] / 100
+            C_ref = torch.zeros((M, N), dtype=torch.float16, device=device)
+            C = torch.zeros_like(C_ref)
+            C2 = torch.zeros_like(C_ref)
+            B_T = B.transpose(0, 1).contiguous()
+            torch.matmul(A, B, out=C_ref)
+            dispatch_func_btrans(f, A, B_T, C)
+            torch.cuda.synchronize()
+            dispatch_func_btrans(f, A, B_T, C2)
+            torch.cuda.synchronize()
+            entry = {"op": _name(f), "M": M, "K": K, "N": N,
+                     "runs_allclose": bool(torch.allclose(C2, C, rtol=1e-1, atol=1e-2)),
+                     "runs_bitwise_equal": bool(torch.equal(C2.view(torch.int16), C.view(torch.int16))),
+                     "allclose_to_torch": bool(torch.allclose(C_ref, C, rtol=1e-1, atol=1e-2))}
+            entry["torch_ms"] = speed_test(lambda: torch.matmul(A, B, out=C_ref), warmup, iters)
+            C_t = torch.zeros_like(C_ref)
+            entry["ms"] = speed_test(lambda: dispatch_func_btrans(f, A, B_T, C_t), warmup, iters)
+            out.append(entry)
+    return out
 
 
 def format_row(row) -> str:

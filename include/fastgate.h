@@ -96,7 +96,8 @@ typedef struct fg_plan_t {
 /*
  * C = A·W (accumulate = 0) or C += A·W (accumulate = 1; C holds fp16 on entry and the sum
  * is formed in fp32 before the single rounding).
- *   splitk  0 = library heuristic, S >= 1 = forced (the reference's trailing `int bz`).  With 0 and
+ *   splitk  0 = library heuristic, S >= 1 = forced.  (The reference's trailing `int bz` is a split
+ *           factor tuned for another GPU; the pybind layer accepts it and passes 0 here.)  With 0 and
  *           no (or too small a) workspace the call runs unsplit instead of failing; a forced
  *           S > 1 without workspace is FG_ERR_WORKSPACE.
  *   ws      device scratch of at least fg_workspace_bytes() bytes when the plan's

@@ -194,6 +194,20 @@ def test_reference_harness_flow(device):
     assert all(e["allclose"] for e in row["ops"].values())
 
 
+def test_reference_iter_func_flow(device):
+    # script/standard-test.py:190-250: each operator twice on fresh outputs, run against run (here
+    # bit for bit), run against torch.matmul, then the timing loops
+    import eed.backend as backend
+    from fastgate_amd import harness
+    funcs = [backend.edgemm_m8n128k64x4, backend.edgemm_m8n128k64x4_bt, backend.flat_gemm_m8n256k32x16,
+             backend.gemm_m8n64k128x8_bt_exp, backend.fastgemv_extend]
+    rows = harness.iter_func(funcs, [(8, 1024, 2048), (1, 4096, 1024), (16, 2048, 1152)], warmup=1, iters=2)
+    assert len(rows) == len(funcs) * 3
+    for e in rows:
+        assert e["runs_allclose"] and e["runs_bitwise_equal"] and e["allclose_to_torch"], e
+        assert e["ms"] > 0 and e["torch_ms"] > 0
+
+
 def test_operators_replay_correctly_from_a_hip_graph(device):
     # serving loops capture the calls once and replay them: every launch (split-K second pass and
     # in-launch completion included) must be capturable and give the eager result on each replay

@@ -326,3 +326,25 @@ def test_row_count_beyond_the_grid_limit_is_rejected():
     assert capi.lib().fg_plan(32 * 65535, 128, 128, capi.FG_W_NK, 0, ctypes.byref(p)) == capi.FG_OK
     assert capi.lib().fg_plan(16 * 65535 + 1, 128, 128, capi.FG_W_KN, 0, ctypes.byref(p)) == capi.FG_ERR_INVALID_ARG
     assert capi.lib().fg_plan(16 * 65535, 128, 128, capi.FG_W_KN, 0, ctypes.byref(p)) == capi.FG_OK
+
+
+def test_bz_does_not_change_the_launch(sg):
+    """The reference's callers pass bz = 1 or 2 (script/standard-test.py:176), its hosts note
+    'orig BZ=2' / 'orig BZ=8' (hk/flatgemm.cu:26,69): split factors of another GPU.  Every
+    bz-taking name must run the plan the library picks by itself, and that plan fills the chip."""
+    import oracle
+
+    for name, (layout, _protocol, has_bz) in oracle.GEMM_OPS.items():
+        if not has_bz:
+            continue
+        for M in (1, 8, 16):
+            auto = sg.plan_for(name, M, 8192, 8192, 0)
+            assert auto == sg.plan(M, 8192, 8192, layout, 0)
+            for bz in (1, 2, 8):
+                assert sg.plan_for(name, M, 8192, 8192, bz) == auto, (name, M, bz)
+            gx, gy, gz = auto["grid"]
+            assert gx * gy * gz >= 192, (name, M, auto)
+    with pytest.raises(ValueError):
+        sg.plan_for("flat_gemm_m8n256k64x8", 8, 8192, 8200, 1)
+    with pytest.raises(ValueError):
+        sg.plan_for("no_such_operator", 8, 8192, 8192, 1)
