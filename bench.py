@@ -37,28 +37,84 @@ MS = (1, 8, 16)
 R = 5  # weight buffers per layout
 HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E peak
 
-# HBM bytes per launch from two rocprofv3 --pmc runs of this script (FETCH_SIZE, then WRITE_SIZE,
-# KiB per dispatch), keyed by kernel family and M.  Each counter is scaled by what it reads for
-# kernels of known traffic (--calibrate-traffic: a 1 GiB read and a 256 MiB copy): FETCH_SIZE
-# reports half the bytes on this part (factor 2.0), WRITE_SIZE all of them (factor 1.0).
-# A kernel/M not listed reports null.
-FETCH_SCALE, WRITE_SCALE = 2.0, 1.0
+# HBM bytes per launch (`roofline.traffic`) come from bench_traffic.json beside this file: the
+# FETCH_SIZE and WRITE_SIZE counters (KiB per dispatch) of two rocprofv3 --pmc runs of this script,
+# each scaled by what the same counter reads for kernels of known traffic (--calibrate-traffic: a
+# 1 GiB read and a 256 MiB copy).  `bench.py --ingest-pmc DIR` rewrites the file from the CSV output
+# of those runs.  Entries are keyed by kernel AND launch plan, so a figure taken under another plan
+# is not reported: a call whose key is missing gets null.
+TRAFFIC_FILE = ROOT / "bench_traffic.json"
 
 
-def _traffic(fetch_kib: float, write_kib: float) -> int:
-    return int(round((fetch_kib * FETCH_SCALE + write_kib * WRITE_SCALE) * 1024))
+def plan_key(p: dict, M: int) -> str:
+    return "%s|M%d|S%d|w%d|f%d|t%d|u%d" % (p["kernel_name"], M, p["splitk"], p["waves"], p["fused"] if p["splitk"] > 1 else 0,
+                                           p["tile_n"], p["unroll"])
 
 
-TRAFFIC_BYTES = {
-    "nk_dot2_M1": _traffic(65630.6, 64.0),
-    "nk_mfma_r_M8": _traffic(66083.0, 128.0),
-    "nk_mfma_r_M16": _traffic(66604.5, 256.0),
-    # [K,N]: split-K partials are written through and read back inside the launch; WRITE_SIZE counts
-    # the write-through stores twice (M=1: 8 x 16 KiB of partials, M=8: 8 x 256 KiB, M=16: 4 x 512 KiB)
-    "kn_dot2_M1": _traffic(65787.4, 290.0),
-    "kn_mfma_M8": _traffic(67145.6, 4242.0),
-    "kn_mfma_M16": _traffic(67667.5, 4362.0),
-}
+def load_traffic() -> dict:
+    try:
+        return json.loads(TRAFFIC_FILE.read_text()).get("entries", {})
+    except (OSError, ValueError):
+        return {}
+
+
+def ingest_pmc(directory: Path, capi) -> int:
+    """Rewrites bench_traffic.json from DIR/pmc_FETCH_SIZE, DIR/pmc_WRITE_SIZE (this script under
+    rocprofv3 --pmc) and DIR/cal_FETCH_SIZE, DIR/cal_WRITE_SIZE (--calibrate-traffic under the same).
+    Dispatches are matched to the six calls of the step by kernel family, grid and workgroup size."""
+    import csv
+    import re
+
+    def rows(sub):
+        out = []
+        for f in sorted((directory / sub).rglob("*counter_collection.csv")):
+            with open(f, newline="") as fh:
+                out += list(csv.DictReader(fh))
+        return out
+
+    def mean(rs):
+        return sum(float(r["Counter_Value"]) for r in rs) / len(rs) if rs else None
+
+    scale = {}
+    for counter, known in (("FETCH_SIZE", [("stream_read_kernel", (1 << 30) / 1024.0), ("copyBuffer", (256 << 20) / 1024.0)]),
+                           ("WRITE_SIZE", [("copyBuffer", (256 << 20) / 1024.0)])):
+        cal = rows("cal_" + counter)
+        factors = []
+        for frag, true_kib in known:
+            got = mean([r for r in cal if frag in r["Kernel_Name"] and r["Counter_Name"] == counter])
+            if got:
+                factors.append(true_kib / got)
+        if not factors:
+            print("bench.py: no calibration rows for %s under %s" % (counter, directory), file=sys.stderr)
+            return 2
+        scale[counter] = sum(factors) / len(factors)
+    entries = {}
+    for M, layout in ((1, capi.FG_W_NK), (8, capi.FG_W_NK), (16, capi.FG_W_NK), (1, capi.FG_W_KN), (8, capi.FG_W_KN), (16, capi.FG_W_KN)):
+        p = capi.plan(M, N, K, layout).as_dict()
+        wgs = p["grid_x"] * p["grid_y"] * p["grid_z"]
+        vals = {}
+        for counter in ("FETCH_SIZE", "WRITE_SIZE"):
+            def match(r):
+                # names come demangled (fg::kn_mfma_kernel<2, true, 8>) or mangled (_ZN2fg14kn_mfma_kernelILi2E...)
+                if r["Counter_Name"] != counter or not re.search(r"fg(::|\d+)%s_kernel" % p["kernel_name"], r["Kernel_Name"]):
+                    return False
+                if int(r["Workgroup_Size"]) != p["block"] or int(r["Grid_Size"]) != wgs * p["block"]:
+                    return False
+                if p["kernel_name"] == "nk_mfma_r":   # M = 8 and 16 share grid and block: first template argument
+                    m = re.search(r"nk_mfma_r_kernel(?:<|ILi)(\d+)", r["Kernel_Name"])
+                    return m is not None and int(m.group(1)) == (8 if M <= 8 else 16)
+                return True
+            vals[counter] = mean([r for r in rows("pmc_" + counter) if match(r)])
+        if vals["FETCH_SIZE"] is None or vals["WRITE_SIZE"] is None:
+            print("bench.py: no dispatch matches %s" % plan_key(p, M), file=sys.stderr)
+            continue
+        entries[plan_key(p, M)] = {
+            "fetch_kib": round(vals["FETCH_SIZE"], 1), "write_kib": round(vals["WRITE_SIZE"], 1),
+            "bytes": int(round((vals["FETCH_SIZE"] * scale["FETCH_SIZE"] + vals["WRITE_SIZE"] * scale["WRITE_SIZE"]) * 1024)),
+            "algorithmic_bytes": algorithmic_bytes(M)}
+    TRAFFIC_FILE.write_text(json.dumps({"scale": {k: round(v, 4) for k, v in scale.items()}, "entries": entries}, indent=1) + "\n")
+    print(json.dumps({"written": str(TRAFFIC_FILE.name), "entries": len(entries), "scale": scale}))
+    return 0
 
 
 def algorithmic_bytes(M: int) -> int:
@@ -273,12 +329,19 @@ def main() -> int:
     ap.add_argument("--sweep-models", action="store_true",
                     help="as --sweep, over the projection shapes of common decoder layers (both layouts, M = 1, 8, 16)")
     ap.add_argument("--cpu-repeats", type=int, default=8, help="repetitions of the step on the CPU oracle (0 = skip)")
+    ap.add_argument("--ingest-pmc", metavar="DIR", default=None,
+                    help="host only: rewrite bench_traffic.json from DIR/{pmc,cal}_{FETCH,WRITE}_SIZE, the CSV output of "
+                         "this script and of --calibrate-traffic under rocprofv3 --pmc, then exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU; --gpus %d is not supported "
               "(the path shards by output columns without any collective; each GPU would run this same kernel on its share)" % args.gpus,
               file=sys.stderr)
         return 2
+
+    if args.ingest_pmc:
+        from fastgate_amd import capi as capi_host
+        return ingest_pmc(Path(args.ingest_pmc), capi_host)
 
     import numpy as np
     import torch
@@ -418,12 +481,45 @@ def main() -> int:
         per_call.append({
             "op": label, "M": M, "w_layout": "[N,K]" if layout == capi.FG_W_NK else "[K,N]",
             "kernel": p["kernel_name"], "splitk": p["splitk"], "tile_n": p["tile_n"], "waves": p["waves"],
-            "unroll": p["unroll"], "launches": 1 + (p["splitk"] > 1 and not p["fused"]),
+            "unroll": p["unroll"], "completion": ("second kernel", "counter", "atomic")[p["fused"]] if p["splitk"] > 1 else "-",
+            "plan_key": plan_key(p, M), "launches": 1 + (p["splitk"] > 1 and not p["fused"]),
             "bytes": algorithmic_bytes(M), "us_per_call": round(us, 2), "GBps": round(gbps, 1),
             "us_per_call_single_buffer": round(us_hot, 2),
             "TFLOPs": round(2.0 * M * N * K / (us * 1e-6) / 1e12, 2),
             "frac_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4),
             "frac_read_ceiling": round(gbps / ceiling_gbps, 4)})
+
+    # ---- int8 GEMV (fastgemv_int8, K = N = 8192, per-channel scale) against the fp16 GEMV of the
+    # same shape: the two alternate, `steps` back-to-back launches each, five rounds; the ratio of
+    # the medians is the int8 path's weight throughput relative to fp16 (target 1.8) ---------------
+    gi = torch.Generator(device=dev).manual_seed(1004)
+    wq = [torch.randint(-127, 128, (N, K), device=dev, generator=gi, dtype=torch.int8) for _ in range(2 * R)]
+    xi = torch.randn((1, K), device=dev, generator=gi).half()
+    sc = (torch.rand(N, device=dev, generator=gi) * 0.009 + 0.001).half()
+    yi = torch.empty(N, dtype=torch.half, device=dev)
+
+    def timed(fn):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        barrier()
+        e0.record()
+        for s_ in range(args.steps):
+            fn(s_)
+        e1.record()
+        barrier()
+        return e0.elapsed_time(e1) * 1e3 / args.steps
+
+    t_i8, t_f16 = [], []
+    for _ in range(5):
+        t_f16.append(timed(lambda i: sg.fastgemv(w_nk[i % R], acts_d[1], y1)))
+        t_i8.append(timed(lambda i: sg.fastgemv_int8(wq[i % (2 * R)], xi, yi, scale=sc)))
+    us_i8, us_f16 = sorted(t_i8)[2], sorted(t_f16)[2]
+    i8_bytes = K * N + 2 * K + 2 * N + 2 * N
+    int8 = {"op": "fastgemv_int8", "M": 1, "K": K, "N": N, "kernel": "w8a16_m1", "bytes": i8_bytes,
+            "us_per_call": round(us_i8, 2), "GBps": round(i8_bytes / us_i8 / 1e3, 1),
+            "frac_read_ceiling": round(i8_bytes / us_i8 / 1e3 / ceiling_gbps, 4),
+            "fp16_fastgemv_us_per_call": round(us_f16, 2),
+            "weight_throughput_vs_fp16": round(us_f16 / us_i8, 3), "target": 1.8}
+    del wq
 
     # The roofline entry describes the single-launch call that takes the longest: its time between
     # the events is one kernel's launch-to-launch time, which the rocprofv3 kernel trace must match.
@@ -432,7 +528,7 @@ def main() -> int:
     roofline = {
         "bound": "hbm", "achieved": dom["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
         "frac": round(dom["GBps"] / HBM_PEAK_GBPS, 4),
-        "traffic": TRAFFIC_BYTES.get("%s_M%d" % (dom["kernel"], dom["M"])),
+        "traffic": (load_traffic().get(dom["plan_key"]) or {}).get("bytes"),
         "kernel": "%s (%s M=%d %s)" % (dom["kernel"], dom["op"], dom["M"], dom["w_layout"]),
         "launches_in_call": dom["launches"], "us": dom["us_per_call"],
         "algorithmic_bytes": dom["bytes"], "measured_read_ceiling_GBps": round(ceiling_gbps, 1),
@@ -491,6 +587,7 @@ def main() -> int:
         "read_ceiling_GBps": round(ceiling_gbps, 1), "frac_read_ceiling": round(value / ceiling_gbps, 4),
         "copy_ceiling_GBps": round(copy_gbps, 1),
         "per_call": per_call,
+        "int8_gemv": int8,
     }
     print(json.dumps(out))
     return 0
