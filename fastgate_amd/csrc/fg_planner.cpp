@@ -348,12 +348,13 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
     }
   } else {
     const size_t weights = (size_t)N * K;
-    const bool dot2_m1 = weights < ((size_t)1 << 27) || (weights < ((size_t)1 << 28) && N >= 25600);
-    if (M == 1 ? dot2_m1 : (M == 2 && weights < ((size_t)1 << 27))) {
-      // (at K = N = 16384 the MFMA kernel streams better even for M = 1: 80 us against 90; two rows
-      // from 2^27 weights on: K=8192 N=16384 43.7 / 46.0, K=28672 N=8192 76.5 / 78.4, K=8192 N=28672
-      // 73.9 / 75.3; one row too where such weights still need a split: K=11008 N=16384 56.7 / 59.9,
-      // K=14336 N=16384 71.7 / 77.2, while K=8192 N=28672, unsplit, is 74.9 / 73.8)
+    if (M <= 2 && (weights < ((size_t)1 << 27) || (weights < ((size_t)1 << 28) && (M == 1 || N <= 12288)))) {
+      // One or two rows take the v_dot2 kernel up to 2^28 weights: its deep splits cost little now
+      // that they complete through one atomic per element (M = 1, v_dot2 / MFMA kernel, us:
+      // K=16384 N=8192 42.5 / 45.4, K=11008 N=12288 42.8 / 45.6, K=16384 N=12288 62.0 / 66.2,
+      // K=8192 N=16384 42.2 / 44.0; at K = N = 16384 the two are level and the MFMA kernel stays;
+      // two rows from 2^27 weights on only up to N = 12288: K=16384 N=12288 63.2 / 66.1, but
+      // K=16384 N=14336 76.0 / 74.0).
       p->kernel = FG_KERNEL_KN_DOT2;
       p->m_block = M;
     } else {
@@ -393,15 +394,28 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
         // aim at 128 there (N=2048: K=4096 M=1 9.7 -> 8.1 us, M=16 10.8 -> 9.0; K=8192 12.0 -> 10.6).
         // Eight tiles with long K take a 24-way split (N=1024 K=28672: M=1 15.3 -> 13.8, M=16 17.9
         // -> 16.2) as long as every wave keeps two units.
-        p->waves = 8;
+        // Sixteen column tiles or fewer: with the atomic completion a deep split is cheap, so the
+        // grid aims at every CU (one or two rows: one and a half workgroups of four waves a CU)
+        // instead of half of them (N=2048 K=8192, 8 ways -> deeper: M=1 9.9 -> 8.1 us, M=8 11.3 ->
+        // 9.8, M=16 12.2 -> 11.4; N=2048 K=16384 M=1 14.0 -> 12.7; N=1024 K=11008 M=4 8.7 -> 7.7).
+        // For nine rows and more splits of 3, 6 and 12 are offered too (K = N = 4096 M=16: 6 ways
+        // 10.9 us, 8 ways 11.7).
+        // Eight tiles keep eight waves and three quarters of the CUs (N=1024 K=16384 M=1: 24 ways
+        // of eight waves 8.6 us, 31 ways of four 9.3); nine rows and more go from 192 to 256
+        // workgroups beyond K = 8192 (N=2048 M=16: K=8192 12 ways 11.3 us / 16 ways 12+, K=16384
+        // 17.6 / 16.7).
+        const bool narrow = tiles <= 16;
+        p->waves = (narrow && tiles > 8 && M <= 2) ? 4 : 8;
         p->fused = 1;
-        half_filled = tiles <= 16 && K <= 8192;
-        const double target = half_filled ? 128.0 : 192.0;
+        half_filled = narrow;  // (keeps the search over every integer split below out of this range)
+        double target = 192.0;
+        if (narrow && tiles > 8) target = M <= 2 ? 384.0 : ((M <= 8 || K > 8192) ? 256.0 : 192.0);
         double best_dist = 1e30;
-        static const int kSplits[] = {1, 2, 4, 8, 16, 24};
+        static const int kSplits[] = {1, 2, 3, 4, 6, 8, 12, 16, 24, 31};
         for (int S : kSplits) {
+          if ((S == 3 || S == 6 || S == 12) && M <= 8) continue;
           if (items / (p->waves * S) < 1) break;
-          if (S > 16 && (tiles > 8 || items / (p->waves * S) < 2)) break;
+          if (S > 16 && !narrow) break;
           // 9..16 rows: the partials of a split that leaves a wave one unit cost more than the
           // idle CUs once there are more than 192 workgroups (N=4096 K=2048 M=12: 8 ways 10.3 us,
           // 4 ways 8.3; N=2048 K=2048 M=16: 8 ways 7.4, 4 ways 7.9)
@@ -429,11 +443,25 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
           }
         }
       }
+      // v_dot2 on 2^27 weights and more: four waves, each left with about eight 32-row units, up to
+      // four workgroups a CU (K=16384 N=8192 M=1: 16 ways 42.5 us, 4 ways 45+)
+      bool deep_dot2 = false;
+      if (p->kernel == FG_KERNEL_KN_DOT2 && (size_t)N * K >= ((size_t)1 << 27)) {
+        static const int kDeep[] = {16, 10, 8, 5, 4, 2};
+        for (int S : kDeep) {
+          if (tiles * S <= 4 * kCUs && items / (4 * S) >= 8) {
+            best = S;
+            p->waves = 4;
+            deep_dot2 = true;
+            break;
+          }
+        }
+      }
       p->splitk = best;
       // the v_dot2 kernel wants eight waves on every CU: K=4096 N=16384, M = 1, S = 2:
       // 26.9 us with four waves a workgroup, 24.3 with eight
       if (p->kernel == FG_KERNEL_KN_DOT2 && p->waves == 4 && tiles * best < 2 * kCUs &&
-          items / (8 * best) >= 2) {
+          items / (8 * best) >= 2 && !deep_dot2 && !half_filled) {
         p->waves = 8;
       }
       // 9..16 rows at 8192 x 8192: 26.0 us with eight waves against 26.5 with four (at 16384 x 16384
@@ -459,7 +487,9 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
           // 9..16 rows: two 4-wave workgroups a CU write twice the partials of one 8-wave workgroup
           // for the same K range and lose to it at equal fill (N=5120 K=8192 M=16: 11 splits of 4
           // waves 20.4 us, 5 of 8 waves 19.2; N=9216 K=4096 18.2 / 17.6)
-          const double two_a_cu = (M > 8 && w == 4) ? 0.88 : 1.0;
+          // (four rows and more, too, since the split completes through atomics: N=5120 K=4096 M=8
+          // 11 splits of 4 waves 11.8 us, 6 of 8 waves 10.9)
+          const double two_a_cu = w == 4 ? (M > 8 ? 0.88 : (M >= 4 ? 0.94 : 1.0)) : 1.0;
           return fill * balance(items, w * S) * partials * chain * two_a_cu;
         };
         const int n0 = tiles * p->splitk;
@@ -539,16 +569,16 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
   // In-launch completion through one fixed-point atomic per output element (fused = 2) instead of
   // partials + arrival counter (fused = 1): one memory round trip after the K loop instead of
   // three, but S * M * N atomics.  Measured over 11 N x 7 K x 6 M on both layouts (us gained over
-  // the counter protocol): every v_dot2 split 0.5 .. 2.5, every [N,K] split 0.3 .. 1.9; the [K,N]
-  // MFMA kernel with eight waves 0.1 .. 1.7 below 2^18 atomics or from eight splits on (up to 0.9
-  // lost otherwise), with four waves 0.8 .. 2.5 only for deep splits of few elements (1 .. 2.5 lost
-  // otherwise: K = 8192 N = 12288 M = 16, five splits, 38.4 -> 40.5).
+  // the counter protocol, 514 splits): every v_dot2 split 0.5 .. 2.5, every [N,K] split 0.3 .. 1.9;
+  // the [K,N] MFMA kernel with eight waves 0.1 .. 1.8 below 5 * 2^16 atomics or from eight splits
+  // on (0.1 .. 1.4 lost otherwise), with four waves 0.4 on average below 2^16 atomics, level for
+  // deep splits and 0.4 .. 1.4 lost otherwise (K = 8192 N = 12288 M = 16, five splits).
   if (p->splitk > 1 && p->fused == 1 && p->splitk <= kFixMaxSplit && (size_t)M * N <= kWsAccElems) {
     const size_t atomics = (size_t)p->splitk * M * N;
     bool atomic = true;
     if (p->kernel == FG_KERNEL_KN_MFMA) {
-      atomic = p->waves >= 8 ? (atomics < ((size_t)1 << 18) || p->splitk >= 8)
-                             : (atomics < ((size_t)1 << 17) && p->splitk >= 8);
+      atomic = p->waves >= 8 ? (atomics < ((size_t)5 << 16) || p->splitk >= 8)
+                             : (atomics < ((size_t)1 << 16) || (p->splitk >= 8 && atomics < ((size_t)1 << 19)));
     }
     if (atomic) p->fused = 2;
   }

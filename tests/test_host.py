@@ -116,12 +116,26 @@ def test_plan_choices_that_were_measured():
     assert (p.unroll, p.stagger) == (2, 0)
     assert nk(1, 16384, 16384).kernel == capi.FG_KERNEL_NK_MFMA4
     # [K,N]
-    assert kn(1, 2048, 4096).splitk == 8 and kn(1, 2048, 16384).splitk == 16
-    assert kn(16, 1024, 28672).splitk == 24 and kn(16, 1024, 8192).splitk == 16
+    # sixteen column tiles or fewer: deep splits (they complete through atomics), four waves for one
+    # or two rows from nine tiles on
+    for (M, N, K, S, W) in ((1, 2048, 4096, 24, 4), (1, 2048, 16384, 24, 4), (8, 2048, 8192, 16, 8),
+                            (16, 2048, 8192, 12, 8), (16, 2048, 16384, 16, 8), (1, 1024, 16384, 24, 8),
+                            (16, 1024, 28672, 24, 8), (16, 1024, 8192, 24, 8)):
+        p = kn(M, N, K)
+        assert (p.splitk, p.waves, p.fused) == (S, W, 2), (M, N, K, p.as_dict())
+    # one or two rows: v_dot2 up to 2^28 weights (two rows beyond 2^27 only up to N = 12288)
     assert kn(2, 16384, 8192).kernel == capi.FG_KERNEL_KN_MFMA
-    assert kn(1, 16384, 8192).kernel == capi.FG_KERNEL_KN_MFMA
+    assert kn(2, 14336, 16384).kernel == capi.FG_KERNEL_KN_MFMA
+    assert kn(1, 16384, 16384).kernel == capi.FG_KERNEL_KN_MFMA
     assert kn(1, 28672, 8192).kernel == capi.FG_KERNEL_KN_DOT2
     assert kn(1, 8192, 8192).kernel == capi.FG_KERNEL_KN_DOT2
+    for (M, N, K, S) in ((1, 16384, 8192, 8), (1, 8192, 16384, 16), (2, 12288, 16384, 10)):
+        p = kn(M, N, K)
+        assert (p.kernel, p.splitk, p.waves) == (capi.FG_KERNEL_KN_DOT2, S, 4), (M, N, K, p.as_dict())
+    # completion of the split: atomics for v_dot2, for [N,K] and for few elements; the counter otherwise
+    assert kn(1, 8192, 8192).fused == 2 and kn(8, 4096, 4096).fused == 2 and nk(16, 2048, 8192).fused == 2
+    assert kn(8, 8192, 8192).fused == 1 and kn(16, 8192, 8192).fused == 1 and kn(16, 12288, 8192).fused == 1
+    assert kn(24, 2048, 4096).fused == 0           # more than 16 rows: second kernel
     p = kn(16, 5120, 8192)
     assert (p.splitk, p.waves) == (6, 8)
     p = kn(12, 4096, 2048)
