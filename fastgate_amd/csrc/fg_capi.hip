@@ -132,9 +132,28 @@ const char* fg_strerror(int status) {
 int fg_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* out) {
   if (out == nullptr || splitk < 0) return FG_ERR_INVALID_ARG;
   fg::read_compute_units();
-  const int st = fg::plan_validate_shape(M, N, K, w_layout);
+  int st = fg::plan_validate_shape(M, N, K, w_layout);
   if (st != FG_OK) return st;
-  return fg::plan_make(M, N, K, w_layout, splitk, out);
+  st = fg::plan_make(M, N, K, w_layout, splitk, out);
+  if (st != FG_OK) return st;
+  // FASTGATE_SPLITK_COMPLETION = two-pass | counter | atomic (read once) overrides how the
+  // library's plans complete a split: a way back to the second kernel, whose only communication
+  // is the kernel boundary, without rebuilding.
+  static const int forced = [] {
+    const char* e = std::getenv("FASTGATE_SPLITK_COMPLETION");
+    if (e == nullptr) return -1;
+    if (std::strcmp(e, "two-pass") == 0) return 0;
+    if (std::strcmp(e, "counter") == 0) return 1;
+    if (std::strcmp(e, "atomic") == 0) return 2;
+    return -1;
+  }();
+  if (forced >= 0 && out->splitk > 1) {
+    fg_plan_t q = *out;
+    q.fused = forced;
+    if (forced == 2 && (q.splitk > fg::kFixMaxSplit || (size_t)M * N > fg::kWsAccElems)) q.fused = 1;
+    if (fg::plan_finish(M, N, K, &q) == FG_OK) *out = q;
+  }
+  return FG_OK;
 }
 
 size_t fg_workspace_bytes(int M, int N, int K, int w_layout, int splitk) {

@@ -200,7 +200,13 @@ __device__ __forceinline__ bool splitk_last_arriver(int* counter, int S) {
   // alone does not do that: the waves of a workgroup share a CU, so the compiler emits no wait
   // for it, and an arrival could overtake a partial on its way through another L2 channel.
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0); expcnt and lgkmcnt left alone
+  // s_waitcnt immediate of gfx9 (gfx950 included): vmcnt in bits 3:0 and 15:14, expcnt in 6:4,
+  // lgkmcnt in 11:8.  vmcnt = 0 waits for every outstanding vector-memory access of the wave; the
+  // other two counters are left at their largest value, which waits for nothing.
+  constexpr int kVmcnt = 0, kExpcntNoWait = 7, kLgkmcntNoWait = 15;
+  constexpr int kWaitStores = (kVmcnt & 15) | (kExpcntNoWait << 4) | (kLgkmcntNoWait << 8) | ((kVmcnt >> 4) << 14);
+  static_assert(kWaitStores == 0x0F70, "s_waitcnt vmcnt(0) in the gfx9 encoding");
+  __builtin_amdgcn_s_waitcnt(kWaitStores);
   __syncthreads();
   if (threadIdx.x == 0) {
     const int old = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

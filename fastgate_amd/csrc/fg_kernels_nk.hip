@@ -211,7 +211,10 @@ __global__ __launch_bounds__(256) void nk_mfma4_kernel(const half_t* __restrict_
 // and 16 activation rows per step: 24.5 us against 22.7 us without the activation rows, at
 // K = N = 8192).  So here a wave loads, per step, a BAND-byte band (BAND/2 k) of the tile's weight
 // rows and of the A rows -- 64 lanes x 16 B cover 1024/BAND rows per instruction -- parks both in
-// wave-private LDS strips (rows padded by 16 B: conflict-free in both directions) and reads them
+// wave-private LDS strips (rows padded by 16 B, which spreads both the row-order stores and the
+// operand-order loads over all banks; SQ_LDS_BANK_CONFLICT still counts about 400 cycles per wave
+// at K = N = 8192, M = 16 -- 819 200 per dispatch, under 1 % of a wave's run time -- so the padding
+// is not exact, and not worth more LDS) and reads them
 // back in operand order for BAND/64 MFMAs per 16-column block.  The tile is only 16 (or, with
 // CB = 2, 32) columns wide, so N/16 workgroups fill the chip without split-K and there is no second
 // pass; the waves of a workgroup interleave over the bands of K and meet in LDS once at the end.

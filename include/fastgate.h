@@ -130,7 +130,7 @@ int fg_gemm_f16(const void* A, const void* W, void* C, int M, int N, int K, int 
  * 16-way split of 16 x 16384 outputs) is rejected with FG_ERR_SCRATCH_LIMIT; plans that do not
  * split have no limit.  `splitk` as in fg_gemm_f16.  Results are those of fg_gemm_f16, bit for bit.  All calls on one GPU share that GPU's array: calls that overlap in time on one
  * GPU (two streams, two threads) race, so order them on one stream.  The first call on a device
- * looks the array's address up and clears its counter header; make that call outside graph
+ * looks the array's address up and clears its workspace header; make that call outside graph
  * capture, with the device of `stream` current.
  */
 #define FG_STATIC_SCRATCH_BYTES (65536 + 3145728 + (8 << 20))
@@ -183,8 +183,8 @@ int fg_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* out);
  * does not split across workgroups).  Host only. */
 size_t fg_workspace_bytes(int M, int N, int K, int w_layout, int splitk);
 
-/* Size of the counter header at the start of a split-K workspace, and the call that zeroes it
- * (a fill kernel on `stream`, safe to capture in a HIP graph).  Needed once per workspace, not
+/* Size of the header (arrival counters, then accumulator and class words) at the start of a
+ * split-K workspace, and the call that zeroes it (a fill kernel on `stream`, safe to capture in a HIP graph).  Needed once per workspace, not
  * per call.  The reference has no counterpart: its split-K adds fp16 atomically into a C the
  * host zeroed with an extra memset launch (backend/cuda/hk/edgemm.cu:138-142). */
 size_t fg_workspace_header_bytes(void);

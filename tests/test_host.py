@@ -2,6 +2,7 @@
 header declares, the launch planner is self-consistent, the pybind11 surface carries every
 reference name with the reference's error behaviour, and the product never reaches the oracle."""
 import ctypes
+import os
 import re
 import subprocess
 from pathlib import Path
@@ -362,3 +363,22 @@ def test_bz_does_not_change_the_launch(sg):
         sg.plan_for("flat_gemm_m8n256k64x8", 8, 8192, 8200, 1)
     with pytest.raises(ValueError):
         sg.plan_for("no_such_operator", 8, 8192, 8192, 1)
+
+
+def test_completion_protocol_can_be_forced_from_the_environment():
+    """FASTGATE_SPLITK_COMPLETION is read once per process, so each value gets its own."""
+    import sys
+    code = ("from fastgate_amd import capi\n"
+            "print(capi.plan(1, 8192, 8192, 0).fused, capi.plan(8, 8192, 8192, 0).fused,"
+            " capi.plan(64, 8192, 8192, 0).fused, capi.plan(8, 8192, 8192, 0).splitk)")
+    seen = {}
+    for value in ("", "two-pass", "counter", "atomic", "nonsense"):
+        env = dict(os.environ, FASTGATE_SPLITK_COMPLETION=value)
+        if not value:
+            env.pop("FASTGATE_SPLITK_COMPLETION")
+        out = subprocess.run([sys.executable, "-c", code], env=env, cwd=ROOT, capture_output=True, text=True,
+                             check=True).stdout.split()
+        seen[value] = [int(x) for x in out]
+    assert seen[""] == seen["nonsense"]
+    assert seen["two-pass"][:2] == [0, 0] and seen["counter"][:2] == [1, 1] and seen["atomic"][:2] == [2, 2]
+    assert len({v[3] for v in seen.values()}) == 1       # the split itself is the planner's
