@@ -314,6 +314,104 @@ def run_sweep(torch, sg, capi, dev, steps, warmup, models=False):
             "device": torch.cuda.get_device_name(0)}
 
 
+def run_plan_grid(torch, capi, dev, steps, warmup):
+    """The library's plan for each call of the step against explicit alternatives (kernel family x
+    split-K x waves x unroll x completion), every one checked against torch.matmul before it is
+    timed.  Weights rotate over more than 512 MiB as in the step."""
+    import ctypes
+    import itertools
+    L = capi.lib()
+    KN, NK = capi.FG_W_KN, capi.FG_W_NK
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    vp = lambda t: ctypes.c_void_p(t.data_ptr())
+
+    def time_us(fn):
+        for i in range(warmup):
+            fn(i)
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(steps):
+            fn(i)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / steps
+
+    def candidates(layout, M):
+        out = []
+        if layout == KN:
+            fams = [(capi.FG_KERNEL_KN_MFMA, 16, 0, 0)]
+            if M <= 8:
+                fams.append((capi.FG_KERNEL_KN_DOT2, M, 0, 0))
+            for (kern, mb, tn, band), S, w, U in itertools.product(fams, (2, 4, 8, 16), (4, 8), (1, 2)):
+                for fused in (1, 2):
+                    out.append(dict(kernel=kern, m_block=mb, tile_n=tn, band=band, splitk=S, waves=w, unroll=U,
+                                    fused=fused))
+        else:
+            for tn, band, w, S in itertools.product((16, 32), (128, 256), (4, 8), (1, 2)):
+                out.append(dict(kernel=capi.FG_KERNEL_NK_MFMA_R, m_block=16, tile_n=tn, band=band, splitk=S, waves=w,
+                                unroll=1, fused=2))
+            if M <= 8:
+                for tn, U, w, S in itertools.product((4, 8), (1, 2, 4), (4, 8), (1, 2)):
+                    out.append(dict(kernel=capi.FG_KERNEL_NK_DOT2, m_block=M, tile_n=tn, band=0, splitk=S, waves=w,
+                                    unroll=U, fused=2))
+            if M >= 4:
+                for tn, U, w, S in itertools.product((8, 16), (1, 2), (4, 8), (1, 2)):
+                    out.append(dict(kernel=capi.FG_KERNEL_NK_MFMA4, m_block=(M + 3) // 4 * 4, tile_n=tn, band=0,
+                                    splitk=S, waves=w, unroll=U, fused=2))
+        return out
+
+    g = torch.Generator(device=dev).manual_seed(2040)
+    nbuf = 5
+    weights = [(torch.randn((K, N), device=dev, generator=g) * 0.02).half() for _ in range(nbuf)]
+    ws = torch.zeros(L.fg_workspace_header_bytes() + (64 << 20), dtype=torch.uint8, device=dev)
+    cells = []
+    for layout, M in ((NK, 1), (NK, 8), (NK, 16), (KN, 1), (KN, 8), (KN, 16)):
+        a = torch.randn((M, K), device=dev, generator=g).half()
+        c = torch.empty((M, N), dtype=torch.half, device=dev)
+        w0 = weights[0].float()
+        ref = a.float() @ (w0 if layout == KN else w0.t())
+        lib_plan = capi.plan(M, N, K, layout, 0)
+
+        def timed(plan):
+            def fn(i):
+                st = L.fg_gemm_f16_planned(vp(a), vp(weights[i % nbuf]), vp(c), M, N, K, layout, 0,
+                                           ctypes.byref(plan), vp(ws), ws.numel(), stream)
+                if st != 0:
+                    raise capi.FastgateError(st, "fg_gemm_f16_planned")
+            c.fill_(float("nan"))
+            fn(0)
+            torch.cuda.synchronize()
+            err = float(((c.float() - ref).abs() / (1e-2 + 2e-3 * ref.abs())).max())
+            if not err < 1.0:
+                raise RuntimeError("plan %r gives wrong results (%.2f)" % (plan.as_dict(), err))
+            return min(time_us(fn), time_us(fn))
+
+        rows = []
+        for kw in candidates(layout, M):
+            q = capi.Plan()
+            for k, v in kw.items():
+                setattr(q, k, v)
+            q.stream_w = lib_plan.stream_w
+            try:
+                us = timed(q)
+            except capi.FastgateError:
+                continue          # a combination the kernels do not have
+            rows.append(dict(kw, kernel=capi.KERNEL_NAMES[kw["kernel"]], us=round(us, 2)))
+        rows.sort(key=lambda r: r["us"])
+        us_lib = timed(lib_plan)
+        d = lib_plan.as_dict()
+        cells.append({"M": M, "N": N, "K": K, "w_layout": "[N,K]" if layout == NK else "[K,N]",
+                      "library": {k: d[k] for k in ("kernel_name", "tile_n", "m_block", "band", "splitk", "waves",
+                                                    "unroll", "fused")},
+                      "library_us": round(us_lib, 2), "alternatives_timed": len(rows), "fastest": rows[:6],
+                      "by_split": {str(S): min((r["us"] for r in rows if r["splitk"] == S), default=None)
+                                   for S in (1, 2, 4, 8, 16)}})
+    return {"plan_grid": cells, "steps": steps, "warmup": warmup, "data": "synthetic", "dtype": "f16",
+            "device": torch.cuda.get_device_name(0)}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -328,6 +426,8 @@ def main() -> int:
                          "layouts) and print one JSON object with the plan and roofline figures per shape")
     ap.add_argument("--sweep-models", action="store_true",
                     help="as --sweep, over the projection shapes of common decoder layers (both layouts, M = 1, 8, 16)")
+    ap.add_argument("--plan-grid", action="store_true",
+                    help="time the library's plan for each call of the step against explicit alternative plans")
     ap.add_argument("--cpu-repeats", type=int, default=8, help="repetitions of the step on the CPU oracle (0 = skip)")
     ap.add_argument("--ingest-pmc", metavar="DIR", default=None,
                     help="host only: rewrite bench_traffic.json from DIR/{pmc,cal}_{FETCH,WRITE}_SIZE, the CSV output of "
@@ -372,6 +472,10 @@ def main() -> int:
         print(json.dumps({"calibration": {"stream_read_kernel": {"read_bytes": 1 << 30, "write_bytes": 0, "launches": 5},
                                           "device_copy_kernel": {"read_bytes": 256 << 20, "write_bytes": 256 << 20,
                                                                  "launches": 5}}}))
+        return 0
+
+    if args.plan_grid:
+        print(json.dumps(run_plan_grid(torch, capi, dev, args.steps, args.warmup)))
         return 0
 
     if args.sweep or args.sweep_models:
