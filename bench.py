@@ -157,7 +157,28 @@ def run_sweep(torch, sg, capi, dev, steps, warmup, models=False):
     us = time_us(lambda i: L.fg_stream_read(ctypes.c_void_p(probe[i % 2].data_ptr()), 1 << 30,
                                             ctypes.c_void_p(sink.data_ptr()), stream))
     ceiling = (1 << 30) / us / 1e3
-    del probe
+    del probe[1]
+
+    # what the same read-only kernel takes for as many bytes as a call moves (whole MiB, rotating over
+    # the 1 GiB buffer): launch, ramp-up and tail weigh more the smaller the call
+    same_size = {}
+
+    def same_size_read_us(nbytes):
+        mib = max(1, min(1024, -(-nbytes // (1 << 20))))
+        if mib not in same_size:
+            n = mib << 20
+            nb = (1 << 30) // n
+            base = probe[0].data_ptr()
+            fn = lambda i: L.fg_stream_read(ctypes.c_void_p(base + (i % nb) * n), n,
+                                            ctypes.c_void_p(sink.data_ptr()), stream)
+            same_size[mib] = min(time_us(fn), time_us(fn))
+        return same_size[mib]
+
+    def with_same_size(row):
+        t = same_size_read_us(row["bytes"])
+        row["same_size_read_us"] = round(t, 2)
+        row["frac_same_size_read"] = round(t / row["us_per_call"], 4)
+        return row
 
     rows = []
 
@@ -181,14 +202,14 @@ def run_sweep(torch, sg, capi, dev, steps, warmup, models=False):
         us_vendor = time_us(lambda i: vend(a, ws[i % nbuf], c2))
         by = 2 * Kk * Nn + 2 * M * Kk + 2 * M * Nn
         p = capi.plan(M, Nn, Kk, layout, 0).as_dict()
-        rows.append({"config": name, "op": op, "M": M, "K": Kk, "N": Nn,
+        rows.append(with_same_size({"config": name, "op": op, "M": M, "K": Kk, "N": Nn,
                      "w_layout": "[N,K]" if layout == capi.FG_W_NK else "[K,N]", "seed": seed,
                      "kernel": p["kernel_name"], "splitk": p["splitk"], "in_launch_reduce": p["fused"],
                      "tile_n": p["tile_n"], "bytes": by, "us_per_call": round(us_call, 2),
                      "GBps": round(by / us_call / 1e3, 1), "TFLOPs": round(2.0 * M * Nn * Kk / us_call / 1e6, 2),
                      "frac_hbm_peak": round(by / us_call / 1e3 / HBM_PEAK_GBPS, 4),
                      "frac_read_ceiling": round(by / us_call / 1e3 / ceiling, 4),
-                     "vendor_us_per_call": round(us_vendor, 2)})
+                     "vendor_us_per_call": round(us_vendor, 2)}))
 
     if models:
         for li, (label, Nn, Kk) in enumerate(MODEL_SHAPES):
@@ -221,13 +242,13 @@ def run_sweep(torch, sg, capi, dev, steps, warmup, models=False):
     by = Kk * Nn + 2 * Kk + 2 * Nn + 2 * Nn
     us_f16 = next(r["us_per_call"] for r in rows if r["config"] == "C5 sweep" and r["M"] == 1 and r["K"] == 8192
                   and r["w_layout"] == "[N,K]")
-    rows.append({"config": "C4 int8 fastgemv", "op": "fastgemv_int8", "M": 1, "K": Kk, "N": Nn, "w_layout": "[N,K] int8",
+    rows.append(with_same_size({"config": "C4 int8 fastgemv", "op": "fastgemv_int8", "M": 1, "K": Kk, "N": Nn, "w_layout": "[N,K] int8",
                  "seed": 1004, "kernel": "w8a16", "splitk": 1, "bytes": by, "us_per_call": round(us_i8, 2),
                  "GBps": round(by / us_i8 / 1e3, 1), "frac_hbm_peak": round(by / us_i8 / 1e3 / HBM_PEAK_GBPS, 4),
                  "frac_read_ceiling": round(by / us_i8 / 1e3 / ceiling, 4),
                  "weights_per_ns": round(Kk * Nn / us_i8 / 1e3, 3),
                  "fp16_M1_weights_per_ns": round(Kk * Nn / us_f16 / 1e3, 3),
-                 "weight_throughput_vs_fp16": round(us_f16 / us_i8, 3)})
+                 "weight_throughput_vs_fp16": round(us_f16 / us_i8, 3)}))
     # beyond the benchmark's configurations: the int8 GEMV with 4, 8 and 16 activation rows
     for Mb in (4, 8, 16):
         xb = torch.randn((Mb, Kk), device=dev, generator=g).half()
@@ -236,27 +257,27 @@ def run_sweep(torch, sg, capi, dev, steps, warmup, models=False):
         us_fb = next(r["us_per_call"] for r in rows if r["config"] == "C5 sweep" and r["M"] == Mb
                      and r["K"] == 8192 and r["w_layout"] == "[N,K]")
         by = Kk * Nn + 2 * Mb * Kk + 2 * Mb * Nn + 2 * Nn
-        rows.append({"config": "extra: int8 batched", "op": "fastgemv_int8", "M": Mb, "K": Kk, "N": Nn,
+        rows.append(with_same_size({"config": "extra: int8 batched", "op": "fastgemv_int8", "M": Mb, "K": Kk, "N": Nn,
                      "w_layout": "[N,K] int8", "seed": 1004, "kernel": "w8a16_r", "splitk": 1, "bytes": by,
                      "us_per_call": round(us_b, 2), "GBps": round(by / us_b / 1e3, 1),
                      "frac_hbm_peak": round(by / us_b / 1e3 / HBM_PEAK_GBPS, 4),
                      "frac_read_ceiling": round(by / us_b / 1e3 / ceiling, 4),
                      "weights_per_ns": round(Kk * Nn / us_b / 1e3, 3),
                      "fp16_M1_weights_per_ns": round(Kk * Nn / us_fb / 1e3, 3),
-                     "weight_throughput_vs_fp16": round(us_fb / us_b, 3)})
+                     "weight_throughput_vs_fp16": round(us_fb / us_b, 3)}))
     # beyond the benchmark's configurations: the same GEMV with 4-bit weights (two per byte)
     del wq
     wq4 = [torch.randint(0, 256, (Nn, Kk // 2), device=dev, generator=g, dtype=torch.uint8) for _ in range(20)]
     us_i4 = time_us(lambda i: sg.fastgemv_int4(wq4[i % 20], x, y, scale=scale, zero_point=8.0))
     by = Kk * Nn // 2 + 2 * Kk + 2 * Nn + 2 * Nn
-    rows.append({"config": "extra: int4 fastgemv", "op": "fastgemv_int4", "M": 1, "K": Kk, "N": Nn,
+    rows.append(with_same_size({"config": "extra: int4 fastgemv", "op": "fastgemv_int4", "M": 1, "K": Kk, "N": Nn,
                  "w_layout": "[N,K/2] uint4x2", "seed": 1004, "kernel": "w4a16", "splitk": 1, "bytes": by,
                  "us_per_call": round(us_i4, 2), "GBps": round(by / us_i4 / 1e3, 1),
                  "frac_hbm_peak": round(by / us_i4 / 1e3 / HBM_PEAK_GBPS, 4),
                  "frac_read_ceiling": round(by / us_i4 / 1e3 / ceiling, 4),
                  "weights_per_ns": round(Kk * Nn / us_i4 / 1e3, 3),
                  "fp16_M1_weights_per_ns": round(Kk * Nn / us_f16 / 1e3, 3),
-                 "weight_throughput_vs_fp16": round(us_f16 / us_i4, 3)})
+                 "weight_throughput_vs_fp16": round(us_f16 / us_i4, 3)}))
     # beyond the benchmark's configurations: [K,N] weights of the metric shape padded to a row pitch
     # of N + 128 elements (a view of a [K, N+128] buffer), as a caller that owns the weights can lay
     # them out once at load time
@@ -272,13 +293,13 @@ def run_sweep(torch, sg, capi, dev, steps, warmup, models=False):
                     and r["K"] == Kp and r["w_layout"] == "[K,N]")
         by = 2 * Kp * Np + 2 * Mp * Kp + 2 * Mp * Np
         pl = capi.plan(Mp, Np, Kp, capi.FG_W_KN, 0).as_dict()
-        rows.append({"config": "extra: [K,N] row pitch N+128", "op": "edgemm_m8n128k64x4", "M": Mp, "K": Kp,
+        rows.append(with_same_size({"config": "extra: [K,N] row pitch N+128", "op": "edgemm_m8n128k64x4", "M": Mp, "K": Kp,
                      "N": Np, "w_layout": "[K,N] pitch 8320", "seed": 2040, "kernel": pl["kernel_name"],
                      "splitk": pl["splitk"], "in_launch_reduce": pl["fused"], "tile_n": pl["tile_n"],
                      "bytes": by, "us_per_call": round(us_p, 2), "GBps": round(by / us_p / 1e3, 1),
                      "frac_hbm_peak": round(by / us_p / 1e3 / HBM_PEAK_GBPS, 4),
                      "frac_read_ceiling": round(by / us_p / 1e3 / ceiling, 4),
-                     "us_per_call_dense": us_d})
+                     "us_per_call_dense": us_d}))
     del padded, views
     # beyond the benchmark's configurations: the feed-forward pair of C3 (16 x 3072 x 12288, then
     # 16 x 12288 x 3072) with bias and GELU, fused into the two GEMM launches against the same two
@@ -303,12 +324,12 @@ def run_sweep(torch, sg, capi, dev, steps, warmup, models=False):
 
     us_unfused = time_us(unfused)
     by = 2 * (2 * Kf * Nf) + 2 * Mf * Kf * 2 + 2 * Mf * Nf * 2 + 2 * Nf + 2 * Kf
-    rows.append({"config": "extra: FFN pair, bias + GELU fused", "op": "ffn_bt", "M": Mf, "K": Kf, "N": Nf,
+    rows.append(with_same_size({"config": "extra: FFN pair, bias + GELU fused", "op": "ffn_bt", "M": Mf, "K": Kf, "N": Nf,
                  "w_layout": "[N,K] twice", "seed": 1003, "kernel": "nk_mfma_r x2", "splitk": "-", "bytes": by,
                  "us_per_call": round(us_fused, 2), "GBps": round(by / us_fused / 1e3, 1),
                  "frac_hbm_peak": round(by / us_fused / 1e3 / HBM_PEAK_GBPS, 4),
                  "frac_read_ceiling": round(by / us_fused / 1e3 / ceiling, 4),
-                 "us_unfused_with_torch_elementwise": round(us_unfused, 2)})
+                 "us_unfused_with_torch_elementwise": round(us_unfused, 2)}))
     return {"sweep": rows, "read_ceiling_GBps": round(ceiling, 1), "hbm_peak_GBps": HBM_PEAK_GBPS,
             "steps": steps, "warmup": warmup, "data": "synthetic", "dtype": "f16",
             "device": torch.cuda.get_device_name(0)}
@@ -534,6 +555,23 @@ def main() -> int:
     e1.record()
     barrier()
     copy_gbps = 2 * (1 << 30) * 5 / (e0.elapsed_time(e1) * 1e-3) / 1e9
+
+    # the same read-only kernel on as many bytes as one call moves (128 MiB, and 64 MiB for the int8
+    # GEMV), rotating over the 1 GiB buffer: what launch, ramp-up and tail leave of the ceiling
+    def read_us(n):
+        nb = (1 << 30) // n
+        fn = lambda i: L.fg_stream_read(ctypes.c_void_p(probe[0].data_ptr() + (i % nb) * n), n,
+                                        ctypes.c_void_p(sink.data_ptr()), stream)
+        for i in range(10):
+            fn(i)
+        barrier()
+        e0.record()
+        for i in range(100):
+            fn(i)
+        e1.record()
+        barrier()
+        return e0.elapsed_time(e1) * 1e3 / 100
+    read_us_128, read_us_64 = read_us(128 << 20), read_us(64 << 20)
     del probe
 
     # ---- warm-up, then exactly `steps` timed steps ------------------------------------------------
@@ -591,7 +629,8 @@ def main() -> int:
             "us_per_call_single_buffer": round(us_hot, 2),
             "TFLOPs": round(2.0 * M * N * K / (us * 1e-6) / 1e12, 2),
             "frac_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4),
-            "frac_read_ceiling": round(gbps / ceiling_gbps, 4)})
+            "frac_read_ceiling": round(gbps / ceiling_gbps, 4),
+            "frac_same_size_read": round(read_us_128 * algorithmic_bytes(M) / (128 << 20) / us, 4)})
 
     # ---- int8 GEMV (fastgemv_int8, K = N = 8192, per-channel scale) against the fp16 GEMV of the
     # same shape: the two alternate, `steps` back-to-back launches each, five rounds; the ratio of
@@ -621,6 +660,7 @@ def main() -> int:
     int8 = {"op": "fastgemv_int8", "M": 1, "K": K, "N": N, "kernel": "w8a16_m1", "bytes": i8_bytes,
             "us_per_call": round(us_i8, 2), "GBps": round(i8_bytes / us_i8 / 1e3, 1),
             "frac_read_ceiling": round(i8_bytes / us_i8 / 1e3 / ceiling_gbps, 4),
+            "frac_same_size_read": round(read_us_64 * i8_bytes / (64 << 20) / us_i8, 4),
             "fp16_fastgemv_us_per_call": round(us_f16, 2),
             "weight_throughput_vs_fp16": round(us_f16 / us_i8, 3), "target": 1.8}
     del wq
@@ -637,6 +677,8 @@ def main() -> int:
         "launches_in_call": dom["launches"], "us": dom["us_per_call"],
         "algorithmic_bytes": dom["bytes"], "measured_read_ceiling_GBps": round(ceiling_gbps, 1),
         "frac_of_read_ceiling": dom["frac_read_ceiling"],
+        "same_size_read_us": {"128MiB": round(read_us_128, 2), "64MiB": round(read_us_64, 2)},
+        "frac_of_same_size_read": dom["frac_same_size_read"],
     }
 
     # ---- CPU baseline: the oracle on the same step -------------------------------------------------
