@@ -18,6 +18,7 @@
 #include <torch/extension.h>
 
 #include <map>
+#include <vector>
 #include <mutex>
 #include <stdexcept>
 #include <string>
@@ -72,6 +73,9 @@ Workspace workspace(int device, void* stream, const at::Tensor& like, size_t byt
   auto it = cache.find(key);
   if (it == cache.end() || (size_t)it->second.numel() < bytes) {
     const size_t want = std::max<size_t>(bytes, (size_t)16 << 20);
+    // a buffer that is outgrown stays allocated: another thread may still remember its address
+    static std::vector<at::Tensor> outgrown;
+    if (it != cache.end()) outgrown.push_back(it->second);
     cache[key] = at::zeros({(int64_t)want}, like.options().dtype(at::kByte));
     it = cache.find(key);
   }
