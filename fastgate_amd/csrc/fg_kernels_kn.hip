@@ -127,44 +127,36 @@ __global__ __launch_bounds__(64 * NW) void kn_mfma_kernel(const half_t* __restri
     }
     return;
   }
-  // 16 x 128 outputs, 8 consecutive columns per thread.
-  for (int e = threadIdx.x; e < 256; e += blockDim.x) {
-    const int m = e >> 4, c0 = (e & 15) * 8;
+  // 16 x 128 outputs in groups of four columns: the 32 lanes of a half wave cover one 512-byte row
+  // with consecutive 16-byte pieces, so every store instruction writes whole rows (partials that go
+  // out as 16 bytes at a 32-byte stride, two instructions to fill a row, take the write-through
+  // path twice as long).
+  for (int e = threadIdx.x; e < 512; e += blockDim.x) {
+    const int m = e >> 5, c0 = (e & 31) * 4;
     const int mg = m0 + m;
     if (mg < M) {
       // the reads of all waves in flight before the first add
-      float4_t lo[NW], hi[NW];
+      float4_t v[NW];
 #pragma unroll
-      for (int w = 0; w < NW; ++w) {
-        const float4_t* src = reinterpret_cast<const float4_t*>(&red[w < nw ? w : 0][m][c0]);
-        lo[w] = src[0];
-        hi[w] = src[1];
-      }
-      float sum[8];
+      for (int w = 0; w < NW; ++w) v[w] = *reinterpret_cast<const float4_t*>(&red[w < nw ? w : 0][m][c0]);
+      float4_t sum = {0.f, 0.f, 0.f, 0.f};
+      const float4_t zero4 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int i = 0; i < 8; ++i) sum[i] = 0.f;
-#pragma unroll
-      for (int w = 0; w < NW; ++w)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          sum[i] += w < nw ? lo[w][i] : 0.f;
-          sum[4 + i] += w < nw ? hi[w][i] : 0.f;
-        }
+      for (int w = 0; w < NW; ++w) sum += w < nw ? v[w] : zero4;
       if (gridDim.z == 1) {
-        half_t* c = C + (size_t)mg * N + n0 + c0;
-        half8_t out;
+        typedef half_t half4v __attribute__((ext_vector_type(4)));
+        half4v* c = reinterpret_cast<half4v*>(C + (size_t)mg * N + n0 + c0);
         if (flags & kFlagAccumulate) {
-          const half8_t old = *reinterpret_cast<const half8_t*>(c);
+          const half4v old = *c;
 #pragma unroll
-          for (int i = 0; i < 8; ++i) sum[i] += static_cast<float>(old[i]);
+          for (int i = 0; i < 4; ++i) sum[i] += static_cast<float>(old[i]);
         }
+        half4v out;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) out[i] = static_cast<half_t>(apply_tail(sum[i], n0 + c0 + i, bias, flags));
-        *reinterpret_cast<half8_t*>(c) = out;
+        for (int i = 0; i < 4; ++i) out[i] = static_cast<half_t>(apply_tail(sum[i], n0 + c0 + i, bias, flags));
+        *c = out;
       } else {
-        const size_t o = ((size_t)blockIdx.z * M + mg) * N + n0 + c0;
-        store_partial4(ws, o, float4_t{sum[0], sum[1], sum[2], sum[3]}, counters != nullptr);
-        store_partial4(ws, o + 4, float4_t{sum[4], sum[5], sum[6], sum[7]}, counters != nullptr);
+        store_partial4(ws, ((size_t)blockIdx.z * M + mg) * N + n0 + c0, sum, counters != nullptr);
       }
     }
   }

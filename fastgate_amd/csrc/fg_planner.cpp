@@ -569,16 +569,20 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
   // In-launch completion through one fixed-point atomic per output element (fused = 2) instead of
   // partials + arrival counter (fused = 1): one memory round trip after the K loop instead of
   // three, but S * M * N atomics.  Measured over 11 N x 7 K x 6 M on both layouts (us gained over
-  // the counter protocol, 514 splits): every v_dot2 split 0.5 .. 2.5, every [N,K] split 0.3 .. 1.9;
-  // the [K,N] MFMA kernel with eight waves 0.1 .. 1.8 below 5 * 2^16 atomics or from eight splits
-  // on (0.1 .. 1.4 lost otherwise), with four waves 0.4 on average below 2^16 atomics, level for
-  // deep splits and 0.4 .. 1.4 lost otherwise (K = 8192 N = 12288 M = 16, five splits).
+  // the counter protocol): every v_dot2 split 0.5 .. 2.5, every [N,K] split 0.3 .. 1.9.  For the
+  // [K,N] MFMA kernel, whose counter protocol writes its partials as whole 512-byte rows, 385
+  // splits (M = 3 .. 16) put the break-even at: eight waves, 16 splits or more 0.3 .. 2.4 gained
+  // up to 2^20 atomics; 8 .. 15 splits 0.2 .. 1.4 gained up to 6 * 2^16 atomics, level to 0.9 lost
+  // above; fewer splits 0.2 gained on average below 3 * 2^16, 0.1 .. 1.9 lost above.  Four waves:
+  // gained only from 16 splits on, or from 8 below 3 * 2^16; 0.2 .. 2.0 lost otherwise.
   if (p->splitk > 1 && p->fused == 1 && p->splitk <= kFixMaxSplit && (size_t)M * N <= kWsAccElems) {
     const size_t atomics = (size_t)p->splitk * M * N;
     bool atomic = true;
     if (p->kernel == FG_KERNEL_KN_MFMA) {
-      atomic = p->waves >= 8 ? (atomics < ((size_t)5 << 16) || p->splitk >= 8)
-                             : (atomics < ((size_t)1 << 16) || (p->splitk >= 8 && atomics < ((size_t)1 << 19)));
+      const size_t unit = (size_t)1 << 16;
+      if (p->splitk >= 16) atomic = atomics < 16 * unit;
+      else if (p->splitk >= 8) atomic = atomics <= (p->waves >= 8 ? 6 : 3) * unit;
+      else atomic = p->waves >= 8 && atomics < 3 * unit;
     }
     if (atomic) p->fused = 2;
   }

@@ -136,6 +136,9 @@ def test_plan_choices_that_were_measured():
     # completion of the split: atomics for v_dot2, for [N,K] and for few elements; the counter otherwise
     assert kn(1, 8192, 8192).fused == 2 and kn(8, 4096, 4096).fused == 2 and nk(16, 2048, 8192).fused == 2
     assert kn(8, 8192, 8192).fused == 1 and kn(16, 8192, 8192).fused == 1 and kn(16, 12288, 8192).fused == 1
+    # the [K,N] MFMA kernel: atomics only for deep splits or few elements (four waves: from 8 splits on)
+    assert kn(4, 8192, 8192).fused == 1 and kn(16, 4096, 4096).fused == 1 and kn(16, 4096, 11008).fused == 1
+    assert kn(8, 11008, 4096).fused == 2 and kn(16, 2048, 16384).fused == 2
     assert kn(24, 2048, 4096).fused == 0           # more than 16 rows: second kernel
     p = kn(16, 5120, 8192)
     assert (p.splitk, p.waves) == (6, 8)
