@@ -302,3 +302,35 @@ def test_two_streams_with_split_k_calls_in_flight_do_not_interfere(device, sg):
         assert_close_f16(first, ref[i], "stream %d" % i)
         for it in range(1, 30):
             assert (outs[i][it].cpu().numpy().view(np.uint16) == first.view(np.uint16)).all(), (i, it)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("completion", ["two-pass", "counter", "atomic"])
+def test_completion_switch_end_to_end(completion):
+    """FASTGATE_SPLITK_COMPLETION is read once per process: a child process with the variable set
+    runs split [K,N] and [N,K] products through the binding and compares them with torch.matmul."""
+    import os
+    import subprocess
+    import sys
+    from pathlib import Path
+    code = r'''
+import torch
+from fastgate_amd import capi, speedgate as sg
+want = {"two-pass": 0, "counter": 1, "atomic": 2}[%r]
+torch.manual_seed(3)
+for (M, N, K, op, layout) in ((8, 4096, 4096, "edgemm_m8n128k64x4", 0), (1, 2048, 8192, "edgemm_m8n128k64x4", 0),
+                              (16, 2048, 8192, "edgemm_m8n128k64x4_bt", 1)):
+    p = capi.plan(M, N, K, layout)
+    assert p.splitk > 1 and p.fused == want, (M, N, K, p.as_dict())
+    A = torch.randn(M, K, device="cuda").half()
+    W = (torch.randn((K, N) if layout == 0 else (N, K), device="cuda") * 0.05).half()
+    C = torch.empty(M, N, dtype=torch.half, device="cuda")
+    getattr(sg, op)(A, W, C)
+    ref = A.float() @ (W.float() if layout == 0 else W.float().t())
+    assert bool(((C.float() - ref).abs() <= 1e-2 + 2e-3 * ref.abs()).all()), (M, N, K)
+print("ok")
+''' % completion
+    root = Path(__file__).resolve().parent.parent
+    env = dict(os.environ, FASTGATE_SPLITK_COMPLETION=completion)
+    out = subprocess.run([sys.executable, "-c", code], env=env, cwd=root, capture_output=True, text=True, timeout=110)
+    assert out.returncode == 0 and out.stdout.strip().endswith("ok"), out.stdout + out.stderr
