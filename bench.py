@@ -16,8 +16,10 @@ value = algorithmic bytes of a step / time of a step (GB/s).  Algorithmic bytes 
 2*K*N (weights) + 2*M*K (activations) + 2*M*N (result); split-K partials are not counted.
 
 Prints ONE JSON line.  `roofline` describes the kernel that takes the most time in the step,
-timed with HIP events inside the timed region; `cpu_baseline` is the CPU oracle
-(oracle/fg_oracle.c, one thread) on the same step, timed on this host.
+timed with HIP events on the launch stream; `cpu_baseline` is the reference's CPU path
+(torch.matmul with fp32 accumulation on all host cores) on the same step, timed on this host, with
+the single-thread C restatement (oracle/fg_oracle.c) nested beside it and labelled as ours;
+`configs` carries the benchmark's other configurations (C1-C4) timed the same way.
 """
 from __future__ import annotations
 
@@ -596,30 +598,33 @@ def main() -> int:
     ms_per_step = wall_ms / args.steps
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
 
-    # ---- per-call kernel time: `steps` back-to-back launches of one call between two HIP events
-    # on the launch stream (an event between every two calls of the step above would add about
-    # 3.5 us of bubble per call and distort `value`) --------------------------------------------------
+    # ---- per-call kernel time, outside the timed steps: back-to-back launches of one call between
+    # two HIP events on the launch stream (an event between every two calls of the step above would
+    # add about 3.5 us of bubble per call and distort `value`).  The launch count does not follow
+    # --steps: the gap between the first event and the first kernel (about 10 us) is spread over
+    # at least 200 launches after 20 untimed ones, whatever the step count is. -----------------------
+    launches = max(args.steps, 200)
+
+    def timed_launches(fn, first=0):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        for s_ in range(20):
+            fn(first + s_)
+        barrier()
+        e0.record()
+        for s_ in range(launches):
+            fn(first + 20 + s_)
+        e1.record()
+        barrier()
+        return e0.elapsed_time(e1) * 1e3 / launches
+
     per_call = []
     for c, (label, M, layout, fn) in enumerate(calls):
         p = capi.plan(M, N, K, layout).as_dict()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        barrier()
-        e0.record()
-        for s in range(args.steps):
-            fn(it + s)
-        e1.record()
-        barrier()
-        it += args.steps
-        us = e0.elapsed_time(e1) * 1e3 / args.steps
+        us = timed_launches(fn, it)
+        it += launches + 20
         gbps = algorithmic_bytes(M) / (us * 1e-6) / 1e9
         # the same call on one weight buffer: 128 MiB stays in the 256 MB Infinity Cache
-        barrier()
-        e0.record()
-        for s in range(args.steps):
-            fn(0)
-        e1.record()
-        barrier()
-        us_hot = e0.elapsed_time(e1) * 1e3 / args.steps
+        us_hot = timed_launches(lambda i: fn(0))
         per_call.append({
             "op": label, "M": M, "w_layout": "[N,K]" if layout == capi.FG_W_NK else "[K,N]",
             "kernel": p["kernel_name"], "splitk": p["splitk"], "tile_n": p["tile_n"], "waves": p["waves"],
@@ -633,7 +638,7 @@ def main() -> int:
             "frac_same_size_read": round(read_us_128 * algorithmic_bytes(M) / (128 << 20) / us, 4)})
 
     # ---- int8 GEMV (fastgemv_int8, K = N = 8192, per-channel scale) against the fp16 GEMV of the
-    # same shape: the two alternate, `steps` back-to-back launches each, five rounds; the ratio of
+    # same shape: the two alternate, `launches` back-to-back launches each, five rounds; the ratio of
     # the medians is the int8 path's weight throughput relative to fp16 (target 1.8) ---------------
     gi = torch.Generator(device=dev).manual_seed(1004)
     wq = [torch.randint(-127, 128, (N, K), device=dev, generator=gi, dtype=torch.int8) for _ in range(2 * R)]
@@ -641,20 +646,10 @@ def main() -> int:
     sc = (torch.rand(N, device=dev, generator=gi) * 0.009 + 0.001).half()
     yi = torch.empty(N, dtype=torch.half, device=dev)
 
-    def timed(fn):
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        barrier()
-        e0.record()
-        for s_ in range(args.steps):
-            fn(s_)
-        e1.record()
-        barrier()
-        return e0.elapsed_time(e1) * 1e3 / args.steps
-
     t_i8, t_f16 = [], []
     for _ in range(5):
-        t_f16.append(timed(lambda i: sg.fastgemv(w_nk[i % R], acts_d[1], y1)))
-        t_i8.append(timed(lambda i: sg.fastgemv_int8(wq[i % (2 * R)], xi, yi, scale=sc)))
+        t_f16.append(timed_launches(lambda i: sg.fastgemv(w_nk[i % R], acts_d[1], y1)))
+        t_i8.append(timed_launches(lambda i: sg.fastgemv_int8(wq[i % (2 * R)], xi, yi, scale=sc)))
     us_i8, us_f16 = sorted(t_i8)[2], sorted(t_f16)[2]
     i8_bytes = K * N + 2 * K + 2 * N + 2 * N
     int8 = {"op": "fastgemv_int8", "M": 1, "K": K, "N": N, "kernel": "w8a16_m1", "bytes": i8_bytes,
@@ -664,6 +659,55 @@ def main() -> int:
             "fp16_fastgemv_us_per_call": round(us_f16, 2),
             "weight_throughput_vs_fp16": round(us_f16 / us_i8, 3), "target": 1.8}
     del wq
+
+    # ---- the benchmark's other configurations (C1 fastgemv 4096^2, C2 edgemm 8 x 4096 x 11008 on both
+    # layouts, C3 the feed-forward pair at 16 rows, C4 the int8 GEMV), timed like the calls above:
+    # rotating over more than 512 MiB of weights, `launches` back-to-back launches after 20 untimed
+    # ones, outside the timed steps --------------------------------------------------------------
+    def read_us_for(nbytes):
+        mib = max(1, -(-nbytes // (1 << 20)))
+        n = mib << 20
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).random_(0, 256)
+        nb = (1 << 30) // n
+        t = timed_launches(lambda i: L.fg_stream_read(ctypes.c_void_p(src.data_ptr() + (i % nb) * n), n,
+                                                      ctypes.c_void_p(sink.data_ptr()), stream))
+        del src
+        return t
+
+    def config_row(name, op, M, Kc, Nc, layout, seed):
+        gc = torch.Generator(device=dev).manual_seed(seed)
+        nbuf = max(2, -(-(640 << 20) // (2 * Kc * Nc)))
+        shape = (Nc, Kc) if layout == capi.FG_W_NK else (Kc, Nc)
+        wsb = [(torch.randn(shape, device=dev, generator=gc) * 0.02).half() for _ in range(nbuf)]
+        a = torch.randn((M, Kc), device=dev, generator=gc).half()
+        c = torch.zeros((M, Nc), dtype=torch.half, device=dev)
+        f = getattr(sg, op)
+        call = (lambda i: f(wsb[i % nbuf], a, c)) if op.startswith("fastgemv") else (lambda i: f(a, wsb[i % nbuf], c))
+        us = min(timed_launches(call), timed_launches(call))
+        del wsb
+        by = 2 * Kc * Nc + 2 * M * Kc + 2 * M * Nc
+        pc = capi.plan(M, Nc, Kc, layout).as_dict()
+        t_read = read_us_for(by)
+        return {"name": name, "op": op, "M": M, "K": Kc, "N": Nc,
+                "w_layout": "[N,K]" if layout == capi.FG_W_NK else "[K,N]", "seed": seed, "bytes": by,
+                "us": round(us, 2), "GBps": round(by / us / 1e3, 1),
+                "frac_hbm_peak": round(by / us / 1e3 / HBM_PEAK_GBPS, 4),
+                "frac_read_ceiling": round(by / us / 1e3 / ceiling_gbps, 4),
+                "same_size_read_us": round(t_read, 2), "frac_same_size_read": round(t_read / us, 4),
+                "plan_key": plan_key(pc, M)}
+
+    configs = [
+        config_row("C1 fastgemv", "fastgemv", 1, 4096, 4096, capi.FG_W_NK, 1001),
+        config_row("C2 edgemm", "edgemm_m8n128k64x4", 8, 4096, 11008, capi.FG_W_KN, 1002),
+        config_row("C2 edgemm_bt", "edgemm_m8n128k64x4_bt", 8, 4096, 11008, capi.FG_W_NK, 1002),
+        config_row("C3a flat up-projection", "gemm_m8n128k64x4_bt", 16, 3072, 12288, capi.FG_W_NK, 1003),
+        config_row("C3b flat down-projection", "gemm_m8n128k64x4_bt", 16, 12288, 3072, capi.FG_W_NK, 1003),
+        {"name": "C4 int8 fastgemv", "op": "fastgemv_int8", "M": 1, "K": K, "N": N, "w_layout": "[N,K] int8",
+         "seed": 1004, "bytes": i8_bytes, "us": int8["us_per_call"], "GBps": int8["GBps"],
+         "frac_hbm_peak": round(int8["GBps"] / HBM_PEAK_GBPS, 4), "frac_read_ceiling": int8["frac_read_ceiling"],
+         "same_size_read_us": round(read_us_64, 2), "frac_same_size_read": int8["frac_same_size_read"],
+         "plan_key": "w8a16_m1|M1"},
+    ]
 
     # The roofline entry describes the single-launch call that takes the longest: its time between
     # the events is one kernel's launch-to-launch time, which the rocprofv3 kernel trace must match.
@@ -710,12 +754,15 @@ def main() -> int:
             tt.append(time.perf_counter() - q0)
         tm = sorted(tt)[len(tt) // 2]
         cpu = {
-            "value": round(step_bytes / cpu_s / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
-            "sample": "the full step (six calls, K=N=8192, M=1/8/16, both weight layouts) on oracle/fg_oracle.c, "
-                      "%d repetitions, %.1f s per step" % (args.cpu_repeats, cpu_s),
-            "torch_matmul_fp32": {"value": round(step_bytes / tm / 1e9, 2), "unit": "GB/s",
-                                  "cores": torch.get_num_threads(), "s_per_step": round(tm, 4),
-                                  "note": "the reference's own check (torch.matmul, fp32 copies made outside the timed region)"},
+            "value": round(step_bytes / tm / 1e9, 2), "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "reference",
+            "sample": "the full step (six calls, K=N=8192, M=1/8/16, both weight layouts) through torch.matmul on fp32 "
+                      "copies made outside the timed region -- the reference's own CPU check "
+                      "(script/standard-test.py:152) -- median of 5 repetitions, %.3f s per step" % tm,
+            "s_per_step": round(tm, 4),
+            "own_port_single_thread": {
+                "value": round(step_bytes / cpu_s / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+                "note": "ours, not the reference's: oracle/fg_oracle.c (fp32 C loop, one thread) on the same step, "
+                        "%d repetitions, %.1f s per step" % (args.cpu_repeats, cpu_s)},
         }
 
     out = {
@@ -734,6 +781,8 @@ def main() -> int:
         "copy_ceiling_GBps": round(copy_gbps, 1),
         "per_call": per_call,
         "int8_gemv": int8,
+        "configs": configs,
+        "launches_per_timing": launches,
     }
     print(json.dumps(out))
     return 0

@@ -46,6 +46,9 @@ EXPORTS = (
     "fg_workspace_bytes",
     "fg_workspace_header_bytes",
     "fg_workspace_init",
+    "fg_set_compute_units",
+    "fg_compute_units",
+    "fg_use_device_compute_units",
     "fg_gemv_w8a16",
     "fg_gemv_w4a16",
     "fg_gemv_i8i8_i32",
@@ -121,6 +124,12 @@ def lib() -> ctypes.CDLL:
         L.fg_workspace_header_bytes.argtypes = []
         L.fg_workspace_init.restype = ci
         L.fg_workspace_init.argtypes = [vp, sz, vp]
+        L.fg_set_compute_units.restype = ci
+        L.fg_set_compute_units.argtypes = [ci]
+        L.fg_compute_units.restype = ci
+        L.fg_compute_units.argtypes = []
+        L.fg_use_device_compute_units.restype = ci
+        L.fg_use_device_compute_units.argtypes = []
         L.fg_gemv_w8a16.restype = ci
         L.fg_gemv_w8a16.argtypes = [vp, vp, vp, cf, cf, vp, ci, ci, ci, vp]
         L.fg_gemv_w4a16.restype = ci

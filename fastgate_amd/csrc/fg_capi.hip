@@ -5,6 +5,7 @@
 #include <algorithm>
 #include <atomic>
 #include <cmath>
+#include <cstdio>
 #include <cstdlib>
 #include <cstring>
 #include <mutex>
@@ -16,21 +17,28 @@
 // is a host-side stand-in for the symbol, never a device address: host code reaches the memory
 // only through the per-device pointer that static_scratch() obtains with hipGetSymbolAddress.
 static __device__ __align__(256) unsigned char scratch[FG_STATIC_SCRATCH_BYTES];
+static_assert(FG_STATIC_SCRATCH_BYTES == fg::kWsHeaderBytes + (8u << 20), "the header documented in fastgate.h plus 8 MiB of partials");
 
 namespace fg {
 namespace {
 
 int check_launch() { return hipGetLastError() == hipSuccess ? FG_OK : FG_ERR_LAUNCH; }
 
-// The planner's rules and the [K,N] kernels' band spreading count compute units: read the current
-// device's once.  Without a device (host-only planning) the count stays at MI355X's 256.
+// The planner's rules and the [K,N] kernels' band spreading count compute units.  The entry points
+// that launch read the current device's count once, before they plan; fg_plan and
+// fg_workspace_bytes never call into the HIP runtime and plan for the count the library holds
+// at that moment (MI355X's 256 until a launch or fg_set_compute_units changed it).
+std::atomic<bool> g_cus_pinned{false};  // fg_set_compute_units was called: keep the caller's count
 void read_compute_units() {
   static std::once_flag once;
   std::call_once(once, [] {
+    if (g_cus_pinned.load()) return;
     int dev = 0, n = 0;
     if (hipGetDevice(&dev) == hipSuccess &&
         hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) {
       set_compute_units(n);
+      int x = 0;
+      if (hipDeviceGetAttribute(&x, hipDeviceAttributeNumberOfXccs, dev) == hipSuccess && x > 0) set_xccs(x);
     }
     (void)hipGetLastError();
   });
@@ -41,6 +49,7 @@ int run_gemm(const void* A, const void* W, void* C, int M, int N, int K, int acc
              const fg_plan_t& p, void* ws, size_t ws_bytes, hipStream_t s, int tail = 0,
              const void* bias = nullptr, int ldw = 0) {
   if (p.splitk > 1 && (ws == nullptr || ws_bytes < p.workspace_bytes)) return FG_ERR_WORKSPACE;
+  read_compute_units();  // the [K,N] kernels take the count as an argument
   if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(W) |
        reinterpret_cast<uintptr_t>(C) | reinterpret_cast<uintptr_t>(ws)) & 15) {
     return FG_ERR_INVALID_ARG;  // 16-byte loads and stores
@@ -50,13 +59,20 @@ int run_gemm(const void* A, const void* W, void* C, int M, int N, int K, int acc
   if (ldw != (kn ? N : K) && (!kn || ldw < N || ldw % 8 != 0)) return FG_ERR_INVALID_ARG;
   GemmArgs a{A, W, C, nullptr, nullptr, M, N, K,
              (accumulate ? kFlagAccumulate : 0) | (p.stagger ? kFlagStagger : 0) | tail, bias, ldw,
-             compute_units()};
+             compute_units(), xccs()};
   if (p.splitk > 1) {
     a.ws = reinterpret_cast<float*>(static_cast<unsigned char*>(ws) + kWsHeaderBytes);
     a.counters = p.fused ? static_cast<int*>(ws) : nullptr;
     if (p.fused == 2) {
       if (p.splitk > kFixMaxSplit || (size_t)M * N > kWsAccElems) return FG_ERR_UNSUPPORTED;
       a.accumulate |= kFlagFixSplit;
+    }
+    if (p.fused == 3 || p.fused == 4) {
+      if (p.kernel != FG_KERNEL_KN_MFMA || p.splitk > kMailboxMaxSplit ||
+          (size_t)p.grid_x * p.grid_y * p.splitk * p.waves > kWsMailboxFlags) {
+        return FG_ERR_UNSUPPORTED;
+      }
+      a.accumulate |= kFlagXcdLocal | (p.fused == 4 ? kFlagPretendForeign : 0);
     }
   }
   (void)hipGetLastError();
@@ -131,7 +147,6 @@ const char* fg_strerror(int status) {
 
 int fg_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* out) {
   if (out == nullptr || splitk < 0) return FG_ERR_INVALID_ARG;
-  fg::read_compute_units();
   int st = fg::plan_validate_shape(M, N, K, w_layout);
   if (st != FG_OK) return st;
   st = fg::plan_make(M, N, K, w_layout, splitk, out);
@@ -141,17 +156,26 @@ int fg_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* out) {
   // is the kernel boundary, without rebuilding.
   static const int forced = [] {
     const char* e = std::getenv("FASTGATE_SPLITK_COMPLETION");
-    if (e == nullptr) return -1;
+    if (e == nullptr || *e == 0) return -1;
     if (std::strcmp(e, "two-pass") == 0) return 0;
     if (std::strcmp(e, "counter") == 0) return 1;
     if (std::strcmp(e, "atomic") == 0) return 2;
+    if (std::strcmp(e, "xcd-local") == 0) return 3;
+    std::fprintf(stderr, "libfastgate: FASTGATE_SPLITK_COMPLETION=%s is not one of two-pass, counter, atomic, "
+                         "xcd-local; ignored\n", e);
     return -1;
   }();
   if (forced >= 0 && out->splitk > 1) {
-    fg_plan_t q = *out;
-    q.fused = forced;
-    if (forced == 2 && (q.splitk > fg::kFixMaxSplit || (size_t)M * N > fg::kWsAccElems)) q.fused = 1;
-    if (fg::plan_finish(M, N, K, &q) == FG_OK) *out = q;
+    // a plan the forced completion does not apply to keeps the planner's own
+    const bool applies = forced <= 1 ||
+                         (forced == 2 && out->splitk <= fg::kFixMaxSplit && (size_t)M * N <= fg::kWsAccElems) ||
+                         (forced == 3 && out->kernel == FG_KERNEL_KN_MFMA && out->splitk <= fg::kMailboxMaxSplit &&
+                          (size_t)out->grid_x * out->grid_y * out->splitk * out->waves <= fg::kWsMailboxFlags);
+    if (applies) {
+      fg_plan_t q = *out;
+      q.fused = forced;
+      if (fg::plan_finish(M, N, K, &q) == FG_OK) *out = q;
+    }
   }
   return FG_OK;
 }
@@ -163,6 +187,20 @@ size_t fg_workspace_bytes(int M, int N, int K, int w_layout, int splitk) {
 }
 
 size_t fg_workspace_header_bytes(void) { return fg::kWsHeaderBytes; }
+
+int fg_set_compute_units(int cus) {
+  if (cus < 16 || cus > 4096) return FG_ERR_INVALID_ARG;
+  fg::g_cus_pinned.store(true);
+  fg::set_compute_units(cus);
+  return FG_OK;
+}
+
+int fg_compute_units(void) { return fg::compute_units(); }
+
+int fg_use_device_compute_units(void) {
+  fg::read_compute_units();
+  return fg::compute_units();
+}
 
 int fg_workspace_init(void* ws, size_t ws_bytes, void* stream) {
   if (ws == nullptr || ws_bytes < fg::kWsHeaderBytes || (reinterpret_cast<uintptr_t>(ws) & 15)) {
@@ -176,6 +214,7 @@ int fg_workspace_init(void* ws, size_t ws_bytes, void* stream) {
 int fg_gemm_f16(const void* A, const void* W, void* C, int M, int N, int K, int w_layout,
                 int accumulate, int splitk, void* ws, size_t ws_bytes, void* stream) {
   if (A == nullptr || W == nullptr || C == nullptr) return FG_ERR_INVALID_ARG;
+  fg::read_compute_units();
   fg_plan_t p;
   int st = fg_plan(M, N, K, w_layout, splitk, &p);
   if (st != FG_OK) return st;
@@ -192,6 +231,7 @@ int fg_gemm_f16(const void* A, const void* W, void* C, int M, int N, int K, int 
 int fg_gemm_f16_static(const void* A, const void* W, void* C, int M, int N, int K, int w_layout,
                        int accumulate, int splitk, void* stream) {
   if (A == nullptr || W == nullptr || C == nullptr) return FG_ERR_INVALID_ARG;
+  fg::read_compute_units();
   fg_plan_t p;
   const int st = fg_plan(M, N, K, w_layout, splitk, &p);
   if (st != FG_OK) return st;
@@ -209,6 +249,7 @@ int fg_gemm_f16_pitched(const void* A, const void* W, void* C, int M, int N, int
                         int accumulate, int splitk, void* ws, size_t ws_bytes, void* stream) {
   if (A == nullptr || W == nullptr || C == nullptr) return FG_ERR_INVALID_ARG;
   if (ldw < N || ldw % 8 != 0) return FG_ERR_INVALID_ARG;
+  fg::read_compute_units();
   fg_plan_t p;
   int st = fg_plan(M, N, K, FG_W_KN, splitk, &p);
   if (st != FG_OK) return st;
@@ -242,6 +283,7 @@ int fg_gemm_f16_bias_act(const void* A, const void* W, const void* bias, int act
   if (act < FG_ACT_NONE || act > FG_ACT_SILU) return FG_ERR_INVALID_ARG;
   if (reinterpret_cast<uintptr_t>(bias) & 1) return FG_ERR_INVALID_ARG;
   const int tail = (bias != nullptr ? fg::kFlagBias : 0) | (act << fg::kFlagActShift);
+  fg::read_compute_units();
   fg_plan_t p;
   int st;
   if (plan == nullptr) {

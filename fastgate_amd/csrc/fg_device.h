@@ -307,6 +307,61 @@ __device__ __forceinline__ void fix_arrive(uint64_t* acc, uint32_t* clsw, const 
   }
 }
 
+// Arrival of a workgroup at its tile's counter; the ordering is splitk_last_arriver's.  Returns 1 to
+// the workgroup that arrives last (which has put the counter back to zero), 0 to the others.
+__device__ __forceinline__ int splitk_arrive(int* counter, int S, int* s_word) {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's partial stores are acknowledged
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const int old = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const bool last = old == S - 1;
+    if (last) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    *s_word = last ? 1 : 0;
+  }
+  __syncthreads();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+  return *s_word;
+}
+
+// 16 bytes of a partial that a workgroup of the same XCD stored with an ordinary store: a load that
+// is not served from this CU's L1 but by the XCD's L2, where that store landed.
+__device__ __forceinline__ float4_t load_partial4_l2(const float* base, size_t idx) {
+  constexpr int kCachePolicyWorkgroup = 1;  // sc0: not served from this CU's L1
+  return __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(
+                                          partials_rsrc(base), (int)(idx * 4), 0, kCachePolicyWorkgroup));
+}
+// NQ groups of a thread at once: sum[q] = Σ_z part[z][off[q]..+3], z ascending; the loads of all groups
+// of a batch of partials are in flight together.  Slots past S re-read the last partial and add +0.
+template <int NQ, int BATCH, bool MEM>
+__device__ __forceinline__ void sum_partials_z_batched(const float* part, int S, size_t MN, const size_t (&off)[NQ],
+                                                       float4_t (&sum)[NQ]) {
+#pragma unroll
+  for (int q = 0; q < NQ; ++q) sum[q] = float4_t{0.f, 0.f, 0.f, 0.f};
+  for (int z0 = 0; z0 < S; z0 += BATCH) {
+    float4_t v[NQ][BATCH];
+#pragma unroll
+    for (int u = 0; u < BATCH; ++u) {
+      const int z = z0 + u < S ? z0 + u : S - 1;
+#pragma unroll
+      for (int q = 0; q < NQ; ++q)
+        v[q][u] = MEM ? load_partial4(part, (size_t)z * MN + off[q]) : load_partial4_l2(part, (size_t)z * MN + off[q]);
+    }
+#pragma unroll
+    for (int u = 0; u < BATCH; ++u) {
+      const float4_t zero = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int q = 0; q < NQ; ++q) sum[q] += z0 + u < S ? v[q][u] : zero;
+    }
+  }
+}
+template <int NQ, bool MEM>
+__device__ __forceinline__ void sum_partials_z(const float* part, int S, size_t MN, const size_t (&off)[NQ],
+                                               float4_t (&sum)[NQ]) {
+  if (S <= 4) sum_partials_z_batched<NQ, 4, MEM>(part, S, MN, off, sum);
+  else sum_partials_z_batched<NQ, 8, MEM>(part, S, MN, off, sum);
+}
+
 // Σ_z part[z][off..off+3] in ascending z.  The loads of a batch are all issued before the first
 // add: one memory round trip per batch instead of one per partial (a plain `for z` loop compiles
 // to load, wait, add).  Slots past S re-read the last partial and contribute +0, which leaves

@@ -24,6 +24,20 @@ struct GemmArgs {
   const void* bias;  // fp16 [N] when bit 4 is set
   int ldw;           // elements between consecutive rows of W; [K,N] kernels only (else N or K)
   int cus;           // compute units of the device ([K,N] kernels spread column bands over them)
+  int xccs = 8;      // XCDs (L2 domains) the device dispatches workgroups to round-robin
+};
+
+// Geometry of the [K,N] MFMA kernel's one-dimensional grid.
+struct KnGeo {
+  int tiles;   // 128-column tiles of the output
+  int splitk;  // workgroups per tile
+  int cus;     // compute units of the device
+  int xccs;    // XCDs of the device
+  int spin_limit;  // polls of the mailbox owner before it recomputes what has not been delivered
+  unsigned int nonce;  // host-side enqueue number of the launch (mailbox tags), 0 when unused
+#ifdef FG_PROBE
+  int probe;   // stage after which the kernel returns (timing probes; never in the product build)
+#endif
 };
 
 // Tile sets that exist as instantiations (the planner and the validators share these).

@@ -13,6 +13,10 @@
 // (backend/cuda/hk/flatgemm.cuh:18-915) of the reference.
 #include "fg_device.h"
 #include "fg_internal.h"
+#include <atomic>
+#ifdef FG_PROBE
+#include <cstdlib>
+#endif
 
 namespace fg {
 
@@ -45,122 +49,366 @@ __device__ __forceinline__ int kn_tile(int x, int z, int gx, int cus) {
 }
 
 // ---------------------------------------------------------------------------------------
-// MFMA variant: 8 MFMAs per step, MFMA i owns the columns n0 + 8*jj + i (jj = B-operand
-// column index), so acc[i][r] = D[m = 4g + r][n = n0 + 8j + i]: a lane ends up with 8
-// consecutive columns per row, which makes the epilogue 16-byte stores.
+// MFMA variant.  The weights are the MFMA's first operand (rows of the 16 x 16 result = columns
+// of W) and the activations its second, so the result comes out transposed: MFMA i of a step owns
+// the columns n0 + 8*jj + i (jj = row of the result) and lane (j, g) ends up with
+//   acc[i][r] = C[m = j][n = n0 + 32g + 8r + i],
+// 32 consecutive columns of one row of C.  That makes every later step row-shaped: 16-byte LDS
+// writes and reads, 16-byte partial stores that fill whole 512-byte rows, 8-byte stores to C.
+//
+// Work items (column tile, K split z, row block y) come from a one-dimensional grid:
+//  * plain order: x fastest, every z plane shifted by the rounds of CUs dispatched before it
+//    (kn_tile's rule);
+//  * XCD-local order (kFlagXcdLocal): workgroups go to the XCDs round-robin by their linear id, so
+//    id % xccs names the XCD a workgroup runs on.  Every XCD is handed a contiguous run of column
+//    tiles and all S workgroups of a tile get ids that are equal modulo xccs, z ascending with the
+//    id: the partners of a tile share one L2 and one dispatch queue.
+//
+// Split-K completion in XCD-local order ("mailbox").  The partners exchange their partials with
+// ordinary stores and loads that stay in the XCD's L2 (acknowledged by the L2, not by memory) and
+// signal them with flags, without any atomic, counter or workgroup barrier on the way:
+//   partner z < S - 1   every wave stores its share of the partial, waits for the L2's
+//                       acknowledgement (vmcnt) and stores the launch's tag to its flag word;
+//   owner   z = S - 1   the partner that is dispatched last.  After its own K walk wave 0 polls the
+//                       (S - 1) x waves flags of the tile (L1-bypassing loads served by the L2),
+//                       then every thread adds the partials in ascending z, its own last, and
+//                       writes C.
+// The tag names the launch: a number the host counts up with every enqueue, the queue the
+// dispatch packet sits in and the packet's index in that queue (which also tells apart the
+// replays of a captured graph, whose kernel arguments never change).  Flags left behind by
+// earlier launches never match, so nothing has to be cleared and nothing is read or counted
+// when a workgroup starts.
+// Nothing depends on where the hardware really puts a workgroup.  Every workgroup compares the XCC id
+// register with id % xccs: a partner on another XCD does nothing (its stores would land in an L2
+// the owner cannot see), an owner on another XCD does not poll.  The owner polls a bounded
+// number of times -- partners are dispatched before it from the same queue, so their flags come
+// within microseconds -- and recomputes from A and W every partial it has no flag for, in the
+// same order of operations: the result is bit for bit the same, only later.  kFlagPretendForeign
+// makes a fifth of the workgroups claim to be misplaced (tests).
 // ---------------------------------------------------------------------------------------
-template <int U, bool STREAM, int NW>
+constexpr int kRedStride = 132;  // floats per row of the cross-wave buffer: 128 + 4 keeps 16-byte
+                                 // alignment and puts consecutive rows on different LDS banks
+
+// XCC (= XCD) the wave runs on: bits 3:0 of hardware register 20 on gfx942 / gfx950.
+__device__ __forceinline__ int xcc_id() {
+  return (int)__builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 20) & 15;
+}
+
+// AQL dispatch packet index of this launch in its queue (64-bit, counts up with every packet).
+extern "C" __device__ unsigned long long fg_dispatch_id(void) __asm("llvm.amdgcn.dispatch.id");
+
+// 64-bit name of this launch, never zero: host enqueue count (24 bits, 1..2^24-1) | queue (8 bits of
+// the queue descriptor's address) | low 32 bits of the packet index.
+__device__ __forceinline__ unsigned long long launch_tag(unsigned int nonce) {
+  const unsigned long long q = reinterpret_cast<unsigned long long>(__builtin_amdgcn_queue_ptr());
+  return ((unsigned long long)nonce << 40) | (((q >> 12) & 0xFFull) << 32) | (fg_dispatch_id() & 0xFFFFFFFFull);
+}
+
+struct KnItem {
+  int tile, z, y;
+  bool home;  // runs on the XCD its tile's partials live in (always true in plain order)
+};
+__device__ __forceinline__ KnItem kn_item(int M, int flags, const KnGeo& geo) {
+  KnItem it;
+  const int gy = (M + 15) >> 4;
+  const int per_y = (int)gridDim.x / gy;
+  const int L = (int)blockIdx.x;
+  it.y = L / per_y;
+  const int l = L - it.y * per_y;
+  it.home = true;
+  if (flags & kFlagXcdLocal) {
+    const int xcd = l % geo.xccs, n = l / geo.xccs;
+    const int tq = (geo.tiles + geo.xccs - 1) / geo.xccs;  // column tiles per XCD
+    const int a = n % tq;
+    it.z = n / tq;
+    const int round = (L - xcd - a * geo.xccs) / geo.cus;  // full rounds of CUs before this plane
+    it.tile = xcd * tq + (a + round) % tq;                 // >= tiles: nothing to do
+    it.home = geo.xccs == 1 || xcc_id() == xcd;
+    if (flags & kFlagPretendForeign) it.home = it.home && (L % 5 != 3);
+  } else {
+    const int x = l % geo.tiles;
+    it.z = l / geo.tiles;
+    const int round = (L - x) / geo.cus;
+    it.tile = (x + round) % geo.tiles;
+  }
+  return it;
+}
+
+template <int U, int NW>
 __global__ __launch_bounds__(64 * NW) void kn_mfma_kernel(const half_t* __restrict__ A,
                                                       const half_t* __restrict__ W,
                                                       half_t* __restrict__ C,
                                                       float* __restrict__ ws, int* counters, int M, int N,
-                                                      int K, int flags, const void* bias, int ldw, int cus) {
-  __shared__ float red[NW][16][128];  // NW = most waves per workgroup
+                                                      int K, int flags, const void* bias, int ldw, KnGeo geo) {
+  typedef half_t half4v __attribute__((ext_vector_type(4)));
+  constexpr int NT = 64 * NW;     // threads
+  constexpr int NQ = 512 / NT;    // 16-byte groups of the 16 x 128 tile per thread
+  __shared__ __attribute__((aligned(16))) float red[NW][16][kRedStride];
+  __shared__ int s_arrival;
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  const int nw = blockDim.x >> 6;
   const int j = lane & 15, g = lane >> 4;
-  const int tile_x = kn_tile(blockIdx.x, blockIdx.z, gridDim.x, cus);
-  const int n0 = tile_x * 128;
-  const int m0 = blockIdx.y * 16;
-  const int slots = nw * gridDim.z;
-  const int slot = blockIdx.z * nw + wave;
+  const KnItem it = kn_item(M, flags, geo);
+  const int S = geo.splitk;
+  const bool mailbox = (flags & kFlagXcdLocal) != 0 && S > 1;
+  if (it.tile >= geo.tiles) return;
+  if (mailbox && !it.home && it.z != S - 1) return;  // the owner will recompute this share
+  const int n0 = it.tile * 128;
+  const int m0 = it.y * 16;
+  const int rows = M - m0 < 16 ? M - m0 : 16;
   const int nunits = K >> 5;
-
-  float4_t acc[8];
-#pragma unroll
-  for (int i = 0; i < 8; ++i) acc[i] = float4_t{0.f, 0.f, 0.f, 0.f};
-
-  const bool arow = (m0 + j) < M;
+  const bool arow = j < rows;
   const half_t* Ap = A + (size_t)(m0 + (arow ? j : 0)) * K + g * 8;
   const half_t* Wp = W + (size_t)(g * 8) * ldw + n0 + j * 8;
-  const u32x4 zero = {0u, 0u, 0u, 0u};
 
-  for (int u0 = slot * U; u0 < nunits; u0 += slots * U) {
-    u32x4 rows[U][8];
-    u32x4 a[U];
+  // Partial sum of K split zz over this workgroup's waves: part[q] = four columns of row
+  // (q * NT + tid) / 32.  Called with zz = it.z, and by the recomputing fallback with every zz.
+  float4_t part[NQ];
+  auto compute_partial = [&](int zz) {
+    float4_t acc[8];
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int unit = u0 + u;
-      const bool ok = unit < nunits;
+    for (int i = 0; i < 8; ++i) acc[i] = float4_t{0.f, 0.f, 0.f, 0.f};
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+    const int slots = NW * S;
+    for (int u0 = (zz * NW + wave) * U; u0 < nunits; u0 += slots * U) {
+      u32x4 rws[U][8];
+      u32x4 a[U];
 #pragma unroll
-      for (int i = 0; i < 8; ++i)
-        rows[u][i] = ok ? load16<STREAM>(Wp + (size_t)(unit * 32 + i) * ldw) : zero;
-      a[u] = (ok && arow) ? load16<false>(Ap + (size_t)unit * 32) : zero;
-    }
+      for (int u = 0; u < U; ++u) {
+        const int unit = u0 + u;
+        const bool ok = unit < nunits;
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      u32x4 bt[8];
-      transpose8x8(rows[u], bt);
-#pragma unroll
-      for (int i = 0; i < 8; ++i)
-        acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(a[u]), as_half8(bt[i]), acc[i], 0,
-                                                        0, 0);
-    }
-  }
-
-#pragma unroll
-  for (int r = 0; r < 4; ++r)
-#pragma unroll
-    for (int i = 0; i < 8; ++i) red[wave][4 * g + r][8 * j + i] = acc[i][r];
-  __syncthreads();
-  if (gridDim.z > 1 && (flags & kFlagFixSplit)) {
-    // one atomic per output element, consecutive lanes on consecutive columns
-    uint64_t* facc = reinterpret_cast<uint64_t*>(reinterpret_cast<unsigned char*>(counters) + kWsCounterBytes);
-    uint32_t* fcls = reinterpret_cast<uint32_t*>(facc + kWsAccElems);
-    const int rows = M - m0 < 16 ? M - m0 : 16;
-    // up to eight elements a thread (16 rows on four waves), their atomics in flight together
-    constexpr int NB = NW >= 8 ? 4 : 8;
-    for (int base = 0; base < rows * 128; base += NB * blockDim.x) {
-      size_t idx[NB];
-      float part[NB];
-      bool valid[NB];
-#pragma unroll
-      for (int i = 0; i < NB; ++i) {
-        const int e = base + i * (int)blockDim.x + (int)threadIdx.x;
-        valid[i] = e < rows * 128;
-        const int m = valid[i] ? e >> 7 : 0, c = e & 127;
-        part[i] = lds_sum<NW>(&red[0][m][c], 16 * 128, nw);
-        idx[i] = (size_t)(m0 + m) * N + n0 + c;
+        for (int i = 0; i < 8; ++i)
+          rws[u][i] = ok ? load16<true>(Wp + (size_t)(unit * 32 + i) * ldw) : zero;
+        a[u] = (ok && arow) ? load16<false>(Ap + (size_t)unit * 32) : zero;
+#ifdef FG_PROBE
+        if (geo.probe == 101) a[u] = u32x4{0x3c003c00u, 0x3c003c00u, 0x3c003c00u, 0x3c003c00u};
+#endif
       }
-      fix_arrive<NB>(facc, fcls, idx, part, valid, gridDim.z, C, N, bias, flags);
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        u32x4 bt[8];
+        transpose8x8(rws[u], bt);
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(bt[i]), as_half8(a[u]), acc[i], 0,
+                                                          0, 0);
+      }
     }
-    return;
-  }
-  // 16 x 128 outputs in groups of four columns: the 32 lanes of a half wave cover one 512-byte row
-  // with consecutive 16-byte pieces, so every store instruction writes whole rows (partials that go
-  // out as 16 bytes at a 32-byte stride, two instructions to fill a row, take the write-through
-  // path twice as long).
-  for (int e = threadIdx.x; e < 512; e += blockDim.x) {
-    const int m = e >> 5, c0 = (e & 31) * 4;
-    const int mg = m0 + m;
-    if (mg < M) {
-      // the reads of all waves in flight before the first add
+#ifdef FG_PROBE
+    if (geo.probe >= 100 && threadIdx.x == 0 && zz == it.z) { asm volatile("s_nop 0" :: "v"(acc[0]), "v"(acc[7])); reinterpret_cast<long long*>(reinterpret_cast<unsigned char*>(counters) + kWsHeaderBytes + (80u << 20))[(size_t)blockIdx.x * 8 + 1] = wall_clock64(); }
+    if (geo.probe == 1) { part[0] = acc[0] + acc[1] + acc[2] + acc[3] + acc[4] + acc[5] + acc[6] + acc[7]; if (part[0][0] == 12345.678f) C[0] = (half_t)1.f; return; }
+#endif
+    float* mine = &red[wave][j][32 * g];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      *reinterpret_cast<float4_t*>(mine + 8 * r) = float4_t{acc[0][r], acc[1][r], acc[2][r], acc[3][r]};
+      *reinterpret_cast<float4_t*>(mine + 8 * r + 4) = float4_t{acc[4][r], acc[5][r], acc[6][r], acc[7][r]};
+    }
+    __syncthreads();
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) {
+      const int e = q * NT + (int)threadIdx.x;
       float4_t v[NW];
 #pragma unroll
-      for (int w = 0; w < NW; ++w) v[w] = *reinterpret_cast<const float4_t*>(&red[w < nw ? w : 0][m][c0]);
+      for (int w = 0; w < NW; ++w) v[w] = *reinterpret_cast<const float4_t*>(&red[w][e >> 5][(e & 31) * 4]);
       float4_t sum = {0.f, 0.f, 0.f, 0.f};
-      const float4_t zero4 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int w = 0; w < NW; ++w) sum += w < nw ? v[w] : zero4;
-      if (gridDim.z == 1) {
-        typedef half_t half4v __attribute__((ext_vector_type(4)));
-        half4v* c = reinterpret_cast<half4v*>(C + (size_t)mg * N + n0 + c0);
+      for (int w = 0; w < NW; ++w) sum += v[w];
+      part[q] = sum;
+    }
+  };
+
+  // Finished sums of this thread's groups to C (the only place that looks at the flag word's
+  // accumulate / bias / activation bits: a plain product pays one uniform branch).
+  auto write_out = [&](const float4_t (&tot)[NQ]) {
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) {
+      const int e = q * NT + (int)threadIdx.x;
+      const int m = e >> 5, c0 = (e & 31) * 4;
+      if (m >= rows) continue;
+      half4v* c = reinterpret_cast<half4v*>(C + (size_t)(m0 + m) * N + n0 + c0);
+      float4_t v = tot[q];
+      if (flags & (kFlagAccumulate | kFlagTailMask)) {
         if (flags & kFlagAccumulate) {
           const half4v old = *c;
 #pragma unroll
-          for (int i = 0; i < 4; ++i) sum[i] += static_cast<float>(old[i]);
+          for (int k = 0; k < 4; ++k) v[k] += static_cast<float>(old[k]);
         }
-        half4v out;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) out[i] = static_cast<half_t>(apply_tail(sum[i], n0 + c0 + i, bias, flags));
-        *c = out;
-      } else {
-        store_partial4(ws, ((size_t)blockIdx.z * M + mg) * N + n0 + c0, sum, counters != nullptr);
+        for (int k = 0; k < 4; ++k) v[k] = apply_tail(v[k], n0 + c0 + k, bias, flags);
       }
+      half4v out;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) out[k] = static_cast<half_t>(v[k]);
+      *c = out;
+    }
+  };
+
+#ifdef FG_PROBE
+  long long* tdbg = reinterpret_cast<long long*>(reinterpret_cast<unsigned char*>(counters) + kWsHeaderBytes + (80u << 20)) + (size_t)blockIdx.x * 8;
+  const bool tstamp = geo.probe >= 100 && threadIdx.x == 0;
+  if (tstamp) { tdbg[0] = wall_clock64(); tdbg[7] = ((long long)xcc_id() << 32) | __builtin_amdgcn_s_getreg((31 << 11) | (0 << 6) | 4); }
+#define FG_TSTAMP(i) do { if (tstamp) tdbg[i] = wall_clock64(); } while (0)
+#else
+#define FG_TSTAMP(i) do { } while (0)
+#endif
+  compute_partial(it.z);
+  FG_TSTAMP(2);
+#ifdef FG_PROBE
+  if (geo.probe == 2) { if (part[0][0] == 12345.678f) C[0] = (half_t)1.f; return; }
+#endif
+  if (S == 1) {
+    write_out(part);
+    return;
+  }
+  if (flags & kFlagFixSplit) {
+    // one atomic per output element, consecutive lanes on consecutive columns
+    uint64_t* facc = reinterpret_cast<uint64_t*>(reinterpret_cast<unsigned char*>(counters) + kWsCounterBytes);
+    uint32_t* fcls = reinterpret_cast<uint32_t*>(facc + kWsAccElems);
+    constexpr int NB = NW >= 8 ? 4 : 8;  // elements a thread: 16 x 128 over the workgroup
+    size_t idx[NB];
+    float p[NB];
+    bool valid[NB];
+#pragma unroll
+    for (int i = 0; i < NB; ++i) {
+      const int e = i * NT + (int)threadIdx.x;
+      const int m = e >> 7, c = e & 127;
+      valid[i] = m < rows;
+      float v[NW];
+#pragma unroll
+      for (int w = 0; w < NW; ++w) v[w] = red[w][m][c];
+      float sum = 0.f;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) sum += v[w];
+      p[i] = sum;
+      idx[i] = (size_t)(m0 + (valid[i] ? m : 0)) * N + n0 + c;
+    }
+    fix_arrive<NB>(facc, fcls, idx, p, valid, S, C, N, bias, flags);
+    return;
+  }
+  // partials [z][m][n]: through memory (write-through) for the counter protocol across XCDs,
+  // ordinary stores when the kernel boundary or the shared L2 makes them visible
+  const bool coherent = counters != nullptr && !mailbox;
+  const bool owner = mailbox && it.z == S - 1;
+  if (!owner) {
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) {
+      const int e = q * NT + (int)threadIdx.x;
+      const int m = e >> 5, c0 = (e & 31) * 4;
+      if (m < rows) store_partial4(ws, ((size_t)it.z * M + m0 + m) * N + n0 + c0, part[q], coherent);
     }
   }
-  finish_splitk<16, 128, true>(ws, counters, C, M, N, m0, n0, flags, bias, tile_x);
+  if (counters == nullptr) return;  // a second kernel sums the partials
+#ifdef FG_PROBE
+  if (geo.probe == 3) return;
+#endif
+  FG_TSTAMP(3);
+
+  float4_t tot[NQ];
+  size_t off[NQ];
+#pragma unroll
+  for (int q = 0; q < NQ; ++q) {
+    const int e = q * NT + (int)threadIdx.x;
+    const int m = e >> 5;
+    off[q] = (size_t)(m0 + (m < rows ? m : 0)) * N + n0 + (e & 31) * 4;
+  }
+  if (!mailbox) {
+    const int arrived = splitk_arrive(counters + it.y * geo.tiles + it.tile, S, &s_arrival);
+    FG_TSTAMP(4);
+    if (arrived == 0) return;
+#ifdef FG_PROBE
+    if (geo.probe == 4) return;
+#endif
+    sum_partials_z<NQ, true>(ws, S, (size_t)M * N, off, tot);
+    FG_TSTAMP(5);
+    write_out(tot);
+#ifdef FG_PROBE
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+#endif
+    FG_TSTAMP(6);
+    return;
+  }
+
+  // ---- mailbox ----
+  unsigned long long* mb_flags = reinterpret_cast<unsigned long long*>(reinterpret_cast<unsigned char*>(counters) + kWsMailboxFlagsOffset) +
+                                 (size_t)((it.y * geo.tiles + it.tile) * S) * NW;
+  const unsigned long long tag = launch_tag(geo.nonce);
+  if (!owner) {
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's share of the partial is in the L2
+    if (lane == 0) __hip_atomic_store(mb_flags + it.z * NW + wave, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    FG_TSTAMP(4);
+    return;
+  }
+  // owner: which partners have delivered?  Wave 0 polls, one flag per lane and pass.
+  const int nflags = (S - 1) * NW;
+  const unsigned int all = (1u << (S - 1)) - 1u;  // S <= 32
+  if (wave == 0) {
+    unsigned int ready = 0;  // bit z: all waves of partner z have flagged
+    if (it.home) {
+      bool done = false;
+      for (int spins = 0; !done && spins < geo.spin_limit; ++spins) {
+        done = true;
+        for (int base = 0; base < nflags; base += 64) {
+          const int idx = base + lane;
+          const bool ok = idx >= nflags ||
+                          __hip_atomic_load(mb_flags + idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == tag;
+          done = done && __builtin_amdgcn_ballot_w64(ok) == ~0ull;
+        }
+        if (!done) __builtin_amdgcn_s_sleep(1);
+      }
+      if (done) {
+        ready = all;
+      } else {
+        // not everything came: one more look, partner by partner (NW consecutive lanes each)
+        for (int base = 0; base < nflags; base += 64) {
+          const int idx = base + lane;
+          const bool ok = idx < nflags &&
+                          __hip_atomic_load(mb_flags + idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == tag;
+          const unsigned long long b = __builtin_amdgcn_ballot_w64(ok);
+          for (int k = 0; k < 64 / NW && base / NW + k < S - 1; ++k)
+            if (((b >> (k * NW)) & ((1ull << NW) - 1)) == ((1ull << NW) - 1)) ready |= 1u << (base / NW + k);
+        }
+      }
+    }
+    if (lane == 0) s_arrival = (int)ready;
+  }
+  __syncthreads();
+  const unsigned int ready = (unsigned int)s_arrival;
+  FG_TSTAMP(4);
+  if (ready == all) {
+    sum_partials_z<NQ, false>(ws, S - 1, (size_t)M * N, off, tot);
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) tot[q] += part[q];
+  } else {
+    // some partial is missing (its workgroup runs on another XCD, or the flag did not come in
+    // time): take what has been delivered, recompute the rest, same order of additions
+    float4_t own[NQ];
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) {
+      own[q] = part[q];
+      tot[q] = float4_t{0.f, 0.f, 0.f, 0.f};
+    }
+    for (int zz = 0; zz < S - 1; ++zz) {
+      if ((ready >> zz) & 1u) {
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) tot[q] += load_partial4_l2(ws, (size_t)zz * M * N + off[q]);
+      } else {
+        __syncthreads();  // the cross-wave buffer is read by every wave until here
+        compute_partial(zz);
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) tot[q] += part[q];
+      }
+    }
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) tot[q] += own[q];
+  }
+  FG_TSTAMP(5);
+  write_out(tot);
+#ifdef FG_PROBE
+  __builtin_amdgcn_s_waitcnt(0x0F70);
+#endif
+  FG_TSTAMP(6);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -313,23 +561,37 @@ bool launch_kn_dot2(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
 
 template <int U>
 static void kn_mfma_go(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
-  const dim3 grid(p.grid_x, p.grid_y, p.grid_z), block(p.block);
   auto* A = static_cast<const half_t*>(a.A);
   auto* W = static_cast<const half_t*>(a.W);
   auto* C = static_cast<half_t*>(a.C);
+  KnGeo geo;
+  geo.tiles = p.grid_x;
+  geo.splitk = p.splitk;
+  geo.cus = a.cus;
+  geo.xccs = a.xccs;
+  geo.spin_limit = (a.accumulate & kFlagPretendForeign) ? 64 : (1 << 18);
+  // a new number for every enqueue of a launch that uses the flags (1 .. 2^24 - 1, wrapping)
+  static std::atomic<unsigned int> enqueues{0};
+  geo.nonce = (a.accumulate & kFlagXcdLocal) ? enqueues.fetch_add(1, std::memory_order_relaxed) % 0xFFFFFFu + 1u : 0u;
+#ifdef FG_PROBE
+  { const char* e = getenv("FG_PROBE"); geo.probe = e ? atoi(e) : 0; }
+#endif
+  // one-dimensional grid: row blocks x splits x column tiles; in XCD-local order every XCD gets the
+  // same number of column tiles (the last ones may be empty)
+  const int tiles_padded = (a.accumulate & kFlagXcdLocal) ? (p.grid_x + a.xccs - 1) / a.xccs * a.xccs : p.grid_x;
+  const dim3 grid((unsigned)tiles_padded * p.splitk * p.grid_y), block(p.block);
   if (p.waves == 8) {
-    hipLaunchKernelGGL((kn_mfma_kernel<U, true, 8>), grid, block, 0, s, A, W, C, a.ws, a.counters, a.M, a.N, a.K,
-                       a.accumulate, a.bias, a.ldw, a.cus);
-  } else if (p.stream_w) {
-    hipLaunchKernelGGL((kn_mfma_kernel<U, true, 4>), grid, block, 0, s, A, W, C, a.ws, a.counters, a.M, a.N, a.K,
-                       a.accumulate, a.bias, a.ldw, a.cus);
+    hipLaunchKernelGGL((kn_mfma_kernel<U, 8>), grid, block, 0, s, A, W, C, a.ws, a.counters, a.M, a.N, a.K,
+                       a.accumulate, a.bias, a.ldw, geo);
   } else {
-    hipLaunchKernelGGL((kn_mfma_kernel<U, false, 4>), grid, block, 0, s, A, W, C, a.ws, a.counters, a.M, a.N, a.K,
-                       a.accumulate, a.bias, a.ldw, a.cus);
+    hipLaunchKernelGGL((kn_mfma_kernel<U, 4>), grid, block, 0, s, A, W, C, a.ws, a.counters, a.M, a.N, a.K,
+                       a.accumulate, a.bias, a.ldw, geo);
   }
 }
 
 bool launch_kn_mfma(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
+  if (p.waves != 4 && p.waves != 8) return false;
+  if ((long long)p.grid_x * p.splitk * p.grid_y + 8LL * p.splitk * p.grid_y > 0x7fffffffLL) return false;
   switch (p.unroll) {
     case 1: kn_mfma_go<1>(p, a, s); return true;
     case 2: kn_mfma_go<2>(p, a, s); return true;

@@ -23,6 +23,9 @@ int plan_finish(int M, int N, int K, fg_plan_t* p);
 // Compute units of the device the plans are for (default 256).
 void set_compute_units(int cus);
 int compute_units();
+// XCDs (L2 domains) of that device (default 8).
+void set_xccs(int xccs);
+int xccs();
 
 constexpr int kWsMaxTiles = (int)(kWsCounterBytes / sizeof(int));
 

@@ -38,6 +38,7 @@ namespace {
 // Compute units the rules aim at.  The rules were fitted on 256 (MI355X); the C ABI sets the
 // current device's count once.
 int kCUs = 256;
+int kXccs = 8;
 
 
 int ceil_div(int a, int b) { return (a + b - 1) / b; }
@@ -123,6 +124,7 @@ int finish_plan(int M, int N, int K, fg_plan_t* p) {
       p->tile_n = 128;
       p->m_block = 16;
       if (!kn_mfma_supported(p->unroll)) return FG_ERR_UNSUPPORTED;
+      if (p->waves != 4 && p->waves != 8) return FG_ERR_UNSUPPORTED;  // the wave count is a template argument
       break;
     default:
       return FG_ERR_UNSUPPORTED;
@@ -134,6 +136,8 @@ int finish_plan(int M, int N, int K, fg_plan_t* p) {
   if (p->grid_y > 65535) return FG_ERR_INVALID_ARG;  // HIP's limit on grid.y
   p->grid_z = p->splitk;
   p->block = 64 * p->waves;
+  if (p->fused < 0 || p->fused > 4) return FG_ERR_INVALID_ARG;
+  if (p->splitk > 1 && p->fused >= 3 && (p->kernel != FG_KERNEL_KN_MFMA || p->splitk > kMailboxMaxSplit)) return FG_ERR_UNSUPPORTED;
   if (p->splitk > 1) {
     if ((long long)p->grid_x * p->grid_y > kWsMaxTiles) p->fused = 0;
     // the in-launch completion addresses the partials with 32-bit byte offsets
@@ -595,6 +599,10 @@ void set_compute_units(int cus) {
   if (cus >= 16 && cus <= 4096) kCUs = cus;
 }
 int compute_units() { return kCUs; }
+void set_xccs(int x) {
+  if (x >= 1 && x <= 64) kXccs = x;
+}
+int xccs() { return kXccs; }
 
 int plan_validate_shape(int M, int N, int K, int w_layout) { return validate_shape(M, N, K, w_layout); }
 int plan_make(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {

@@ -96,6 +96,9 @@ const fg_plan_t& cached_plan(int M, int N, int K, int w_layout, int* status) {
   const unsigned h = ((unsigned)M * 2654435761u ^ (unsigned)N * 40503u ^ (unsigned)K * 2246822519u ^
                       (unsigned)w_layout) >> 7;
   Entry& e = table[h & 63];
+  // plans are made for the compute units of the device the tensors live on (current here)
+  static thread_local const int cus = fg_use_device_compute_units();
+  (void)cus;
   if (e.M != M || e.N != N || e.K != K || e.layout != w_layout) {
     e.status = fg_plan(M, N, K, w_layout, 0, &e.plan);
     e.M = M, e.N = N, e.K = K, e.layout = w_layout;

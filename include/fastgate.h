@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define FG_VERSION 100
+#define FG_VERSION 110
 
 typedef enum fg_status {
   FG_OK = 0,
@@ -133,7 +133,7 @@ int fg_gemm_f16(const void* A, const void* W, void* C, int M, int N, int K, int 
  * looks the array's address up and clears its workspace header; make that call outside graph
  * capture, with the device of `stream` current.
  */
-#define FG_STATIC_SCRATCH_BYTES (65536 + 3145728 + (8 << 20))
+#define FG_STATIC_SCRATCH_BYTES (65536 + 3145728 + 524288 + (8 << 20))
 int fg_gemm_f16_static(const void* A, const void* W, void* C, int M, int N, int K, int w_layout,
                        int accumulate, int splitk, void* stream);
 
@@ -176,12 +176,23 @@ int fg_gemm_f16_bias_act(const void* A, const void* W, const void* bias, int act
                          int N, int K, int w_layout, int splitk, fg_plan_t* plan, void* ws,
                          size_t ws_bytes, void* stream);
 
-/* The plan fg_gemm_f16 would use for this shape (splitk as above).  Host only. */
+/* The plan fg_gemm_f16 would use for this shape (splitk as above).  Pure host code: it never calls
+ * into the HIP runtime, so a process that only sizes buffers (or plans and then starts workers)
+ * leaves the GPU untouched.  The rules count compute units: the library plans for 256 (MI355X)
+ * until an entry point that launches has read the current device's count, or the caller set one. */
 int fg_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* out);
 
 /* Workspace bytes fg_gemm_f16 needs for this shape and splitk argument (0 when the plan
- * does not split across workgroups).  Host only. */
+ * does not split across workgroups).  Pure host code, as fg_plan. */
 size_t fg_workspace_bytes(int M, int N, int K, int w_layout, int splitk);
+
+/* Compute units the plans are made for.  fg_set_compute_units (16..4096, pure host code) pins a
+ * count, e.g. to plan on a machine without the GPU; fg_use_device_compute_units reads the count
+ * of the current HIP device once (this one initialises the HIP runtime, as every launching entry
+ * point does by itself) unless one was pinned, and returns the count in use. */
+int fg_set_compute_units(int cus);
+int fg_compute_units(void);
+int fg_use_device_compute_units(void);
 
 /* Size of the header (arrival counters, then accumulator and class words) at the start of a
  * split-K workspace, and the call that zeroes it (a fill kernel on `stream`, safe to capture in a HIP graph).  Needed once per workspace, not

@@ -30,7 +30,7 @@ def test_header_symbols_are_exported():
     L = ctypes.CDLL(str(capi.LIB_PATH))
     for n in names:
         assert getattr(L, n) is not None
-    assert capi.lib().fg_version() == 100
+    assert capi.lib().fg_version() == 110
 
 
 def test_header_is_plain_c():
