@@ -102,9 +102,19 @@ def ingest_pmc(directory: Path, capi) -> int:
                     return False
                 if int(r["Workgroup_Size"]) != p["block"] or int(r["Grid_Size"]) != wgs * p["block"]:
                     return False
-                if p["kernel_name"] == "nk_mfma_r":   # M = 8 and 16 share grid and block: first template argument
-                    m = re.search(r"nk_mfma_r_kernel(?:<|ILi)(\d+)", r["Kernel_Name"])
-                    return m is not None and int(m.group(1)) == (8 if M <= 8 else 16)
+                if p["kernel_name"] == "nk_mfma_r":
+                    # other calls of the run (M = 8 against 16, the 48-column tiles of another shape) share grid
+                    # and block: first template argument = staged activation rows, last = 16-column blocks a tile
+                    # (<AROWS, BAND, FULL, NW, CB, ...>; booleans print as words when demangled, as Lb0 / Lb1 when not)
+                    m = re.search(r"nk_mfma_r_kernel(<[^>]*>|I\w*?EE)", r["Kernel_Name"])
+                    if m is None:
+                        return False
+                    args = re.findall(r"L[ib](\d+)E", m.group(1)) if m.group(1).startswith("I") else [a.strip() for a in m.group(1)[1:-1].split(",")]
+                    return len(args) >= 5 and int(args[0]) == (8 if M <= 8 else 16) and int(args[4]) == p["tile_n"] // 16
+                if p["kernel_name"] == "kn_mfma":
+                    # <units in flight, waves>: M = 8 and M = 16 may share grid and block
+                    m = re.search(r"kn_mfma_kernel(?:<|ILi)(\d+)", r["Kernel_Name"])
+                    return m is not None and int(m.group(1)) == p["unroll"]
                 return True
             vals[counter] = mean([r for r in rows("pmc_" + counter) if match(r)])
         if vals["FETCH_SIZE"] is None or vals["WRITE_SIZE"] is None:
@@ -628,7 +638,7 @@ def main() -> int:
         per_call.append({
             "op": label, "M": M, "w_layout": "[N,K]" if layout == capi.FG_W_NK else "[K,N]",
             "kernel": p["kernel_name"], "splitk": p["splitk"], "tile_n": p["tile_n"], "waves": p["waves"],
-            "unroll": p["unroll"], "completion": ("second kernel", "counter", "atomic")[p["fused"]] if p["splitk"] > 1 else "-",
+            "unroll": p["unroll"], "completion": ("second kernel", "counter", "atomic", "flags in one L2", "flags in one L2 (test hook)")[p["fused"]] if p["splitk"] > 1 else "-",
             "plan_key": plan_key(p, M), "launches": 1 + (p["splitk"] > 1 and not p["fused"]),
             "bytes": algorithmic_bytes(M), "us_per_call": round(us, 2), "GBps": round(gbps, 1),
             "us_per_call_single_buffer": round(us_hot, 2),

@@ -296,6 +296,17 @@ __global__ __launch_bounds__(64 * NW) void kn_mfma_kernel(const half_t* __restri
     for (int q = 0; q < NQ; ++q) {
       const int e = q * NT + (int)threadIdx.x;
       const int m = e >> 5, c0 = (e & 31) * 4;
+#ifdef FG_PROBE
+      if (geo.probe == 201 || geo.probe == 202 || geo.probe == 203) {
+        const int byte = (int)((((size_t)it.z * M + m0 + m) * N + n0 + c0) * 4);
+        if (m < rows) {
+          if (geo.probe == 201) __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, part[q]), partials_rsrc(ws), byte, 0, 16);      // sc1
+          else if (geo.probe == 202) __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, part[q]), partials_rsrc(ws), byte, 0, 2);  // nt
+          else __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, part[q]), partials_rsrc(ws), byte, 0, 1);                        // sc0
+        }
+        continue;
+      }
+#endif
       if (m < rows) store_partial4(ws, ((size_t)it.z * M + m0 + m) * N + n0 + c0, part[q], coherent);
     }
   }

@@ -590,6 +590,45 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
     }
     if (atomic) p->fused = 2;
   }
+  // [K,N] MFMA kernel, up to 16 rows: completion through flags in one XCD's L2 (fused = 3).  Its
+  // partials never leave the L2 and nobody waits for an atomic, so it pays where the partials are
+  // large (nine rows and more) and it favours deeper splits of 4-wave workgroups, two or three a CU.
+  // Fitted to a sweep of 10 N x 8 K x M in {4, 8, 16} with about 100 plans a cell (us, this rule /
+  // the counter or atomic plan it replaces): N = K = 8192 M=8 24.1 / 24.7, M=16 24.5 / 25.3;
+  // N=8192 K=16384 M=16 43.8 / 46.3; N=12288 K=8192 M=8 34.4 / 36.3, K=12288 M=16 50.0 / 52.7;
+  // N=16384 K=3072 M=8 18.6 / 19.8; N=11008 K=4096 M=16 18.6 / 19.3; N=4096 K=4096 M=16 10.1 / 10.6;
+  // N=3072 K=4096 M=16 8.8 / 9.9; N=2048 K=12288 M=16 13.0 / 14.1.  Not taken where it measured level
+  // or behind: 14 336 columns, N = 16384 with few rows and long K, short K.
+  if (splitk == 0 && p->kernel == FG_KERNEL_KN_MFMA && M >= 3 && M <= 16 && p->grid_y == 1 && kXccs > 1 &&
+      p->splitk > 1) {
+    const int tiles = N / 128, units = K / 32;
+    int S = 0, w = 4, U = 1;
+    // (only the column counts the sweep covered: a split that fills the CUs unevenly costs far more
+    // than the completion saves -- 48 tiles x 6 = 288 workgroups: 25 % slower than 5 x 8 waves)
+    if (M > 8) {
+      if (tiles == 16) S = 16;
+      else if (tiles == 24 && K <= 8192 && M > 12) S = 8;
+      else if (tiles == 32) S = 8;
+      else if (tiles == 64 && K >= 8192) S = 8, U = 2;
+      else if (tiles == 86) S = 5;
+      else if (tiles == 96) S = 8;
+      else if (tiles == 128 && K <= 4096) S = 4, w = 8;
+      else if (tiles == 128) S = p->splitk, w = p->waves, U = p->unroll;
+    } else {
+      if (tiles == 64 && K >= 8192 && M >= 7) S = 8;
+      else if (tiles == 86 && K >= 3072 && K <= 4096 && M == 8) S = 5;
+      else if (tiles == 96 && K >= 4096) S = 8;
+      else if (tiles == 128 && K < 4096) S = 4, w = 8;
+      else if (tiles == 128 && K == 4096) S = p->splitk, w = p->waves, U = p->unroll;
+    }
+    // every wave keeps two K units at least; the flag words and the owner's mask have their limits
+    if (S > 1 && S <= kMailboxMaxSplit && units / (w * S * U) >= 2 &&
+        (size_t)tiles * S * w <= kWsMailboxFlags) {
+      fg_plan_t q = *p;
+      q.splitk = S, q.waves = w, q.unroll = U, q.fused = 3;
+      if (finish_plan(M, N, K, &q) == FG_OK && q.fused == 3) *p = q;
+    }
+  }
   return FG_OK;
 }
 

@@ -46,7 +46,7 @@ static void check(int M, int N, int K, int layout, int splitk) {
   REQUIRE(p.grid_x >= 1 && p.grid_y >= 1 && p.grid_y <= 65535 && p.grid_z == p.splitk && p.grid_z <= 65535);
   REQUIRE(p.waves == 1 || p.waves == 2 || p.waves == 4 || p.waves == 8);
   REQUIRE(p.block == 64 * p.waves);
-  REQUIRE(p.fused == 0 || p.fused == 1 || p.fused == 2);
+  REQUIRE(p.fused == 0 || p.fused == 1 || p.fused == 2 || p.fused == 3);
   const unsigned long long partials = 4ull * (unsigned long long)p.splitk * (unsigned long long)M * (unsigned long long)N;
   REQUIRE(p.workspace_bytes == (p.splitk > 1 ? (size_t)(fg::kWsHeaderBytes + partials) : (size_t)0));
   if (p.splitk > 1 && p.fused == 1) {
@@ -57,6 +57,14 @@ static void check(int M, int N, int K, int layout, int splitk) {
     REQUIRE(p.splitk <= fg::kFixMaxSplit);
     REQUIRE((unsigned long long)M * N <= fg::kWsAccElems);
   }
+  if (p.splitk > 1 && p.fused == 3) {
+    // flags in one XCD's L2: the [K,N] MFMA kernel only, one block of rows, within the flag words and the owner's mask
+    REQUIRE(p.kernel == FG_KERNEL_KN_MFMA && p.grid_y == 1 && splitk == 0);
+    REQUIRE(p.splitk <= fg::kMailboxMaxSplit);
+    REQUIRE((unsigned long long)p.grid_x * p.splitk * p.waves <= fg::kWsMailboxFlags);
+    REQUIRE((K / 32) / (p.waves * p.splitk * p.unroll) >= 2);
+  }
+  if (p.kernel == FG_KERNEL_KN_MFMA) REQUIRE(p.waves == 4 || p.waves == 8);
   if (splitk == 0 && M <= 16) REQUIRE(p.splitk == 1 || p.fused != 0);  // up to 16 rows complete in the launch
   // the combination is instantiated: the launchers' own validator accepts it and changes nothing
   fg_plan_t q = p;

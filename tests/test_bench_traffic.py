@@ -59,7 +59,11 @@ def test_ingest_scales_by_the_calibration_kernels(bench, tmp_path, monkeypatch):
     for M, layout in CALLS:
         p = capi.plan(M, bench.N, bench.K, layout).as_dict()
         grid = p["grid_x"] * p["grid_y"] * p["grid_z"] * p["block"]
-        name = "_ZN2fg%d%s_kernelILi%dELi1EEEvPKDF16_" % (len(p["kernel_name"]) + 7, p["kernel_name"], 8 if M <= 8 else 16)
+        # template arguments as the kernels carry them: the row-load kernel <rows, band, full, waves, column
+        # blocks, ...>, the [K,N] MFMA kernel <units in flight, waves>
+        targs = {"nk_mfma_r": "ILi%dELi128ELb1ELi8ELi%dELb0EEE" % (8 if M <= 8 else 16, p["tile_n"] // 16),
+                 "kn_mfma": "ILi%dELi%dEEE" % (p["unroll"], p["waves"])}.get(p["kernel_name"], "ILi%dELi1EEE" % M)
+        name = "_ZN2fg%d%s_kernel%svPKDF16_" % (len(p["kernel_name"]) + 7, p["kernel_name"], targs)
         for value in (1000.0 * M, 1002.0 * M):          # two dispatches: the mean counts
             fetch.append(dict(Kernel_Name=name, Counter_Name="FETCH_SIZE", Counter_Value=value, Workgroup_Size=p["block"], Grid_Size=grid))
         write.append(dict(Kernel_Name=name, Counter_Name="WRITE_SIZE", Counter_Value=10.0 * M, Workgroup_Size=p["block"], Grid_Size=grid))
@@ -76,7 +80,7 @@ def test_ingest_scales_by_the_calibration_kernels(bench, tmp_path, monkeypatch):
         key = bench.plan_key(p, M)
         keys.add(key)
         if p["kernel_name"] == "nk_mfma_r" and M == 8:
-            # M = 8 and M = 16 share grid and block; the first template argument tells them apart
+            # M = 8 and M = 16 share grid and block; the template arguments tell them apart
             assert got["entries"][key]["fetch_kib"] == 8008.0
         want = int(round((1001.0 * M * 2.0 + 10.0 * M) * 1024))
         assert got["entries"][key]["bytes"] == want, key

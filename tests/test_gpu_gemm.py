@@ -420,11 +420,12 @@ def test_planner_uses_32_row_blocks_beyond_16_rows(device, M):
 
 @pytest.mark.parametrize("M", [1, 8, 16])
 def test_planner_splits_narrow_kn_outputs(device, M):
-    # sixteen [K,N] tiles or fewer: deep splits that complete through atomics (the pinned factors are
-    # in tests/test_host.py) -- each checked against the oracle through the library's plan
+    # sixteen [K,N] tiles or fewer: deep splits that complete through atomics, or for nine rows and more
+    # through flags in one L2 (the pinned factors are in tests/test_host.py) -- each checked against the
+    # oracle through the library's plan
     for (N, K) in ((2048, 4096), (2048, 8192), (1024, 16384), (2048, 16384), (1024, 11008)):
         p = capi.plan(M, N, K, KN, 0)
-        assert p.splitk >= 12 and p.fused == 2, p.as_dict()
+        assert p.splitk >= 12 and p.fused in (2, 3), p.as_dict()
         A, W = _case(M, N, K, KN, 140 + M)
         ref, _ = oracle.gemm_f16(A.numpy(), W.numpy(), KN)
         got, _ = _run(A, W, KN, device)

@@ -120,8 +120,7 @@ def test_plan_choices_that_were_measured():
     # sixteen column tiles or fewer: deep splits (they complete through atomics), four waves for one
     # or two rows from nine tiles on
     for (M, N, K, S, W) in ((1, 2048, 4096, 24, 4), (1, 2048, 16384, 24, 4), (8, 2048, 8192, 16, 8),
-                            (16, 2048, 8192, 12, 8), (16, 2048, 16384, 16, 8), (1, 1024, 16384, 24, 8),
-                            (16, 1024, 28672, 24, 8), (16, 1024, 8192, 24, 8)):
+                            (1, 1024, 16384, 24, 8), (16, 1024, 28672, 24, 8), (16, 1024, 8192, 24, 8)):
         p = kn(M, N, K)
         assert (p.splitk, p.waves, p.fused) == (S, W, 2), (M, N, K, p.as_dict())
     # one or two rows: v_dot2 up to 2^28 weights (two rows beyond 2^27 only up to N = 12288)
@@ -135,15 +134,26 @@ def test_plan_choices_that_were_measured():
         assert (p.kernel, p.splitk, p.waves) == (capi.FG_KERNEL_KN_DOT2, S, 4), (M, N, K, p.as_dict())
     # completion of the split: atomics for v_dot2, for [N,K] and for few elements; the counter otherwise
     assert kn(1, 8192, 8192).fused == 2 and kn(8, 4096, 4096).fused == 2 and nk(16, 2048, 8192).fused == 2
-    assert kn(8, 8192, 8192).fused == 1 and kn(16, 8192, 8192).fused == 1 and kn(16, 12288, 8192).fused == 1
+    assert kn(4, 8192, 8192).fused == 1 and kn(16, 5120, 8192).fused == 1 and kn(8, 14336, 8192).fused == 1
     # the [K,N] MFMA kernel: atomics only for deep splits or few elements (four waves: from 8 splits on)
-    assert kn(4, 8192, 8192).fused == 1 and kn(16, 4096, 4096).fused == 1 and kn(16, 4096, 11008).fused == 1
-    assert kn(8, 11008, 4096).fused == 2 and kn(16, 2048, 16384).fused == 2
+    assert kn(8, 4096, 8192).fused == 2 and kn(8, 11008, 2048).fused == 2
+    # ... and flags in one XCD's L2 where the partials are large, with two or three 4-wave workgroups a
+    # CU: (M, N, K) -> (split, waves, units in flight)
+    for (M, N, K, S, W, U) in ((8, 8192, 8192, 8, 4, 1), (16, 8192, 8192, 8, 4, 2), (16, 8192, 16384, 8, 4, 2),
+                               (8, 12288, 8192, 8, 4, 1), (16, 12288, 12288, 8, 4, 1), (4, 12288, 4096, 8, 4, 1),
+                               (16, 4096, 4096, 8, 4, 1), (16, 4096, 11008, 8, 4, 1), (16, 3072, 4096, 8, 4, 1),
+                               (16, 2048, 8192, 16, 4, 1), (16, 2048, 16384, 16, 4, 1), (16, 11008, 4096, 5, 4, 1),
+                               (8, 11008, 4096, 5, 4, 1), (8, 16384, 2048, 4, 8, 1), (16, 16384, 16384, 2, 4, 1)):
+        p = kn(M, N, K)
+        assert (p.splitk, p.waves, p.unroll, p.fused) == (S, W, U, 3), (M, N, K, p.as_dict())
+    # not where the sweep did not go (48 tiles x 6 splits would fill the CUs unevenly) or measured level
+    assert kn(16, 6144, 8192).fused != 3 and kn(16, 14336, 8192).fused != 3 and kn(8, 16384, 8192).fused != 3
+    assert kn(6, 8192, 8192).fused != 3 and kn(16, 8192, 4096).fused != 3
     assert kn(24, 2048, 4096).fused == 0           # more than 16 rows: second kernel
     p = kn(16, 5120, 8192)
     assert (p.splitk, p.waves) == (6, 8)
     p = kn(12, 4096, 2048)
-    assert (p.splitk, p.waves) == (4, 8)
+    assert (p.splitk, p.waves, p.fused) == (8, 4, 3)    # 7.65 us against 8.34 for four splits of 8 waves and the counter
     assert kn(16, 2048, 2048).splitk == 8
     # one or two rows: two 4-wave workgroups a CU where that lands on 448..512 workgroups
     for (N, K, S) in ((8192, 14336, 8), (8192, 4096, 8), (16384, 5120, 4), (4096, 11008, 16), (10240, 4096, 6)):
