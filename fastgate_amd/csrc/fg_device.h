@@ -333,9 +333,13 @@ __device__ __forceinline__ float4_t load_partial4_l2(const float* base, size_t i
 }
 // NQ groups of a thread at once: sum[q] = Σ_z part[z][off[q]..+3], z ascending; the loads of all groups
 // of a batch of partials are in flight together.  Slots past S re-read the last partial and add +0.
+// Offsets are bytes: the lane's own in the vector offset, z * (bytes of one partial) in the scalar
+// offset of the buffer load, so a load costs one instruction (the buffer is below 2 GiB).
 template <int NQ, int BATCH, bool MEM>
-__device__ __forceinline__ void sum_partials_z_batched(const float* part, int S, size_t MN, const size_t (&off)[NQ],
+__device__ __forceinline__ void sum_partials_z_batched(const float* part, int S, int z_bytes, const int (&off)[NQ],
                                                        float4_t (&sum)[NQ]) {
+  constexpr int kPolicy = MEM ? kCachePolicyAgent : 1;  // sc1: past the L2s; sc0: past this CU's L1 only
+  const __amdgpu_buffer_rsrc_t rsrc = partials_rsrc(part);
 #pragma unroll
   for (int q = 0; q < NQ; ++q) sum[q] = float4_t{0.f, 0.f, 0.f, 0.f};
   for (int z0 = 0; z0 < S; z0 += BATCH) {
@@ -345,7 +349,7 @@ __device__ __forceinline__ void sum_partials_z_batched(const float* part, int S,
       const int z = z0 + u < S ? z0 + u : S - 1;
 #pragma unroll
       for (int q = 0; q < NQ; ++q)
-        v[q][u] = MEM ? load_partial4(part, (size_t)z * MN + off[q]) : load_partial4_l2(part, (size_t)z * MN + off[q]);
+        v[q][u] = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc, off[q], z * z_bytes, kPolicy));
     }
 #pragma unroll
     for (int u = 0; u < BATCH; ++u) {
@@ -356,10 +360,10 @@ __device__ __forceinline__ void sum_partials_z_batched(const float* part, int S,
   }
 }
 template <int NQ, bool MEM>
-__device__ __forceinline__ void sum_partials_z(const float* part, int S, size_t MN, const size_t (&off)[NQ],
+__device__ __forceinline__ void sum_partials_z(const float* part, int S, int z_bytes, const int (&off)[NQ],
                                                float4_t (&sum)[NQ]) {
-  if (S <= 4) sum_partials_z_batched<NQ, 4, MEM>(part, S, MN, off, sum);
-  else sum_partials_z_batched<NQ, 8, MEM>(part, S, MN, off, sum);
+  if (S <= 4) sum_partials_z_batched<NQ, 4, MEM>(part, S, z_bytes, off, sum);
+  else sum_partials_z_batched<NQ, 8, MEM>(part, S, z_bytes, off, sum);
 }
 
 // Σ_z part[z][off..off+3] in ascending z.  The loads of a batch are all issued before the first

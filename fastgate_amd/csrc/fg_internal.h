@@ -33,6 +33,8 @@ struct KnGeo {
   int splitk;  // workgroups per tile
   int cus;     // compute units of the device
   int xccs;    // XCDs of the device
+  int tq;      // column tiles per XCD in XCD-local order: ceil(tiles / xccs)
+  int log2_tiles, log2_tq, log2_xccs, log2_cus;  // log2 of those that are powers of two, else -1
   int spin_limit;  // polls of the mailbox owner before it recomputes what has not been delivered
   unsigned int nonce;  // host-side enqueue number of the launch (mailbox tags), 0 when unused
 #ifdef FG_PROBE

@@ -108,34 +108,43 @@ struct KnItem {
   int tile, z, y;
   bool home;  // runs on the XCD its tile's partials live in (always true in plain order)
 };
+// x / d and x % d for a divisor whose log2 the host passes when it is a power of two (-1 otherwise):
+// the usual tile, XCD and CU counts are, and a division by a run-time value costs some 40
+// instructions before the workgroup's first load can go out.
+__device__ __forceinline__ int div_by(int x, int d, int log2d) { return log2d >= 0 ? x >> log2d : x / d; }
+__device__ __forceinline__ int mod_by(int x, int d, int log2d) { return log2d >= 0 ? x & (d - 1) : x % d; }
+
 __device__ __forceinline__ KnItem kn_item(int M, int flags, const KnGeo& geo) {
   KnItem it;
-  const int gy = (M + 15) >> 4;
-  const int per_y = (int)gridDim.x / gy;
   const int L = (int)blockIdx.x;
-  it.y = L / per_y;
-  const int l = L - it.y * per_y;
+  int l = L;
+  it.y = 0;
+  if (M > 16) {  // more than one block of rows: the grid repeats per block
+    const int per_y = (int)gridDim.x / ((M + 15) >> 4);
+    it.y = L / per_y;
+    l = L - it.y * per_y;
+  }
   it.home = true;
   if (flags & kFlagXcdLocal) {
-    const int xcd = l % geo.xccs, n = l / geo.xccs;
-    const int tq = (geo.tiles + geo.xccs - 1) / geo.xccs;  // column tiles per XCD
-    const int a = n % tq;
-    it.z = n / tq;
-    const int round = (L - xcd - a * geo.xccs) / geo.cus;  // full rounds of CUs before this plane
-    it.tile = xcd * tq + (a + round) % tq;                 // >= tiles: nothing to do
+    const int xcd = mod_by(l, geo.xccs, geo.log2_xccs), n = div_by(l, geo.xccs, geo.log2_xccs);
+    const int a = mod_by(n, geo.tq, geo.log2_tq);
+    it.z = div_by(n, geo.tq, geo.log2_tq);
+    const int round = div_by(L - xcd - a * geo.xccs, geo.cus, geo.log2_cus);  // full rounds of CUs before this plane
+    it.tile = xcd * geo.tq + mod_by(a + round, geo.tq, geo.log2_tq);           // >= tiles: nothing to do
     it.home = geo.xccs == 1 || xcc_id() == xcd;
     if (flags & kFlagPretendForeign) it.home = it.home && (L % 5 != 3);
   } else {
-    const int x = l % geo.tiles;
-    it.z = l / geo.tiles;
-    const int round = (L - x) / geo.cus;
-    it.tile = (x + round) % geo.tiles;
+    const int x = mod_by(l, geo.tiles, geo.log2_tiles);
+    it.z = div_by(l, geo.tiles, geo.log2_tiles);
+    const int round = div_by(L - x, geo.cus, geo.log2_cus);
+    it.tile = mod_by(x + round, geo.tiles, geo.log2_tiles);
   }
   return it;
 }
 
+// (8 waves with one K unit in flight: two workgroups must fit a CU, i.e. four waves a SIMD, at most 128 registers)
 template <int U, int NW>
-__global__ __launch_bounds__(64 * NW) void kn_mfma_kernel(const half_t* __restrict__ A,
+__global__ __launch_bounds__(64 * NW, (NW == 8 && U == 1) ? 4 : 1) void kn_mfma_kernel(const half_t* __restrict__ A,
                                                       const half_t* __restrict__ W,
                                                       half_t* __restrict__ C,
                                                       float* __restrict__ ws, int* counters, int M, int N,
@@ -145,11 +154,13 @@ __global__ __launch_bounds__(64 * NW) void kn_mfma_kernel(const half_t* __restri
   constexpr int NQ = 512 / NT;    // 16-byte groups of the 16 x 128 tile per thread
   __shared__ __attribute__((aligned(16))) float red[NW][16][kRedStride];
   __shared__ int s_arrival;
+  __shared__ int s_state;  // the mailbox owner's waves agree here (see there)
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int j = lane & 15, g = lane >> 4;
   const KnItem it = kn_item(M, flags, geo);
   const int S = geo.splitk;
+  if (threadIdx.x == 0) s_state = 0;  // published by the barrier of the cross-wave sum
   const bool mailbox = (flags & kFlagXcdLocal) != 0 && S > 1;
   if (it.tile >= geo.tiles) return;
   if (mailbox && !it.home && it.z != S - 1) return;  // the owner will recompute this share
@@ -317,12 +328,13 @@ __global__ __launch_bounds__(64 * NW) void kn_mfma_kernel(const half_t* __restri
   FG_TSTAMP(3);
 
   float4_t tot[NQ];
-  size_t off[NQ];
+  int off[NQ];                      // byte offset of the thread's groups within one partial
+  const int z_bytes = M * N * 4;    // the in-launch completions keep all partials below 2 GiB
 #pragma unroll
   for (int q = 0; q < NQ; ++q) {
     const int e = q * NT + (int)threadIdx.x;
     const int m = e >> 5;
-    off[q] = (size_t)(m0 + (m < rows ? m : 0)) * N + n0 + (e & 31) * 4;
+    off[q] = ((m0 + (m < rows ? m : 0)) * N + n0 + (e & 31) * 4) * 4;
   }
   if (!mailbox) {
     const int arrived = splitk_arrive(counters + it.y * geo.tiles + it.tile, S, &s_arrival);
@@ -331,7 +343,7 @@ __global__ __launch_bounds__(64 * NW) void kn_mfma_kernel(const half_t* __restri
 #ifdef FG_PROBE
     if (geo.probe == 4) return;
 #endif
-    sum_partials_z<NQ, true>(ws, S, (size_t)M * N, off, tot);
+    sum_partials_z<NQ, true>(ws, S, z_bytes, off, tot);
     FG_TSTAMP(5);
     write_out(tot);
 #ifdef FG_PROBE
@@ -351,44 +363,124 @@ __global__ __launch_bounds__(64 * NW) void kn_mfma_kernel(const half_t* __restri
     FG_TSTAMP(4);
     return;
   }
-  // owner: which partners have delivered?  Wave 0 polls, one flag per lane and pass.
-  const int nflags = (S - 1) * NW;
+  // Owner, up to eight partners (one flag per lane, one pass): every wave polls for itself and
+  // loads a partner's partial the moment that partner's flags are up.  Partials of partners that
+  // finished microseconds ago have left the L2 by now; loading them while waiting for the last
+  // partner takes that memory latency off the end of the kernel.  The values wait in registers and
+  // are added in ascending z afterwards.  The waves do not meet at a barrier, so they agree through
+  // one LDS word on whether anybody gives up: 0 undecided, 1 some wave has seen every flag (then
+  // every wave will), 2 wave 0 has polled `spin_limit` times in vain (everybody recomputes).
+  constexpr int PF = 8;
   const unsigned int all = (1u << (S - 1)) - 1u;  // S <= 32
-  if (wave == 0) {
-    unsigned int ready = 0;  // bit z: all waves of partner z have flagged
-    if (it.home) {
-      bool done = false;
-      for (int spins = 0; !done && spins < geo.spin_limit; ++spins) {
-        done = true;
-        for (int base = 0; base < nflags; base += 64) {
-          const int idx = base + lane;
-          const bool ok = idx >= nflags ||
-                          __hip_atomic_load(mb_flags + idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == tag;
-          done = done && __builtin_amdgcn_ballot_w64(ok) == ~0ull;
-        }
-        if (!done) __builtin_amdgcn_s_sleep(1);
-      }
-      if (done) {
-        ready = all;
-      } else {
-        // not everything came: one more look, partner by partner (NW consecutive lanes each)
-        for (int base = 0; base < nflags; base += 64) {
-          const int idx = base + lane;
-          const bool ok = idx < nflags &&
-                          __hip_atomic_load(mb_flags + idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == tag;
-          const unsigned long long b = __builtin_amdgcn_ballot_w64(ok);
-          for (int k = 0; k < 64 / NW && base / NW + k < S - 1; ++k)
-            if (((b >> (k * NW)) & ((1ull << NW) - 1)) == ((1ull << NW) - 1)) ready |= 1u << (base / NW + k);
+  if (it.home && S - 1 <= PF && (S - 1) * NW <= 64) {
+    const int nflags = (S - 1) * NW;
+    const __amdgpu_buffer_rsrc_t rsrc = partials_rsrc(ws);
+    float4_t v[PF][NQ];
+#pragma unroll
+    for (int z = 0; z < PF; ++z)
+#pragma unroll
+      for (int q = 0; q < NQ; ++q) v[z][q] = float4_t{0.f, 0.f, 0.f, 0.f};
+    unsigned int loaded = 0;
+    bool give_up = false;
+    for (int spins = 0;; ++spins) {
+      const bool ok = lane >= nflags ||
+                      __hip_atomic_load(mb_flags + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == tag;
+      const unsigned long long b = __builtin_amdgcn_ballot_w64(ok);
+#pragma unroll
+      for (int z = 0; z < PF; ++z) {
+        const unsigned long long lanes = ((1ull << NW) - 1) << (z * NW);
+        if (z < S - 1 && !((loaded >> z) & 1u) && (b & lanes) == lanes) {
+#pragma unroll
+          for (int q = 0; q < NQ; ++q)
+            v[z][q] = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc, off[q], z * z_bytes, 1));
+          loaded |= 1u << z;
         }
       }
+      if (loaded == all) break;
+      if (__hip_atomic_load(&s_state, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) == 2) {
+        give_up = true;
+        break;
+      }
+      if (wave == 0 && spins >= geo.spin_limit) {
+        int seen = 0;
+        if (lane == 0) {
+          __hip_atomic_compare_exchange_strong(&s_state, &seen, 2, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                               __HIP_MEMORY_SCOPE_WORKGROUP);
+        }
+        seen = __builtin_amdgcn_readfirstlane(seen);
+        if (seen != 1) {  // nobody has everything: give up (a wave that has, keeps the others going)
+          give_up = true;
+          break;
+        }
+      }
+      __builtin_amdgcn_s_sleep(1);
     }
-    if (lane == 0) s_arrival = (int)ready;
+    if (!give_up) {
+      int seen = 0;
+      if (lane == 0) {
+        __hip_atomic_compare_exchange_strong(&s_state, &seen, 1, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                             __HIP_MEMORY_SCOPE_WORKGROUP);
+      }
+      give_up = __builtin_amdgcn_readfirstlane(seen) == 2;
+    }
+    if (!give_up) {
+      FG_TSTAMP(4);
+#pragma unroll
+      for (int q = 0; q < NQ; ++q) {
+        float4_t sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int z = 0; z < PF; ++z) sum += v[z][q];  // partners past S - 1 stayed +0
+        tot[q] = sum + part[q];
+      }
+      FG_TSTAMP(5);
+      write_out(tot);
+#ifdef FG_PROBE
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+#endif
+      FG_TSTAMP(6);
+      return;
+    }
+    // every wave arrives here: recompute all partials (what was loaded is not used)
+    if (threadIdx.x == 0) s_arrival = 0;
+  } else {
+    // owner: which partners have delivered?  Wave 0 polls, one flag per lane and pass.
+    const int nflags = (S - 1) * NW;
+    if (wave == 0) {
+      unsigned int ready = 0;  // bit z: all waves of partner z have flagged
+      if (it.home) {
+        bool done = false;
+        for (int spins = 0; !done && spins < geo.spin_limit; ++spins) {
+          done = true;
+          for (int base = 0; base < nflags; base += 64) {
+            const int idx = base + lane;
+            const bool ok = idx >= nflags ||
+                            __hip_atomic_load(mb_flags + idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == tag;
+            done = done && __builtin_amdgcn_ballot_w64(ok) == ~0ull;
+          }
+          if (!done) __builtin_amdgcn_s_sleep(1);
+        }
+        if (done) {
+          ready = all;
+        } else {
+          // not everything came: one more look, partner by partner (NW consecutive lanes each)
+          for (int base = 0; base < nflags; base += 64) {
+            const int idx = base + lane;
+            const bool ok = idx < nflags &&
+                            __hip_atomic_load(mb_flags + idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == tag;
+            const unsigned long long b = __builtin_amdgcn_ballot_w64(ok);
+            for (int k = 0; k < 64 / NW && base / NW + k < S - 1; ++k)
+              if (((b >> (k * NW)) & ((1ull << NW) - 1)) == ((1ull << NW) - 1)) ready |= 1u << (base / NW + k);
+          }
+        }
+      }
+      if (lane == 0) s_arrival = (int)ready;
+    }
   }
   __syncthreads();
   const unsigned int ready = (unsigned int)s_arrival;
   FG_TSTAMP(4);
   if (ready == all) {
-    sum_partials_z<NQ, false>(ws, S - 1, (size_t)M * N, off, tot);
+    sum_partials_z<NQ, false>(ws, S - 1, z_bytes, off, tot);
 #pragma unroll
     for (int q = 0; q < NQ; ++q) tot[q] += part[q];
   } else {
@@ -403,7 +495,7 @@ __global__ __launch_bounds__(64 * NW) void kn_mfma_kernel(const half_t* __restri
     for (int zz = 0; zz < S - 1; ++zz) {
       if ((ready >> zz) & 1u) {
 #pragma unroll
-        for (int q = 0; q < NQ; ++q) tot[q] += load_partial4_l2(ws, (size_t)zz * M * N + off[q]);
+        for (int q = 0; q < NQ; ++q) tot[q] += load_partial4_l2(ws, (size_t)zz * M * N + (size_t)(off[q] >> 2));
       } else {
         __syncthreads();  // the cross-wave buffer is read by every wave until here
         compute_partial(zz);
@@ -580,6 +672,14 @@ static void kn_mfma_go(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
   geo.splitk = p.splitk;
   geo.cus = a.cus;
   geo.xccs = a.xccs;
+  geo.tq = (p.grid_x + a.xccs - 1) / a.xccs;
+  auto log2_of = [](int v) {
+    int l = -1;
+    if (v > 0 && (v & (v - 1)) == 0)
+      for (l = 0; (1 << l) < v; ++l) {}
+    return l;
+  };
+  geo.log2_tiles = log2_of(geo.tiles), geo.log2_tq = log2_of(geo.tq), geo.log2_xccs = log2_of(geo.xccs), geo.log2_cus = log2_of(geo.cus);
   geo.spin_limit = (a.accumulate & kFlagPretendForeign) ? 64 : (1 << 18);
   // a new number for every enqueue of a launch that uses the flags (1 .. 2^24 - 1, wrapping)
   static std::atomic<unsigned int> enqueues{0};
