@@ -20,7 +20,7 @@ FG_ERR_WORKSPACE = -3
 FG_ERR_LAUNCH = -4
 FG_ERR_UNSUPPORTED = -5
 FG_ERR_SCRATCH_LIMIT = -6
-FG_STATIC_SCRATCH_BYTES = 65536 + 3145728 + (8 << 20)
+FG_STATIC_SCRATCH_BYTES = 65536 + 3145728 + 524288 + (8 << 20)
 
 FG_W_KN = 0
 FG_W_NK = 1

@@ -231,12 +231,15 @@ __device__ __forceinline__ bool splitk_last_arriver(int* counter, int S) {
 // tile may be completed by different workgroups.
 //   word = value (54 bits, two's complement, units of 2^-28) | poisoned arrivals (5) | arrivals (5)
 // A partial that fixed point cannot hold (NaN, infinite, or |p| >= 2^20, sixteen times the fp16
-// range) arrives "poisoned": value 0, its class (NaN, +overflow, -overflow) counted in a second
-// word of the element, written before the arrival with release / acquire fences around the
-// pair (that path alone pays for agent-scope fences).
+// range) arrives "poisoned": value 0, the fp32 partial itself stored in its slot [z][m][n] of the
+// partial area behind the header, and bit z set in a second word of the element, both before the
+// arrival, with release / acquire fences around the pair (that path alone pays for agent-scope
+// fences and for memory beyond the header).  The thread that completes a poisoned element adds the
+// flagged partials in ascending z, in fp32, to the fixed-point sum of the others: two huge
+// partials of opposite sign cancel as they do in every other completion, and NaN and the
+// infinities follow from fp32 arithmetic.
 // ---------------------------------------------------------------------------------------
 constexpr float kFixLimit = 1048576.f;  // 2^20
-constexpr uint32_t kFixNaN = 1u, kFixPos = 1u << 8, kFixNeg = 1u << 16;
 
 // Fixed-point image of p (|p| < 2^20) in units of 2^-28, rounded to nearest: exact for every fp32
 // value of magnitude 2^-4 or more, off by at most 2^-29 below (the smallest fp16 step is 2^-24).
@@ -251,38 +254,31 @@ __device__ __forceinline__ float fix_to_float(int64_t v) {
   const double d = (double)(int)(v >> 24) * 16777216.0 + (double)(int)(v & 0xFFFFFF);
   return (float)d * 3.7252902984619140625e-09f;          // 2^-28
 }
-__device__ __forceinline__ uint32_t fix_class(float p) {
-  if (__builtin_fabsf(p) < kFixLimit) return 0u;
-  return p != p ? kFixNaN : (p > 0.f ? kFixPos : kFixNeg);
-}
+// True for a partial that must arrive poisoned (the comparison is false for NaN).
+__device__ __forceinline__ bool fix_poisoned(float p) { return !(__builtin_fabsf(p) < kFixLimit); }
 // Word a partial arrives with.
-__device__ __forceinline__ uint64_t fix_word(float p, uint32_t cls) {
-  if (cls) return (1ull << 5) | 1ull;
+__device__ __forceinline__ uint64_t fix_word(float p, bool poisoned) {
+  if (poisoned) return (1ull << 5) | 1ull;
   return ((uint64_t)fix_from_float(p) << 10) | 1ull;
 }
-// Sum a complete word stands for; `cls` is the element's class word (read only when poisoned).
-__device__ __forceinline__ float fix_total(uint64_t word, uint32_t cls) {
-  if ((word >> 5) & 31u) {
-    const bool nan = (cls & 0xFFu) != 0, pos = (cls & 0xFF00u) != 0, neg = (cls & 0xFF0000u) != 0;
-    if (nan || (pos && neg)) return __builtin_nanf("");
-    return pos ? __builtin_inff() : -__builtin_inff();
-  }
-  return fix_to_float((int64_t)word >> 10);
-}
 
-// NB elements of one thread: partial p[i] of output element idx[i] (= m * N + n) arrives; the
-// atomics of the batch are issued back to back before the first result is looked at.
+// NB elements of one thread: partial p[i] of output element idx[i] (= m * N + n) from K range z
+// arrives; the atomics of the batch are issued back to back before the first result is looked
+// at.  `part` is the partial area ([S][MN] floats), touched for poisoned partials only; `maskw`
+// holds one word per element (bit z: slot z of the element holds a poisoned partial).
 template <int NB>
-__device__ __forceinline__ void fix_arrive(uint64_t* acc, uint32_t* clsw, const size_t (&idx)[NB],
-                                           const float (&p)[NB], const bool (&valid)[NB], int S,
-                                           half_t* C, int N, const void* bias, int flags) {
+__device__ __forceinline__ void fix_arrive(uint64_t* acc, uint32_t* maskw, float* part, int z, size_t MN,
+                                           const size_t (&idx)[NB], const float (&p)[NB],
+                                           const bool (&valid)[NB], int S, half_t* C, int N,
+                                           const void* bias, int flags) {
   uint64_t own[NB], old[NB];
 #pragma unroll
   for (int i = 0; i < NB; ++i) {
-    const uint32_t cls = fix_class(p[i]);
-    own[i] = fix_word(p[i], cls);
-    if (valid[i] && cls) {
-      __hip_atomic_fetch_add(clsw + idx[i], cls, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const bool poisoned = fix_poisoned(p[i]);
+    own[i] = fix_word(p[i], poisoned);
+    if (valid[i] && poisoned) {
+      __hip_atomic_store(part + (size_t)z * MN + idx[i], p[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_fetch_or(maskw + idx[i], 1u << z, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
     }
   }
@@ -295,15 +291,22 @@ __device__ __forceinline__ void fix_arrive(uint64_t* acc, uint32_t* clsw, const 
   for (int i = 0; i < NB; ++i) {
     if (!valid[i] || (int)(old[i] & 31u) != S - 1) continue;
     const uint64_t word = old[i] + own[i];
-    uint32_t cls = 0;
+    float total = fix_to_float((int64_t)word >> 10);
     if ((word >> 5) & 31u) {
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-      cls = __hip_atomic_load(clsw + idx[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      __hip_atomic_store(clsw + idx[i], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      uint32_t mask = __hip_atomic_load(maskw + idx[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(maskw + idx[i], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      float huge = 0.f;
+      while (mask) {
+        const int zz = __builtin_ctz(mask);
+        mask &= mask - 1u;
+        huge += __hip_atomic_load(part + (size_t)zz * MN + idx[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      total += huge;
     }
     __hip_atomic_store(acc + idx[i], 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     half_t* c = C + idx[i];
-    *c = finish_value(fix_total(word, cls), c, (int)(idx[i] % (size_t)N), bias, flags);
+    *c = finish_value(total, c, (int)(idx[i] % (size_t)N), bias, flags);
   }
 }
 
@@ -437,7 +440,7 @@ __device__ __forceinline__ void publish_partial(float* ws, int* counters, half_t
     const size_t idx[1] = {(size_t)mg * N + n};
     const float part[1] = {sum};
     const bool valid[1] = {true};
-    fix_arrive<1>(facc, fcls, idx, part, valid, gridDim.z, C, N, bias, flags);
+    fix_arrive<1>(facc, fcls, ws, (int)blockIdx.z, (size_t)M * N, idx, part, valid, gridDim.z, C, N, bias, flags);
   } else {
     store_partial(ws + ((size_t)blockIdx.z * M + mg) * N + n, sum, counters != nullptr);
   }

@@ -295,7 +295,7 @@ __global__ __launch_bounds__(64 * NW, (NW == 8 && U == 1) ? 4 : 1) void kn_mfma_
       p[i] = sum;
       idx[i] = (size_t)(m0 + (valid[i] ? m : 0)) * N + n0 + c;
     }
-    fix_arrive<NB>(facc, fcls, idx, p, valid, S, C, N, bias, flags);
+    fix_arrive<NB>(facc, fcls, ws, it.z, (size_t)M * N, idx, p, valid, S, C, N, bias, flags);
     return;
   }
   // partials [z][m][n]: through memory (write-through) for the counter protocol across XCDs,
@@ -595,7 +595,7 @@ __global__ __launch_bounds__(64 * NW) void kn_dot2_kernel(const half_t* __restri
         part[i] = lds_sum<4 * NW>(&red[0][m][nn], MB * 128, nw * 4);
         idx[i] = (size_t)(m0 + m) * N + n0 + nn;
       }
-      fix_arrive<NB>(facc, fcls, idx, part, valid, gridDim.z, C, N, bias, flags);
+      fix_arrive<NB>(facc, fcls, ws, (int)blockIdx.z, (size_t)M * N, idx, part, valid, gridDim.z, C, N, bias, flags);
     }
     return;
   }

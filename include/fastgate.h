@@ -65,18 +65,29 @@ enum {
  */
 typedef struct fg_plan_t {
   int kernel;   /* FG_KERNEL_*                                                        */
-  int splitk;   /* S >= 1: K is divided over S workgroups per output tile; S > 1 writes
-                   fp32 partials [S,M,N] to the workspace; they are summed in ascending
-                   order of S, so results are reproducible (no data atomics)          */
-  int fused;    /* with S > 1, how the split completes: 0 = a second kernel sums the partials;
-                   1 = the workgroup that finishes a tile last sums them in the same launch
-                   (one counter atomic per workgroup); 2 = every workgroup adds its partial,
-                   in 2^-28 fixed point, to the element's 64-bit word of the workspace header
-                   with one atomic, and the arrival that completes an element writes it (no
-                   partials in memory; S <= 31, M*N <= 262144; a partial that is not finite
-                   or beyond +-2^20 counts as overflow of its sign).  0 and 1 sum in ascending
-                   order of S in fp32, 2 sums exactly: each is reproducible run to run, the
-                   two families may differ in the last bit                             */
+  int splitk;   /* S >= 1: K is divided over S workgroups per output tile.  S > 1 needs the
+                   workspace; how the S partial sums of an element meet is `fused`.  Every
+                   completion is reproducible run to run (none depends on arrival order)  */
+  int fused;    /* with S > 1, how the split completes:
+                   0 = fp32 partials [S,M,N] go to the workspace and a second kernel sums them;
+                   1 = same partials; the workgroup that finishes a tile last sums them in the
+                       same launch (one counter atomic per workgroup);
+                   2 = every workgroup adds its partial, in 2^-28 fixed point, to the element's
+                       64-bit word of the workspace header with one atomic, and the arrival
+                       that completes an element writes it (S <= 31, M*N <= 262144).  Partials
+                       stay out of memory except those fixed point cannot hold (not finite, or
+                       of magnitude 2^20 and more): these go to their [S,M,N] slot and are
+                       added in fp32, in ascending order of S, when the element completes;
+                   3 = FG_KERNEL_KN_MFMA only, S <= 32: the S workgroups of a tile run on one
+                       XCD and hand their partials over through that XCD's L2, announced by
+                       per-wave flag words in the workspace header that carry a tag unique to
+                       the launch; the workgroup with the last K range sums them.  If the
+                       partners are not on its XCD or stay silent it computes their K ranges
+                       itself (same result, slower);
+                   4 = as 3 with a fifth of the workgroups taking that fallback on purpose (for
+                       tests).
+                   0, 1, 3 and 4 sum in ascending order of S in fp32 and agree bit for bit; 2
+                   sums exactly and may differ from them in the last bit                  */
   int tile_n;   /* output columns per workgroup; FG_KERNEL_NK_MFMA_R takes 16, 32, 48, 64 or,
                    with band = 128, 8 waves and no split, any divisor of N from 17 to 47  */
   int m_block;  /* rows of A per workgroup (grid.y = ceil(M / m_block))               */
@@ -102,10 +113,14 @@ typedef struct fg_plan_t {
  *           S > 1 without workspace is FG_ERR_WORKSPACE.
  *   ws      device scratch of at least fg_workspace_bytes() bytes when the plan's
  *           splitk > 1, else may be NULL.  Its first fg_workspace_header_bytes() bytes (64 KiB of
- *           arrival counters, then 3 MiB of per-element accumulator words) must be zero before
- *           the first call: zero them once with fg_workspace_init() (or allocate zeroed
- *           memory); every call leaves them zero again.  Calls that share a workspace must
- *           be ordered on one stream.
+ *           arrival counters, 3 MiB of per-element accumulator words, 512 KiB of flag words)
+ *           must be zero before the first call (a library older than FG_VERSION 110 had a
+ *           shorter header: size the clear from fg_workspace_header_bytes(), never a
+ *           constant): zero them once with fg_workspace_init() (or allocate zeroed memory).
+ *           Every call leaves counters and accumulator words zero again; flag words keep the
+ *           tag of the launch that wrote them, which no later launch takes for its own.
+ *           Calls that share a workspace must not overlap: order them on one stream, or
+ *           with events.
  * Services, with w_layout = FG_W_KN: edgemm_m8n128k64x4 (backend/cuda/hk/edgemm.cu:102-156),
  * edgemm_m8n128k64x4_amd (:159-213), edgemm_m8n256k32x8 (:363-385, accumulate),
  * flat_gemm_m8n128k64x4_bz1, flat_gemm_m8n256k32x8_bz1, flat_gemm_m8n256k64x8,

@@ -99,7 +99,7 @@ def test_exact_integers_are_exact(device, layout):
 @pytest.mark.parametrize("M", [1, 5, 16])
 def test_special_values_keep_their_class(device, layout, M):
     """NaN / inf in the inputs stay in the outputs they belong to; +inf and -inf from different
-    K ranges meet as NaN; a K-range partial beyond 2^20 counts as overflow of its sign."""
+    K ranges meet as NaN; K-range partials beyond 2^20 of one sign add up to an infinite fp16."""
     K, N = 2048, 256
     g = gen(8300 + M)
     A = normal((M, K), g)
@@ -112,11 +112,7 @@ def test_special_values_keep_their_class(device, layout, M):
     A[:, 2000] = 1.0
     W = Wnk if layout == NK else Wnk.t().contiguous()
     ref, _ = oracle.gemm_f16(A.numpy(), W.numpy(), layout)
-    kern = dict(kernel=capi.FG_KERNEL_KN_MFMA, unroll=1, waves=4) if layout == KN else dict(
-        kernel=capi.FG_KERNEL_NK_MFMA_R, tile_n=16, unroll=1, waves=8)
-    if M == 1:
-        kern = dict(kernel=capi.FG_KERNEL_KN_DOT2, m_block=1, unroll=1, waves=4) if layout == KN else dict(
-            kernel=capi.FG_KERNEL_NK_DOT2, tile_n=4, m_block=1, unroll=1, waves=4)
+    kern = _kernel_for(layout, M)
     for splitk in (2, 4, 8):
         got = _run(A, W, layout, device, make_plan(splitk=splitk, fused=2, **kern))
         assert (np.isnan(got) == np.isnan(ref)).all(), splitk
@@ -135,6 +131,60 @@ def test_special_values_keep_their_class(device, layout, M):
     A2 = -A2
     got = _run(A2, W, layout, device, make_plan(splitk=4, fused=2, **kern))
     assert (got[:, 20] == -np.inf).all()
+
+
+def _kernel_for(layout, M):
+    if M == 1:
+        return dict(kernel=capi.FG_KERNEL_KN_DOT2, m_block=1, unroll=1, waves=4) if layout == KN else dict(
+            kernel=capi.FG_KERNEL_NK_DOT2, tile_n=4, m_block=1, unroll=1, waves=4)
+    return dict(kernel=capi.FG_KERNEL_KN_MFMA, unroll=1, waves=4) if layout == KN else dict(
+        kernel=capi.FG_KERNEL_NK_MFMA_R, tile_n=16, unroll=1, waves=8)
+
+
+@pytest.mark.parametrize("layout", [KN, NK])
+@pytest.mark.parametrize("M", [1, 6, 16])
+def test_huge_partials_of_opposite_sign_cancel(device, layout, M):
+    """K-range partials of 2^21 .. 2^24, too large for the fixed-point word, whose sum is a small
+    finite number: the result is that number, as in every other completion, not inf or NaN.  All
+    values are integers, so every fp32 sum on the way is exact and the comparison is for equality."""
+    K, N = 8192, 256
+    A = torch.full((M, K), 64.0, dtype=torch.half)
+    A[1::2] = 1.0                                  # odd rows: partials of 2^16 .. 2^18, inside the range
+    Wnk = torch.zeros((N, K), dtype=torch.half)
+    q = K // 4
+    cols = torch.arange(N)
+    # columns 0 mod 4: +64 on the first half of K, -64 on the second
+    c0 = cols[cols % 4 == 0]
+    Wnk[c0, : 2 * q] = 64.0
+    Wnk[c0, 2 * q:] = -64.0
+    # columns 1 mod 4: +64, -32, -32 on three quarters, a few ones on the last (a partial inside the range)
+    c1 = cols[cols % 4 == 1]
+    Wnk[c1, :q] = 64.0
+    Wnk[c1, q: 3 * q] = -32.0
+    Wnk[c1, 3 * q + 5: 3 * q + 8] = 1.0
+    # columns 2 mod 4: -64 then +64, and a column-dependent remainder inside the first quarter
+    c2 = cols[cols % 4 == 2]
+    Wnk[c2, : 2 * q] = -64.0
+    Wnk[c2, 2 * q:] = 64.0
+    Wnk[c2, 3] += (c2 % 5).to(torch.half)
+    Wnk[c2, q + 3] += 2.0
+    # columns 3 mod 4: one sign only, the sum leaves the fp16 range
+    c3 = cols[cols % 4 == 3]
+    Wnk[c3, :] = 64.0
+    W = Wnk if layout == NK else Wnk.t().contiguous()
+    ref, _ = oracle.gemm_f16(A.numpy(), W.numpy(), layout)
+    assert np.isfinite(ref[:, c0.numpy()]).all() and np.isinf(ref[0, 3])
+    assert ref[0, 1] == 64.0 * 3 and ref[0, 2] == 64.0 * (2 + 2)
+    kern = _kernel_for(layout, M)
+    for splitk in (2, 4, 8, 16):
+        for fused in (2, 1, 0):
+            got = _run(A, W, layout, device, make_plan(splitk=splitk, fused=fused, **kern))
+            assert (got.view(np.uint16) == ref.view(np.uint16)).all(), (splitk, fused)
+    # on top of C: the old value joins after the cancellation
+    C0 = torch.full((M, N), 3.0, dtype=torch.half)
+    refa, _ = oracle.gemm_f16(A.numpy(), W.numpy(), layout, C=C0.numpy(), accumulate=True)
+    got = _run(A, W, layout, device, make_plan(splitk=4, fused=2, **kern), C0=C0, accumulate=True)
+    assert (got.view(np.uint16) == refa.view(np.uint16)).all()
 
 
 def test_limits_of_the_protocol_are_refused(device):

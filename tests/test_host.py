@@ -33,6 +33,75 @@ def test_header_symbols_are_exported():
     assert capi.lib().fg_version() == 110
 
 
+def test_python_constants_match_the_header():
+    text = HEADER.read_text()
+    m = re.search(r"#define\s+FG_STATIC_SCRATCH_BYTES\s+\(([^\n]*)\)\s*$", text, flags=re.M)
+    assert m and re.fullmatch(r"[0-9 +<()]+", m.group(1))
+    assert eval(m.group(1)) == capi.FG_STATIC_SCRATCH_BYTES       # digits, +, << and brackets only
+    assert capi.FG_STATIC_SCRATCH_BYTES == capi.lib().fg_workspace_header_bytes() + (8 << 20)
+    for name in ("FG_OK", "FG_ERR_INVALID_ARG", "FG_ERR_ALIGN128", "FG_ERR_WORKSPACE", "FG_ERR_LAUNCH",
+                 "FG_ERR_UNSUPPORTED", "FG_ERR_SCRATCH_LIMIT", "FG_W_KN", "FG_W_NK"):
+        m = re.search(r"\b%s\s*=\s*(-?\d+)" % name, text) or re.search(r"#define\s+%s\s+(-?\d+)" % name, text)
+        assert m and int(m.group(1)) == getattr(capi, name), name
+
+
+_PLAN_ONLY = r"""
+import ctypes, os, sys
+def state():
+    fds = set()
+    for f in os.listdir('/proc/self/fd'):
+        try:
+            fds.add(os.readlink('/proc/self/fd/' + f))
+        except OSError:
+            pass
+    maps = {l.split()[-1] for l in open('/proc/self/maps') if '/' in l}
+    threads = len(os.listdir('/proc/self/task'))
+    return fds, maps, threads
+L = ctypes.CDLL(sys.argv[1])
+class Plan(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int) for n in ('kernel', 'splitk', 'fused', 'tile_n', 'm_block', 'waves', 'unroll',
+                'stream_w', 'stagger', 'band', 'grid_x', 'grid_y', 'grid_z', 'block')] + [('workspace_bytes', ctypes.c_size_t)]
+L.fg_plan.argtypes = [ctypes.c_int] * 5 + [ctypes.c_void_p]
+L.fg_workspace_bytes.restype = ctypes.c_size_t
+before = state()
+p = Plan()
+for (M, N, K) in ((1, 4096, 4096), (16, 8192, 8192), (8, 11008, 4096)):
+    for layout in (0, 1):
+        assert L.fg_plan(M, N, K, layout, 0, ctypes.byref(p)) == 0
+        assert L.fg_workspace_bytes(M, N, K, layout, 0) == p.workspace_bytes
+assert L.fg_compute_units() == 256
+L.fg_set_compute_units(304)
+assert L.fg_compute_units() == 304
+assert L.fg_plan(16, 8192, 8192, 0, 0, ctypes.byref(p)) == 0
+after = state()
+new_fds = {f for f in after[0] - before[0] if not f.startswith('/proc/')}
+assert not new_fds, new_fds
+assert not any('kfd' in f or 'renderD' in f for f in after[0]), after[0]
+assert after[1] == before[1], after[1] ^ before[1]
+assert after[2] == before[2], (before[2], after[2])
+print('plan-only process clean')
+"""
+
+
+def _plan_only_process():
+    import sys
+    out = subprocess.run([sys.executable, "-c", _PLAN_ONLY, str(capi.LIB_PATH)], capture_output=True, text=True,
+                         timeout=120)
+    assert out.returncode == 0, out.stdout + out.stderr
+    assert "plan-only process clean" in out.stdout
+
+
+def test_planning_leaves_the_hip_runtime_untouched():
+    """A process that loads the library and only plans and sizes buffers opens no device node,
+    maps no further library and starts no thread: fg_plan and fg_workspace_bytes are host code."""
+    _plan_only_process()
+
+
+@pytest.mark.gpu
+def test_planning_leaves_the_hip_runtime_untouched_with_a_gpu_present():
+    _plan_only_process()
+
+
 def test_header_is_plain_c():
     subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-fsyntax-only", "-x", "c", str(HEADER)], check=True)
 

@@ -79,15 +79,26 @@ def test_static_scratch_unsplit_shapes_and_repeats(device):
         assert torch.equal(got, ref)
 
 
-def test_static_scratch_rejects_plans_beyond_its_limit():
-    # host-only: the size check comes before any device work, so dummy pointers are never touched
-    import ctypes
-    L = capi.lib()
-    M, N, K = 16, 16384, 8192
+def test_static_scratch_limit_from_the_plan():
+    # host-only: the limit follows from the plan's workspace size; no launching entry point is called
+    M, N, K = 16, 16384, 2048
     assert capi.plan(M, N, K, KN, 16).workspace_bytes > capi.FG_STATIC_SCRATCH_BYTES
-    st = L.fg_gemm_f16_static(ctypes.c_void_p(16), ctypes.c_void_p(32), ctypes.c_void_p(48), M, N, K, KN, 0, 16,
-                              None)
-    assert st == capi.FG_ERR_SCRATCH_LIMIT
-    assert "static" in capi.strerror(st)
-    # the library's own plan for the same shape fits
     assert capi.plan(M, N, K, KN).workspace_bytes <= capi.FG_STATIC_SCRATCH_BYTES
+    assert "static" in capi.strerror(capi.FG_ERR_SCRATCH_LIMIT)
+
+
+@pytest.mark.gpu
+def test_static_scratch_rejects_plans_beyond_its_limit(device):
+    L = capi.lib()
+    M, N, K = 16, 16384, 2048
+    A, W = _inputs(M, N, K, KN, 4300, device)
+    C = torch.full((M, N), 7.0, dtype=torch.half, device=device)
+    st = L.fg_gemm_f16_static(h.ptr(A), h.ptr(W), h.ptr(C), M, N, K, KN, 0, 16, h.stream_ptr())
+    assert st == capi.FG_ERR_SCRATCH_LIMIT
+    torch.cuda.synchronize()
+    assert bool((C == 7.0).all())          # refused before any device work
+    # the library's own plan for the same shape fits and runs
+    ref = torch.empty_like(C)
+    h.capi_gemm(A, W, ref, KN)
+    _static(A, W, C, KN)
+    assert torch.equal(C, ref)
