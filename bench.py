@@ -662,7 +662,7 @@ def main() -> int:
         t_i8.append(timed_launches(lambda i: sg.fastgemv_int8(wq[i % (2 * R)], xi, yi, scale=sc)))
     us_i8, us_f16 = sorted(t_i8)[2], sorted(t_f16)[2]
     i8_bytes = K * N + 2 * K + 2 * N + 2 * N
-    int8 = {"op": "fastgemv_int8", "M": 1, "K": K, "N": N, "kernel": "w8a16_m1", "bytes": i8_bytes,
+    int8 = {"op": "fastgemv_int8", "M": 1, "K": K, "N": N, "kernel": "wq_m1<int8>", "bytes": i8_bytes,
             "us_per_call": round(us_i8, 2), "GBps": round(i8_bytes / us_i8 / 1e3, 1),
             "frac_read_ceiling": round(i8_bytes / us_i8 / 1e3 / ceiling_gbps, 4),
             "frac_same_size_read": round(read_us_64 * i8_bytes / (64 << 20) / us_i8, 4),
@@ -716,7 +716,7 @@ def main() -> int:
          "seed": 1004, "bytes": i8_bytes, "us": int8["us_per_call"], "GBps": int8["GBps"],
          "frac_hbm_peak": round(int8["GBps"] / HBM_PEAK_GBPS, 4), "frac_read_ceiling": int8["frac_read_ceiling"],
          "same_size_read_us": round(read_us_64, 2), "frac_same_size_read": int8["frac_same_size_read"],
-         "plan_key": "w8a16_m1|M1"},
+         "plan_key": "wq_m1<int8>|M1"},
     ]
 
     # The roofline entry describes the single-launch call that takes the longest: its time between

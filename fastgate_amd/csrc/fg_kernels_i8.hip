@@ -140,106 +140,131 @@ __global__ __launch_bounds__(512) void w8a16_kernel(const int8_t* __restrict__ W
 }
 
 // ---------------------------------------------------------------------------------------
-// One activation row: the dot products go to the matrix pipe.  v_mfma_f32_4x4x4_16B_f16
-// multiplies, in each block of four lanes, the A rows of the four lanes with the B columns of the
-// four lanes.  With A = the lane's activations and B = the lane's weights, both at the lane's own
-// k positions, the diagonal D[j][j] of a block is lane j's own dot product; the other twelve
-// products are never read.  The memory side is that of w8a16_kernel (lanes along K, 16 weights of
-// RN rows per lane and step); the VALU is left with the int8 -> fp16 conversion alone, 80
-// operations per step instead of 112.  K = N = 8192: 12.4 -> 12.0 us.
+// One activation row (the GEMV proper), int8 and int4 weights.
+//  * Lanes own 8 activations each, not 16 weight bytes: a chunk is UD 16-byte units of x a lane
+//    (unit 64 d + lane, d < UD), so every x load is one contiguous KB per wave, and the weights
+//    under a unit are 8 bytes (int8) or 4 bytes (int4) per row: UD 8- or 4-byte loads a row,
+//    each contiguous over the wave.  With 16 weight bytes a lane, the lane's x is 32 or 64
+//    bytes at that stride from its neighbour's: two or four loads that each touch every cache
+//    line of the wave's span, which cost more than the weight loads themselves.
+//  * The integers reach v_dot2_f32_f16 as fp16 subnormals: a byte or nibble in the low mantissa
+//    bits of a half with a zero exponent field IS that number times 2^-24 (a nibble in bits 4-7:
+//    times 2^-20), exactly.  Kernels keep fp16 subnormals (the compiler's default float mode
+//    for gfx9), products and sums are fp32, and the power of two is put back once per output.
+//    int8: 3 integer operations per 4 weights (sign flip to w + 128, two byte shuffles), the 128
+//    taken out once per output as 128 Σx; int4: 5 per 8 weights (a shift, four masks) and no
+//    constant at all -- against 5 and 7 with a bias to subtract in fp16.
+//  * Waves of a workgroup interleave over the chunks of K; 16-lane sums by DPP, the rest through
+//    LDS in a fixed order.
+// K = N = 8192, one GPU, us per call: int4 9.5 -> 7.6 (a plain read of the 32 MiB: 6.1).  The x
+// loads still cost 0.8 us of that (timed with x replaced by constants), for int8 too: 4 KB of x
+// from L2 per 4 KB of weights from memory, whatever cache policy the weight loads carry; staging x
+// in LDS once per 16-wave workgroup moves the cost into the wait before the first decode.
+// Replaces the device side of gemv_quantized_int8 (backend/cuda/hk/fastgemv.cuh:316-389) and of
+// gemv_quantized_int4 (:394-495, defined there but never launched) for one row.
 // ---------------------------------------------------------------------------------------
-typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
-
-template <int RN, int U, bool FULL>
-__global__ __launch_bounds__(256) void w8a16_m1_kernel(const int8_t* __restrict__ Wq,
-                                                       const half_t* __restrict__ X,
-                                                       const half_t* __restrict__ scale,
-                                                       float scalar_scale, float zero_point,
-                                                       half_t* __restrict__ Y, int N, int K) {
-  __shared__ float red[16][RN];
-  __shared__ float redx[16];
+template <int BITS, int RN, int NWV, int UD>
+__global__ __launch_bounds__(64 * NWV) void wq_m1_kernel(const uint8_t* __restrict__ Wq,
+                                                         const half_t* __restrict__ X,
+                                                         const half_t* __restrict__ scale,
+                                                         float scalar_scale, float zero_point,
+                                                         half_t* __restrict__ Y, int N, int K) {
+  constexpr int WB = BITS == 4 ? 4 : 8;  // weight bytes under one 16-byte unit of x
+  typedef uint32_t wreg_t __attribute__((ext_vector_type(WB / 4)));
+  __shared__ float red[NWV * 4][RN + 1];
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
-  const int nw = blockDim.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: addresses stay scalar
   const int n0 = blockIdx.x * RN;
-  const int nq = K >> 4;  // 16-weight chunks per row
-  const bool use_zp = zero_point != 0.f;
+  const size_t rowb = BITS == 4 ? (size_t)K >> 1 : (size_t)K;
   static_assert(RN <= 64, "one output per thread of the first wave");
   const uint32_t scale_raw = scale_fetch(scale, n0 + (int)threadIdx.x, threadIdx.x < RN);
-
-  float4_t acc[RN];
-  float4_t xsum = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-  for (int r = 0; r < RN; ++r) acc[r] = float4_t{0.f, 0.f, 0.f, 0.f};
-  const int8_t* Wt = Wq + (size_t)n0 * K;
+  // the constant that comes out with Σx: the zero point, and int8's + 128
+  const float zp = BITS == 4 ? zero_point : zero_point + 128.f;
+  const bool use_xsum = zp != 0.f;
+  const uint8_t* Wt = Wq + (size_t)n0 * rowb;  // uniform; the lane's part is a 32-bit offset
+  const uint32_t lane_w = lane * WB, lane_x = lane * 16;
+  const half2_t ones = {static_cast<half_t>(1.f), static_cast<half_t>(1.f)};
   const u32x4 zero = {0u, 0u, 0u, 0u};
-  const half4_t ones = {static_cast<half_t>(1.f), static_cast<half_t>(1.f), static_cast<half_t>(1.f),
-                        static_cast<half_t>(1.f)};
+  float acc0[RN], acc1[RN];
+  float xsum = 0.f;
+#pragma unroll
+  for (int r = 0; r < RN; ++r) acc0[r] = acc1[r] = 0.f;
 
-  const int nsteps = (nq + nw * (64 * U) - 1) / (nw * (64 * U));
-  int step = stagger_start(nsteps, 0);
-  for (int it = 0; it < nsteps; ++it) {
-    const int q0 = (step * nw + wave) * (64 * U);
-    step = step + 1 == nsteps ? 0 : step + 1;
-    u32x4 wr[U][RN];
-    u32x4 xr[U][2];
+  const int nunits = K >> 3;
+  const int nchunks = (nunits + 64 * UD - 1) / (64 * UD);
+  for (int ch = wave; ch < nchunks; ch += NWV) {
+    wreg_t wr[RN][UD];
+    u32x4 xv[UD];
+    bool ok[UD];
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int q = q0 + u * 64 + lane;
-      const bool ok = FULL || q < nq;  // FULL: every step of every wave is inside the row
-      const half_t* xp = X + (size_t)q * 16;
-      xr[u][0] = ok ? load16<false>(xp) : zero;
-      xr[u][1] = ok ? load16<false>(xp + 8) : zero;
+    for (int d = 0; d < UD; ++d) ok[d] = ch * (64 * UD) + 64 * d + lane < nunits;
 #pragma unroll
-      for (int r = 0; r < RN; ++r)
-        wr[u][r] = ok ? load16<true>(Wt + (size_t)r * K + (size_t)q * 16) : zero;
+    for (int r = 0; r < RN; ++r)
+#pragma unroll
+      for (int d = 0; d < UD; ++d) {
+        const wreg_t none = {};
+        wr[r][d] = ok[d] ? __builtin_nontemporal_load(reinterpret_cast<const wreg_t*>(
+                               Wt + (size_t)r * rowb + (size_t)(ch * (64 * UD) + 64 * d) * WB + lane_w))
+                         : none;
+      }
+#pragma unroll
+    for (int d = 0; d < UD; ++d)
+      xv[d] = ok[d] ? load16<false>(reinterpret_cast<const uint8_t*>(X) + (size_t)(ch * (64 * UD) + 64 * d) * 16 + lane_x) : zero;
+    if (use_xsum) {
+#pragma unroll
+      for (int d = 0; d < UD; ++d)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) xsum = __builtin_amdgcn_fdot2(as_half2(xv[d][i]), ones, xsum, false);
+    }
+    if (BITS == 4) {  // (x_j, x_{j+4}): the halves that meet nibbles j and j + 4 of a register
+#pragma unroll
+      for (int d = 0; d < UD; ++d) {
+        const u32x4 t = xv[d];
+        xv[d].x = __builtin_amdgcn_perm(t.z, t.x, 0x05040100u);
+        xv[d].y = __builtin_amdgcn_perm(t.z, t.x, 0x07060302u);
+        xv[d].z = __builtin_amdgcn_perm(t.w, t.y, 0x05040100u);
+        xv[d].w = __builtin_amdgcn_perm(t.w, t.y, 0x07060302u);
+      }
     }
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      half4_t ax[4];  // activations under weight register c: x[4c .. 4c+3]
+    for (int r = 0; r < RN; ++r)
 #pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        const u32x4 xv = xr[u][c >> 1];
-        ax[c] = __builtin_bit_cast(half4_t, (c & 1) ? u32x2{xv.z, xv.w} : u32x2{xv.x, xv.y});
-      }
-      if (use_zp) {
+      for (int d = 0; d < UD; ++d) {
+        if constexpr (BITS == 4) {
+          const uint32_t w = wr[r][d][0], w8 = w >> 8;  // nibbles 0,4 | 1,5 | 2,6 | 3,7
+          acc0[r] = __builtin_amdgcn_fdot2(as_half2(w & 0x000F000Fu), as_half2(xv[d].x), acc0[r], false);
+          acc1[r] = __builtin_amdgcn_fdot2(as_half2(w & 0x00F000F0u), as_half2(xv[d].y), acc1[r], false);
+          acc0[r] = __builtin_amdgcn_fdot2(as_half2(w8 & 0x000F000Fu), as_half2(xv[d].z), acc0[r], false);
+          acc1[r] = __builtin_amdgcn_fdot2(as_half2(w8 & 0x00F000F0u), as_half2(xv[d].w), acc1[r], false);
+        } else {
 #pragma unroll
-        for (int c = 0; c < 4; ++c) xsum = __builtin_amdgcn_mfma_f32_4x4x4f16(ax[c], ones, xsum, 0, 0, 0);
-      }
-#pragma unroll
-      for (int c = 0; c < 4; ++c) {
-#pragma unroll
-        for (int r = 0; r < RN; ++r) {
-          half2_t lo, hi;
-          i8x4_to_half2x2(wr[u][r][c], lo, hi);
-          const half4_t bw = {lo[0], lo[1], hi[0], hi[1]};
-          acc[r] = __builtin_amdgcn_mfma_f32_4x4x4f16(ax[c], bw, acc[r], 0, 0, 0);
+          for (int h = 0; h < 2; ++h) {
+            const uint32_t t = wr[r][d][h] ^ 0x80808080u;  // w + 128 as unsigned bytes
+            const uint32_t b01 = __builtin_amdgcn_perm(0u, t, 0x04010400u);  // halves (b0, b1)
+            const uint32_t b23 = __builtin_amdgcn_perm(0u, t, 0x04030402u);  // halves (b2, b3)
+            acc0[r] = __builtin_amdgcn_fdot2(as_half2(b01), as_half2(xv[d][2 * h]), acc0[r], false);
+            acc1[r] = __builtin_amdgcn_fdot2(as_half2(b23), as_half2(xv[d][2 * h + 1]), acc1[r], false);
+          }
         }
       }
-    }
   }
 
-  // D[i][j] sits in element i of lane j: the diagonal element of this lane's block
-  const bool odd = (lane & 1) != 0, upper = (lane & 2) != 0;
-  auto diag = [&](const float4_t& v) {
-    const float lo = odd ? v[1] : v[0], hi = odd ? v[3] : v[2];
-    return upper ? hi : lo;
-  };
 #pragma unroll
   for (int r = 0; r < RN; ++r) {
-    const float v = row16_allreduce(diag(acc[r]));
+    // int4: acc1 holds the nibbles that sat 4 bits up
+    const float a = BITS == 4 ? acc0[r] * 16777216.f + acc1[r] * 1048576.f : (acc0[r] + acc1[r]) * 16777216.f;
+    const float v = row16_allreduce(a);
     if ((lane & 15) == 0) red[wave * 4 + (lane >> 4)][r] = v;
   }
   {
-    const float xs = row16_allreduce(diag(xsum));
-    if ((lane & 15) == 0) redx[wave * 4 + (lane >> 4)] = xs;
+    const float xs = row16_allreduce(xsum);
+    if ((lane & 15) == 0) red[wave * 4 + (lane >> 4)][RN] = xs;
   }
   __syncthreads();
   if (threadIdx.x < RN) {
-    const int r = threadIdx.x;
-    const float sum = lds_sum<16>(&red[0][r], RN, nw * 4);
-    const float xs = lds_sum<16>(&redx[0], 1, nw * 4);
-    Y[n0 + r] = static_cast<half_t>((sum - zero_point * xs) * (scalar_scale * scale_value(scale_raw)));
+    const float sum = lds_sum<NWV * 4>(&red[0][threadIdx.x], RN + 1, NWV * 4);
+    const float xs = lds_sum<NWV * 4>(&red[0][RN], RN + 1, NWV * 4);
+    Y[n0 + threadIdx.x] = static_cast<half_t>((sum - zp * xs) * (scalar_scale * scale_value(scale_raw)));
   }
 }
 
@@ -316,130 +341,6 @@ __global__ __launch_bounds__(256) void dequant_i32_f16_kernel(const int32_t* __r
     float s = x_scale;
     if (scale != nullptr) s *= static_cast<float>(scale[i % N]);
     y[i] = static_cast<half_t>(static_cast<float>(acc[i]) * s);
-  }
-}
-
-// ---------------------------------------------------------------------------------------
-// w4a16: unsigned 4-bit weights, two per byte, the low nibble first (element 2i in bits 0-3 of
-// byte i, element 2i+1 in bits 4-7: uint4_2 of backend/cuda/hk/utility.cuh:13-36), fp16
-// activations.  A register w of 8 nibbles n0..n7 becomes four half2 with four v_and_or and one
-// shift, by letting the exponent absorb the nibble's position:
-//   (w      & 0x000F000F) | 0x64006400 = (1024 + n0, 1024 + n4)     (w >> 8 likewise: n2, n6)
-//   (w      & 0x00F000F0) | 0x54005400 = (  64 + n1,   64 + n5)     (w >> 8 likewise: n3, n7)
-// The 1024 is subtracted in fp16 (exact); the 64 stays in and is removed once per output as
-// 64·Σ x over the odd positions, which costs two v_dot2 per 8 activations shared by all rows
-// (products of at most 79·|x| instead of 15·|x| in the fp32 sum: two bits of headroom, not ten).
-// The activations are paired the same way, (x_j, x_{j+4}), once per chunk.
-// Replaces gemv_quantized_int4 (backend/cuda/hk/fastgemv.cuh:394-495), which the reference
-// defines but never launches.  Lanes along K: one 16-byte load = 32 weights of one row.
-// Launched for one activation row; two to four rows take w4a16_r_kernel below.
-// ---------------------------------------------------------------------------------------
-template <int MB, int RN>
-__global__ __launch_bounds__(256) void w4a16_kernel(const uint8_t* __restrict__ Wq,
-                                                    const half_t* __restrict__ X,
-                                                    const half_t* __restrict__ scale,
-                                                    float scalar_scale, float zero_point,
-                                                    half_t* __restrict__ Y, int M, int N, int K) {
-  __shared__ float red[16][RN * MB];
-  __shared__ float redx[16][MB];
-  __shared__ float redo[16][MB];
-  const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
-  const int nw = blockDim.x >> 6;
-  const int n0 = blockIdx.x * RN;
-  const int nq = K >> 5;        // 32-weight chunks per row
-  const size_t rowb = (size_t)K >> 1;  // bytes per weight row
-  const bool use_zp = zero_point != 0.f;
-  // scale of the output this thread writes at the end, fetched ahead of the weight stream
-  static_assert(RN * MB <= 64, "one output per thread of the first wave");
-  const uint32_t scale_raw = scale_fetch(scale, n0 + (int)threadIdx.x % RN, threadIdx.x < RN * MB);
-
-  float acc[RN][MB];
-  float xsum[MB], xodd[MB];
-#pragma unroll
-  for (int m = 0; m < MB; ++m) {
-    xsum[m] = 0.f;
-    xodd[m] = 0.f;
-#pragma unroll
-    for (int r = 0; r < RN; ++r) acc[r][m] = 0.f;
-  }
-  const uint8_t* Wt = Wq + (size_t)n0 * rowb;
-  const u32x4 zero = {0u, 0u, 0u, 0u};
-  const half2_t ones = {static_cast<half_t>(1.f), static_cast<half_t>(1.f)};
-  const half2_t bias = {static_cast<half_t>(1024.f), static_cast<half_t>(1024.f)};
-
-  const int nsteps = (nq + nw * 64 - 1) / (nw * 64);
-  int step = stagger_start(nsteps, 0);
-  for (int it = 0; it < nsteps; ++it) {
-    const int q = (step * nw + wave) * 64 + lane;
-    step = step + 1 == nsteps ? 0 : step + 1;
-    const bool ok = q < nq;
-    u32x4 wr[RN];
-#pragma unroll
-    for (int r = 0; r < RN; ++r) wr[r] = ok ? load16<true>(Wt + (size_t)r * rowb + (size_t)q * 16) : zero;
-    // xp[m][d][j] = (x[8d + j], x[8d + j + 4]) for the 8 activations under weight register d
-    uint32_t xp[MB][4][4];
-#pragma unroll
-    for (int m = 0; m < MB; ++m) {
-      const bool okm = ok && m < M;
-      const half_t* xptr = X + (size_t)m * K + (size_t)q * 32;
-#pragma unroll
-      for (int d = 0; d < 4; ++d) {
-        const u32x4 xv = okm ? load16<false>(xptr + 8 * d) : zero;  // x[8d .. 8d+7]
-        xp[m][d][0] = __builtin_amdgcn_perm(xv.z, xv.x, 0x05040100u);  // (x0, x4)
-        xp[m][d][1] = __builtin_amdgcn_perm(xv.z, xv.x, 0x07060302u);  // (x1, x5)
-        xp[m][d][2] = __builtin_amdgcn_perm(xv.w, xv.y, 0x05040100u);  // (x2, x6)
-        xp[m][d][3] = __builtin_amdgcn_perm(xv.w, xv.y, 0x07060302u);  // (x3, x7)
-        xodd[m] = __builtin_amdgcn_fdot2(as_half2(xp[m][d][1]), ones, xodd[m], false);
-        xodd[m] = __builtin_amdgcn_fdot2(as_half2(xp[m][d][3]), ones, xodd[m], false);
-        if (use_zp) {
-          xsum[m] = __builtin_amdgcn_fdot2(as_half2(xp[m][d][0]), ones, xsum[m], false);
-          xsum[m] = __builtin_amdgcn_fdot2(as_half2(xp[m][d][2]), ones, xsum[m], false);
-        }
-      }
-    }
-#pragma unroll
-    for (int r = 0; r < RN; ++r)
-#pragma unroll
-      for (int d = 0; d < 4; ++d) {
-        const uint32_t w = wr[r][d], w8 = w >> 8;
-        const half2_t wv[4] = {as_half2((w & 0x000F000Fu) | 0x64006400u) - bias,
-                               as_half2((w & 0x00F000F0u) | 0x54005400u),
-                               as_half2((w8 & 0x000F000Fu) | 0x64006400u) - bias,
-                               as_half2((w8 & 0x00F000F0u) | 0x54005400u)};
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-          for (int m = 0; m < MB; ++m)
-            acc[r][m] = __builtin_amdgcn_fdot2(wv[j], as_half2(xp[m][d][j]), acc[r][m], false);
-      }
-  }
-
-  // xsum holds Σ x over the even positions (only when a zero point needs it), xodd over the odd
-#pragma unroll
-  for (int m = 0; m < MB; ++m) {
-#pragma unroll
-    for (int r = 0; r < RN; ++r) {
-      const float v = row16_allreduce(acc[r][m]);
-      if ((lane & 15) == 0) red[wave * 4 + (lane >> 4)][r * MB + m] = v;
-    }
-    const float xe = row16_allreduce(xsum[m]);
-    const float xo = row16_allreduce(xodd[m]);
-    if ((lane & 15) == 0) {
-      redx[wave * 4 + (lane >> 4)][m] = xe;
-      redo[wave * 4 + (lane >> 4)][m] = xo;
-    }
-  }
-  __syncthreads();
-  for (int t = threadIdx.x; t < RN * MB; t += blockDim.x) {
-    const int m = t / RN, r = t % RN;
-    const float sum = lds_sum<16>(&red[0][r * MB + m], RN * MB, nw * 4);
-    const float xe = lds_sum<16>(&redx[0][m], MB, nw * 4);
-    const float xo = lds_sum<16>(&redo[0][m], MB, nw * 4);
-    const int n = n0 + r;
-    if (m < M)
-      Y[(size_t)m * N + n] = static_cast<half_t>((sum - 64.f * xo - zero_point * (xe + xo)) *
-                                                 (scalar_scale * scale_value(scale_raw)));
   }
 }
 
@@ -716,6 +617,36 @@ static int i8_waves(int K) {
   return pieces >= 4 ? 4 : (pieces >= 2 ? 2 : 1);
 }
 
+// One activation row.  A wave's chunk is 1 KB of each weight row (2048 k of int4 in four units a
+// lane, 1024 k of int8 in two); a workgroup has as many waves as K has chunks, up to 8, rounded up
+// to a power of two, and takes four weight rows -- two when the whole matrix is 8 MiB or less,
+// where four rows leave too few workgroups.  Measured, us per call, previous kernels -> these
+// (N x K): int4 8192 x 8192 10.6 -> 8.7, 4096 x 4096 5.7 -> 4.1, 28672 x 4096 16.2 -> 11.6,
+// 4096 x 14336 10.1 -> 8.1, 16384 x 16384 27.9 -> 24.5; int8 8192 x 8192 13.3 -> 12.1,
+// 4096 x 4096 5.7 -> 5.25, 28672 x 4096 20.8 -> 18.8, 4096 x 14336 12.6 -> 11.4, 16384 x 16384
+// 41.9 -> 40.6.  int8 with four units a lane (2 KB of a row per wave): 8192 x 8192 13.0.
+template <int BITS>
+static void launch_wq_m1(const W8A16Args& a, hipStream_t s) {
+  auto* Wq = static_cast<const uint8_t*>(a.Wq);
+  auto* X = static_cast<const half_t*>(a.x);
+  auto* sc = static_cast<const half_t*>(a.scale);
+  auto* Y = static_cast<half_t*>(a.y);
+  constexpr int UD = BITS == 4 ? 4 : 2;
+  const int chunks = (a.K + 512 * UD - 1) / (512 * UD);
+  const bool small = (size_t)a.N * a.K * BITS / 8 <= (8u << 20);
+#define FG_WQ_M1(RN, NWV)                                                                     \
+  hipLaunchKernelGGL((wq_m1_kernel<BITS, RN, NWV, UD>), dim3(a.N / RN), dim3(64 * NWV), 0, s, Wq, \
+                     X, sc, a.scalar_scale, a.zero_point, Y, a.N, a.K)
+#define FG_WQ_M1_ROWS(NWV) \
+  if (small) FG_WQ_M1(2, NWV); else FG_WQ_M1(4, NWV)
+  if (chunks > 4) { FG_WQ_M1_ROWS(8); }
+  else if (chunks > 2) { FG_WQ_M1_ROWS(4); }
+  else if (chunks > 1) { FG_WQ_M1_ROWS(2); }
+  else { FG_WQ_M1_ROWS(1); }
+#undef FG_WQ_M1_ROWS
+#undef FG_WQ_M1
+}
+
 // Measured (us per call; lanes-along-K kernel / row-load kernel on 256-byte bands):
 //   K = N = 8192   M=1 12.6 / 14.3   M=2 15.1 / 14.2   M=4 21.1 / 14.9   M=8 32.9 / 17.2
 //   K = N = 16384  M=1 41.2 / 44.8   M=8  -   / 49.7
@@ -749,14 +680,8 @@ bool launch_w8a16(const W8A16Args& a, hipStream_t s) {
 #define FG_W8A16_R(XR, BW, CB)                                                                    \
   hipLaunchKernelGGL((w8a16_r_kernel<XR, 8, BW, CB>), dim3(a.N / (16 * CB)), dim3(512), 0, s, Wq, \
                      X, sc, a.scalar_scale, a.zero_point, Y, a.M, a.N, a.K)
-  if (a.M == 1) {  // 4 rows per workgroup, one load group in flight
-    const int nw = i8_waves(a.K);
-    if ((a.K / 16) % (64 * nw) == 0)
-      hipLaunchKernelGGL((w8a16_m1_kernel<4, 1, true>), dim3(a.N / 4), dim3(64 * nw), 0, s, Wq, X, sc,
-                         a.scalar_scale, a.zero_point, Y, a.N, a.K);
-    else
-      hipLaunchKernelGGL((w8a16_m1_kernel<4, 1, false>), dim3(a.N / 4), dim3(64 * nw), 0, s, Wq, X, sc,
-                         a.scalar_scale, a.zero_point, Y, a.N, a.K);
+  if (a.M == 1) {
+    launch_wq_m1<8>(a, s);
   } else if (a.M <= 4 && (a.N <= 2048 || (a.M == 2 && a.N <= 6144))) {
     // narrow outputs leave the 16-column tiles of the row-load kernel on half the CUs or fewer: lanes
     // along K, four weight rows a workgroup (N=2048 K=8192: M=2 8.8 -> 6.0 us, M=4 9.0 -> 7.3;
@@ -794,17 +719,7 @@ bool launch_w4a16(const W8A16Args& a, hipStream_t s) {
   auto* Y = static_cast<half_t*>(a.y);
   if (a.M < 1 || a.M > 4) return false;
   if (a.M == 1) {
-    // one activation row: the dot2 kernel's straight 1 KB row pieces are the shorter path
-    const int pieces = (a.K / 32 + 63) / 64;  // 1 KB pieces per weight row
-    const dim3 block(64 * (pieces >= 4 ? 4 : (pieces >= 2 ? 2 : 1)));
-    // rows longer than 4 KB: eight rows a workgroup share each activation piece (K = N = 16384
-    // 29.9 -> 26.6 us, N=4096 K=14336 10.5 -> 9.5; K = N = 8192 10.15 -> 10.24 the other way)
-    if (a.K > 8192 && a.N % 8 == 0)
-      hipLaunchKernelGGL((w4a16_kernel<1, 8>), dim3(a.N / 8), block, 0, s, Wq, X, sc, a.scalar_scale,
-                         a.zero_point, Y, a.M, a.N, a.K);
-    else
-      hipLaunchKernelGGL((w4a16_kernel<1, 4>), dim3(a.N / 4), block, 0, s, Wq, X, sc, a.scalar_scale,
-                         a.zero_point, Y, a.M, a.N, a.K);
+    launch_wq_m1<4>(a, s);
   } else if (a.M == 2) {
     hipLaunchKernelGGL((w4a16_r_kernel<2>), dim3(a.N / 16), dim3(512), 0, s, Wq, X, sc, a.scalar_scale,
                        a.zero_point, Y, a.M, a.N, a.K);

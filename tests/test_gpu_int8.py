@@ -335,3 +335,49 @@ def test_w4a16_golden_vectors(device):
     assert_close_f16(_w4a16(Wq4, x, None, 1.0, 8.0, device), want, "golden int4, M=2")
     for m in range(2):
         assert_close_f16(_w4a16(Wq4, x[m:m + 1].contiguous(), None, 1.0, 8.0, device), want[m:m + 1], "golden int4 row %d" % m)
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("N,K", [(128, 128), (128, 1152), (256, 2176), (128, 4224), (128, 9344)])
+def test_one_row_kernels_pick_every_position_exactly(device, bits, N, K):
+    """One activation row, x = 2^e at a single k: the output column is that weight times 2^e,
+    exactly, for positions across every unit, chunk and wave of the row (a full chunk is 1024 k
+    of int8 or 2048 k of int4; these K end inside a chunk) and for activations down in the fp16
+    subnormal range, where the weights themselves travel as subnormals."""
+    g = gen(6100 + bits + K)
+    if bits == 8:
+        W = torch.randint(-128, 128, (N, K), generator=g, dtype=torch.int8)
+        want = W.numpy().astype(np.float32)
+        run = _w8a16
+    else:
+        W = torch.randint(0, 256, (N, K // 2), generator=g, dtype=torch.uint8)
+        want = np.empty((N, K), np.float32)
+        want[:, 0::2] = (W & 0x0F).numpy()
+        want[:, 1::2] = (W >> 4).numpy()
+        run = _w4a16
+    ks = sorted(set(list(range(0, 40)) + list(range(K - 40, K)) + list(range(5, K, 263)) +
+                    [k for c in range(512, K, 512) for k in (c - 1, c)]))
+    for i, k in enumerate(ks):
+        e = (0, -3, -14, -17, -24)[i % 5]            # 2^-17 and 2^-24 are fp16 subnormals
+        x = torch.zeros((1, K), dtype=torch.half)
+        x[0, k] = 2.0 ** e
+        got = run(W, x, None, 1.0, 0.0, device).astype(np.float64)
+        expect = (want[:, k].astype(np.float64) * 2.0 ** e).astype(np.float16).astype(np.float64)
+        assert (got[0] == expect).all(), (k, e)
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_one_row_kernels_small_integers_and_zero_point_are_exact(device, bits):
+    g = gen(6200 + bits)
+    for (N, K) in ((256, 2048), (128, 3200), (512, 8192), (128, 20480)):
+        x = torch.randint(-3, 4, (1, K), generator=g).half()
+        if bits == 8:
+            W = torch.randint(-128, 128, (N, K), generator=g, dtype=torch.int8)
+            ref, _ = oracle.gemv_w8a16(W.numpy(), x.numpy(), None, 1.0, 3.0)
+            got = _w8a16(W, x, None, 1.0, 3.0, device)
+        else:
+            W = torch.randint(0, 256, (N, K // 2), generator=g, dtype=torch.uint8)
+            ref, _ = oracle.gemv_w4a16(W.numpy(), x.numpy(), None, 1.0, 8.0)
+            got = _w4a16(W, x, None, 1.0, 8.0, device)
+        # every fp32 sum on the way is an integer below 2^24: the one rounding to fp16 decides
+        assert (got.view(np.uint16) == ref.view(np.uint16)).all(), (N, K)
