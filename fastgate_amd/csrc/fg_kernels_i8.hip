@@ -387,7 +387,6 @@ __global__ __launch_bounds__(64 * NW) void w8a16_r_kernel(const int8_t* __restri
   const int hx = lane / LPX, cx = lane % LPX;      // activation load order: row RPX*i + hx, piece cx
   const int n0 = blockIdx.x * (16 * CB);
   const int nbands = (K + BW - 1) / BW;            // K % 128 == 0: the last band may be partial
-  const bool use_zp = zero_point != 0.f;
   // scale of the output this thread writes at the end, fetched ahead of the weight stream
   static_assert(16 * 16 * CB <= 64 * NW, "one output per thread");
   const uint32_t scale_raw =
@@ -434,13 +433,14 @@ __global__ __launch_bounds__(64 * NW) void w8a16_r_kernel(const int8_t* __restri
 #pragma unroll
       for (int b = 0; b < CB; ++b) {
         const u32x2 wv = *reinterpret_cast<const u32x2*>(wstrip + b * 16 * RSW + ldw_off + u * 32);
-        half2_t h0, h1, h2, h3;
-        i8x4_to_half2x2(wv.x, h0, h1);
-        i8x4_to_half2x2(wv.y, h2, h3);
-        const half8_t wb = {h0[0], h0[1], h1[0], h1[1], h2[0], h2[1], h3[0], h3[1]};
-        acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(xv), wb, acc[b], 0, 0, 0);
+        // bytes as fp16 subnormals: (w + 128) 2^-24, two integer operations fewer per register than
+        // building normal numbers and subtracting their bias; the 128 leaves with the zero point
+        const uint32_t t0 = wv.x ^ 0x80808080u, t1 = wv.y ^ 0x80808080u;
+        const u32x4 wb = {__builtin_amdgcn_perm(0u, t0, 0x04010400u), __builtin_amdgcn_perm(0u, t0, 0x04030402u),
+                          __builtin_amdgcn_perm(0u, t1, 0x04010400u), __builtin_amdgcn_perm(0u, t1, 0x04030402u)};
+        acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(xv), as_half8(wb), acc[b], 0, 0, 0);
       }
-      if (use_zp) xacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(xv), ones8, xacc, 0, 0, 0);
+      xacc = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(xv), ones8, xacc, 0, 0, 0);
     }
     wave_lds_sync();
   };
@@ -479,8 +479,8 @@ __global__ __launch_bounds__(64 * NW) void w8a16_r_kernel(const int8_t* __restri
     if (m < M) {
       const float sum = lds_sum<NW>(&red[0][0][e], 2 * 16 * TN, nw);
       const float xs = lds_sum<NW>(&red[0][1][m * 16 + (e & 15)], 2 * 16 * TN, nw);
-      Y[(size_t)m * N + n] =
-          static_cast<half_t>((sum - zero_point * xs) * (scalar_scale * scale_value(scale_raw)));
+      Y[(size_t)m * N + n] = static_cast<half_t>((sum * 16777216.f - (zero_point + 128.f) * xs) *
+                                                 (scalar_scale * scale_value(scale_raw)));
     }
   }
 }
