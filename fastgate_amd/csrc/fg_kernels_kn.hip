@@ -59,10 +59,13 @@ __device__ __forceinline__ int kn_tile(int x, int z, int gx, int cus) {
 // Work items (column tile, K split z, row block y) come from a one-dimensional grid:
 //  * plain order: x fastest, every z plane shifted by the rounds of CUs dispatched before it
 //    (kn_tile's rule);
-//  * XCD-local order (kFlagXcdLocal): workgroups go to the XCDs round-robin by their linear id, so
-//    id % xccs names the XCD a workgroup runs on.  Every XCD is handed a contiguous run of column
-//    tiles and all S workgroups of a tile get ids that are equal modulo xccs, z ascending with the
-//    id: the partners of a tile share one L2 and one dispatch queue.
+//  * XCD-local order (kFlagXcdLocal): the hardware deals the workgroups of a launch to the XCDs
+//    round-robin in the order of their linear ids, starting at an XCD that depends on what was
+//    launched before (measured: XCC id == (id + c) % xccs for every workgroup of a launch, c
+//    constant within it and changing between launches, also between the nodes of a graph).  Ids
+//    that are equal modulo xccs therefore share an XCD whatever c is.  Every residue class is
+//    handed a contiguous run of column tiles and all S workgroups of a tile get ids of that
+//    class, z ascending with the id: the partners of a tile share one L2 and one dispatch queue.
 //
 // Split-K completion in XCD-local order ("mailbox").  The partners exchange their partials with
 // ordinary stores and loads that stay in the XCD's L2 (acknowledged by the L2, not by memory) and
@@ -73,18 +76,19 @@ __device__ __forceinline__ int kn_tile(int x, int z, int gx, int cus) {
 //                       (S - 1) x waves flags of the tile (L1-bypassing loads served by the L2),
 //                       then every thread adds the partials in ascending z, its own last, and
 //                       writes C.
-// The tag names the launch: a number the host counts up with every enqueue, the queue the
-// dispatch packet sits in and the packet's index in that queue (which also tells apart the
-// replays of a captured graph, whose kernel arguments never change).  Flags left behind by
-// earlier launches never match, so nothing has to be cleared and nothing is read or counted
-// when a workgroup starts.
-// Nothing depends on where the hardware really puts a workgroup.  Every workgroup compares the XCC id
-// register with id % xccs: a partner on another XCD does nothing (its stores would land in an L2
-// the owner cannot see), an owner on another XCD does not poll.  The owner polls a bounded
-// number of times -- partners are dispatched before it from the same queue, so their flags come
-// within microseconds -- and recomputes from A and W every partial it has no flag for, in the
-// same order of operations: the result is bit for bit the same, only later.  kFlagPretendForeign
-// makes a fifth of the workgroups claim to be misplaced (tests).
+// The tag names the launch and the XCD: a number the host counts up with every enqueue, the XCC id
+// of the wave that writes or expects the flag, the queue the dispatch packet sits in and the
+// packet's index in that queue (which also tells apart the replays of a captured graph, whose
+// kernel arguments never change).  Flags left behind by earlier launches never match, so nothing
+// has to be cleared and nothing is read or counted when a workgroup starts.
+// Nothing depends on where the hardware really puts a workgroup.  A flag counts only when it
+// carries the owner's own XCC id: a partner that ran on another XCD (its stores are in an L2 the
+// owner cannot see) is never taken for delivered, and a flag of this launch from another XCD ends
+// the wait at once.  The owner polls a bounded number of times -- partners are dispatched before it
+// from the same queue, so their flags come within microseconds -- and recomputes from A and W
+// every partial it has no flag for, in the same order of operations: the result is bit for bit
+// the same, only later.  kFlagPretendForeign makes a fifth of the workgroups behave as if they
+// were misplaced (tests): such a partner stores nothing, such an owner does not poll.
 // ---------------------------------------------------------------------------------------
 constexpr int kRedStride = 132;  // floats per row of the cross-wave buffer: 128 + 4 keeps 16-byte
                                  // alignment and puts consecutive rows on different LDS banks
@@ -97,16 +101,22 @@ __device__ __forceinline__ int xcc_id() {
 // AQL dispatch packet index of this launch in its queue (64-bit, counts up with every packet).
 extern "C" __device__ unsigned long long fg_dispatch_id(void) __asm("llvm.amdgcn.dispatch.id");
 
-// 64-bit name of this launch, never zero: host enqueue count (24 bits, 1..2^24-1) | queue (8 bits of
-// the queue descriptor's address) | low 32 bits of the packet index.
+// 64-bit name of this launch on this XCD, never zero: host enqueue count (20 bits, 1..2^20-1) | XCC id
+// (4 bits) | queue (8 bits of the queue descriptor's address) | low 32 bits of the packet index.
+constexpr unsigned long long kTagXccMask = 0xFull << 40;
 __device__ __forceinline__ unsigned long long launch_tag(unsigned int nonce) {
   const unsigned long long q = reinterpret_cast<unsigned long long>(__builtin_amdgcn_queue_ptr());
-  return ((unsigned long long)nonce << 40) | (((q >> 12) & 0xFFull) << 32) | (fg_dispatch_id() & 0xFFFFFFFFull);
+  return ((unsigned long long)nonce << 44) | ((unsigned long long)xcc_id() << 40) | (((q >> 12) & 0xFFull) << 32) |
+         (fg_dispatch_id() & 0xFFFFFFFFull);
+}
+// A flag word of this launch written on another XCD.
+__device__ __forceinline__ bool tag_is_foreign(unsigned long long flag, unsigned long long tag) {
+  return flag != tag && ((flag ^ tag) & ~kTagXccMask) == 0;
 }
 
 struct KnItem {
   int tile, z, y;
-  bool home;  // runs on the XCD its tile's partials live in (always true in plain order)
+  bool home;  // false: behaves as if it ran on another XCD than its partners (tests only)
 };
 // x / d and x % d for a divisor whose log2 the host passes when it is a power of two (-1 otherwise):
 // the usual tile, XCD and CU counts are, and a division by a run-time value costs some 40
@@ -131,8 +141,7 @@ __device__ __forceinline__ KnItem kn_item(int M, int flags, const KnGeo& geo) {
     it.z = div_by(n, geo.tq, geo.log2_tq);
     const int round = div_by(L - xcd - a * geo.xccs, geo.cus, geo.log2_cus);  // full rounds of CUs before this plane
     it.tile = xcd * geo.tq + mod_by(a + round, geo.tq, geo.log2_tq);           // >= tiles: nothing to do
-    it.home = geo.xccs == 1 || xcc_id() == xcd;
-    if (flags & kFlagPretendForeign) it.home = it.home && (L % 5 != 3);
+    if (flags & kFlagPretendForeign) it.home = L % 5 != 3;
   } else {
     const int x = mod_by(l, geo.tiles, geo.log2_tiles);
     it.z = div_by(l, geo.tiles, geo.log2_tiles);
@@ -369,7 +378,8 @@ __global__ __launch_bounds__(64 * NW, (NW == 8 && U == 1) ? 4 : 1) void kn_mfma_
   // partner takes that memory latency off the end of the kernel.  The values wait in registers and
   // are added in ascending z afterwards.  The waves do not meet at a barrier, so they agree through
   // one LDS word on whether anybody gives up: 0 undecided, 1 some wave has seen every flag (then
-  // every wave will), 2 wave 0 has polled `spin_limit` times in vain (everybody recomputes).
+  // every wave will), 2 wave 0 has polled `spin_limit` times in vain or some wave has found a flag of
+  // this launch from another XCD (everybody recomputes).
   constexpr int PF = 8;
   const unsigned int all = (1u << (S - 1)) - 1u;  // S <= 32
   if (it.home && S - 1 <= PF && (S - 1) * NW <= 64) {
@@ -383,9 +393,10 @@ __global__ __launch_bounds__(64 * NW, (NW == 8 && U == 1) ? 4 : 1) void kn_mfma_
     unsigned int loaded = 0;
     bool give_up = false;
     for (int spins = 0;; ++spins) {
-      const bool ok = lane >= nflags ||
-                      __hip_atomic_load(mb_flags + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == tag;
-      const unsigned long long b = __builtin_amdgcn_ballot_w64(ok);
+      const unsigned long long f =
+          lane < nflags ? __hip_atomic_load(mb_flags + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : tag;
+      const unsigned long long b = __builtin_amdgcn_ballot_w64(f == tag);
+      const bool misplaced = __builtin_amdgcn_ballot_w64(tag_is_foreign(f, tag)) != 0;  // a partner on another XCD
 #pragma unroll
       for (int z = 0; z < PF; ++z) {
         const unsigned long long lanes = ((1ull << NW) - 1) << (z * NW);
@@ -401,7 +412,7 @@ __global__ __launch_bounds__(64 * NW, (NW == 8 && U == 1) ? 4 : 1) void kn_mfma_
         give_up = true;
         break;
       }
-      if (wave == 0 && spins >= geo.spin_limit) {
+      if (misplaced || (wave == 0 && spins >= geo.spin_limit)) {
         int seen = 0;
         if (lane == 0) {
           __hip_atomic_compare_exchange_strong(&s_state, &seen, 2, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
@@ -448,16 +459,17 @@ __global__ __launch_bounds__(64 * NW, (NW == 8 && U == 1) ? 4 : 1) void kn_mfma_
     if (wave == 0) {
       unsigned int ready = 0;  // bit z: all waves of partner z have flagged
       if (it.home) {
-        bool done = false;
-        for (int spins = 0; !done && spins < geo.spin_limit; ++spins) {
+        bool done = false, misplaced = false;
+        for (int spins = 0; !done && !misplaced && spins < geo.spin_limit; ++spins) {
           done = true;
           for (int base = 0; base < nflags; base += 64) {
             const int idx = base + lane;
-            const bool ok = idx >= nflags ||
-                            __hip_atomic_load(mb_flags + idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == tag;
-            done = done && __builtin_amdgcn_ballot_w64(ok) == ~0ull;
+            const unsigned long long f =
+                idx < nflags ? __hip_atomic_load(mb_flags + idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : tag;
+            done = done && __builtin_amdgcn_ballot_w64(f == tag) == ~0ull;
+            misplaced = misplaced || __builtin_amdgcn_ballot_w64(tag_is_foreign(f, tag)) != 0;
           }
-          if (!done) __builtin_amdgcn_s_sleep(1);
+          if (!done && !misplaced) __builtin_amdgcn_s_sleep(1);
         }
         if (done) {
           ready = all;
@@ -680,10 +692,10 @@ static void kn_mfma_go(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
     return l;
   };
   geo.log2_tiles = log2_of(geo.tiles), geo.log2_tq = log2_of(geo.tq), geo.log2_xccs = log2_of(geo.xccs), geo.log2_cus = log2_of(geo.cus);
-  geo.spin_limit = (a.accumulate & kFlagPretendForeign) ? 64 : (1 << 18);
+  geo.spin_limit = (a.accumulate & kFlagPretendForeign) ? 64 : (1 << 14);  // some 10 ms of polling
   // a new number for every enqueue of a launch that uses the flags (1 .. 2^24 - 1, wrapping)
   static std::atomic<unsigned int> enqueues{0};
-  geo.nonce = (a.accumulate & kFlagXcdLocal) ? enqueues.fetch_add(1, std::memory_order_relaxed) % 0xFFFFFFu + 1u : 0u;
+  geo.nonce = (a.accumulate & kFlagXcdLocal) ? enqueues.fetch_add(1, std::memory_order_relaxed) % 0xFFFFFu + 1u : 0u;
 #ifdef FG_PROBE
   { const char* e = getenv("FG_PROBE"); geo.probe = e ? atoi(e) : 0; }
 #endif

@@ -153,3 +153,45 @@ def test_mailbox_limits(device):
     st = L.fg_gemm_f16_planned(ptr(A), ptr(W), ptr(C), 4, 256, 4096, KN, 0, ctypes.byref(p), ptr(ws), ws.numel(), stream_ptr())
     assert st == capi.FG_ERR_INVALID_ARG
     torch.cuda.synchronize()
+
+
+def test_mailbox_fast_path_whatever_xcd_the_dispatch_starts_on(device):
+    """The XCD that workgroup 0 of a launch lands on depends on what ran before.  The partners of
+    a tile must still find each other: after launches of assorted grid sizes the mailbox call may
+    not fall back to recomputing its partners' K ranges, which costs several times the call.  The
+    bound is loose (2.5x the counter completion; the fallback measured 4x) and results are checked
+    bit for bit as well."""
+    L = capi.lib()
+    ws = _workspace(device)
+    g = gen(9400)
+    M, N, K, S = 16, 4096, 4096, 8
+    Ad, Wd = normal((M, K), g).to(device), normal((K, N), g, 0.05).to(device)
+    C1 = torch.zeros((M, N), dtype=torch.half, device=device)
+    C3 = torch.zeros_like(C1)
+    Ks = 1024
+    As = normal((4, Ks), g).to(device)
+
+    def shift(tiles, split):
+        # a [K,N] call of tiles x split workgroups in plain order moves the starting XCD of what follows
+        Ws = torch.zeros((Ks, 128 * tiles), dtype=torch.half, device=device)
+        Cs = torch.zeros((4, 128 * tiles), dtype=torch.half, device=device)
+        _call(As, Ws, Cs, make_plan(capi.FG_KERNEL_KN_DOT2, m_block=4, waves=4, splitk=split, fused=1 if split > 1 else 0), ws)
+
+    def timed(plan, C, reps=30):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            _call(Ad, Wd, C, plan, ws)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / reps
+
+    for tiles, split in ((1, 1), (1, 3), (1, 5), (1, 7), (43, 2), (37, 7), (129, 4), (17, 13), (3, 3)):
+        shift(tiles, split)
+        timed(_plan(S, 1), C1, 5)
+        shift(tiles, split)
+        t3 = timed(_plan(S, 3), C3)
+        shift(tiles, split)
+        t1 = timed(_plan(S, 1), C1)
+        assert (_bits(C1) == _bits(C3)).all(), (tiles, split)
+        assert t3 < 2.5 * t1, (tiles, split, t3, t1)
