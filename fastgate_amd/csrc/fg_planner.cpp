@@ -629,6 +629,53 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
       if (finish_plan(M, N, K, &q) == FG_OK && q.fused == 3) *p = q;
     }
   }
+  // Small problems (4 Mi weights or fewer, up to 16 rows).  Their kernels last 3 .. 7 us, a handful
+  // of dependent memory round trips, and what shortens them is more, shorter waves, each with one
+  // or two loads to wait for.  Fitted to per-launch times inside a replayed graph of 64 launches
+  // (no host launch rate in the figure) over N x K in {512 .. 4096}^2, about 150 plans a cell
+  // (us, this rule / the plan it replaces):
+  //  * [K,N]: the v_dot2 kernel on two rows a workgroup, four waves, one 32-row unit a wave (K / 128
+  //    splits, 16 at most), completed by atomics: 1024 x 1024 M=1 3.8 / 4.5, M=8 4.2 / 5.6, M=16
+  //    4.8 / 6.1; N=1024 K=2048 M=8 4.9 / 5.8; N=2048 K=1024 M=8 4.9 / 5.8; N=2048 K=512 M=16 4.8 /
+  //    6.1.  Beyond 2 Mi weights only up to four rows (2048 x 2048 M=4 5.2 / 5.8, N=4096 K=1024 M=2
+  //    4.8 / 5.4), beyond 1 Mi up to eight; nine rows and more (eight from 4096 columns) then take
+  //    the MFMA kernel with the flag completion, one unit a wave (2048 x 2048 M=16 6.2 / 7.3,
+  //    N=4096 K=1024 M=16 5.8 / 6.4, N=1024 K=4096 M=16 6.9 / 7.5, N=2048 K=1024 M=16 5.2 / 6.3).
+  //  * [N,K] row-load kernel: eight waves; 64 tiles or fewer split K four ways, on 128-byte bands up
+  //    to K = 2048 (1024 x 1024 M=8 3.5 / 4.0, M=16 3.9 / 4.3; N=1024 K=2048 M=16 4.2 / 5.0; N=1024
+  //    K=4096 M=4 4.6 / 5.8, M=16 5.2 / 7.3; N=512 K=2048 M=8 3.6 / 4.5); wider outputs with K up to
+  //    1024 stay unsplit on 128-byte bands (N=2048 K=1024 M=8 3.8 / 4.2, N=4096 K=1024 M=16 4.4 / 4.8).
+  if (splitk == 0 && M <= 16 && (size_t)N * K <= ((size_t)1 << 22)) {
+    fg_plan_t q = *p;
+    bool change = false;
+    if (w_layout == FG_W_KN) {
+      if ((size_t)N * K <= ((size_t)1 << 20) || ((size_t)N * K <= ((size_t)1 << 21) && M <= 8) || M <= 4) {
+        q.kernel = FG_KERNEL_KN_DOT2;
+        q.m_block = M == 1 ? 1 : 2;
+        q.waves = 4, q.unroll = 1;
+        q.splitk = K / 128 < 1 ? 1 : (K / 128 > 16 ? 16 : K / 128);
+        q.fused = q.splitk > 1 ? 2 : 0;
+        change = true;
+      } else if ((M > 8 || (M == 8 && N >= 4096)) && kXccs > 1) {
+        q.kernel = FG_KERNEL_KN_MFMA;
+        q.m_block = 16, q.unroll = 1;
+        q.splitk = K <= 2048 ? 8 : 16;
+        q.waves = K / 32 / q.splitk >= 8 ? 8 : 4;
+        q.fused = 3;
+        change = K / 32 >= q.splitk * q.waves;
+      }
+    } else if (p->kernel == FG_KERNEL_NK_MFMA_R && p->tile_n == 16 && p->m_block == 16 && K >= 512) {
+      q.waves = 8, q.unroll = 1;
+      if (N <= 1024 && K >= 1024) {
+        q.splitk = 4, q.fused = 2, q.band = K <= 2048 ? 128 : 0;
+        change = true;
+      } else if (K <= 1024) {
+        q.splitk = 1, q.fused = 0, q.band = 128;
+        change = true;
+      }
+    }
+    if (change && finish_plan(M, N, K, &q) == FG_OK) *p = q;
+  }
   return FG_OK;
 }
 

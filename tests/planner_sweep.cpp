@@ -62,7 +62,8 @@ static void check(int M, int N, int K, int layout, int splitk) {
     REQUIRE(p.kernel == FG_KERNEL_KN_MFMA && p.grid_y == 1 && splitk == 0);
     REQUIRE(p.splitk <= fg::kMailboxMaxSplit);
     REQUIRE((unsigned long long)p.grid_x * p.splitk * p.waves <= fg::kWsMailboxFlags);
-    REQUIRE((K / 32) / (p.waves * p.splitk * p.unroll) >= 2);
+    // every wave has a K unit; two, unless the whole problem is small (4 Mi weights or fewer)
+    REQUIRE((K / 32) / (p.waves * p.splitk * p.unroll) >= ((unsigned long long)N * K <= (1ull << 22) ? 1 : 2));
   }
   if (p.kernel == FG_KERNEL_KN_MFMA) REQUIRE(p.waves == 4 || p.waves == 8);
   if (splitk == 0 && M <= 16) REQUIRE(p.splitk == 1 || p.fused != 0);  // up to 16 rows complete in the launch

@@ -232,6 +232,23 @@ def test_plan_choices_that_were_measured():
     assert (p.splitk, p.waves) == (8, 8)           # two units a wave only: stays one 8-wave workgroup a CU
     p = kn(2, 12288, 4096)
     assert (p.splitk, p.waves) == (2, 8)           # 384 workgroups would fill the CUs unevenly
+    # small problems (4 Mi weights or fewer), fitted to per-launch times inside a replayed graph:
+    # [K,N] v_dot2 on two rows a workgroup with one unit a wave, the MFMA kernel with flags for nine
+    # rows and more beyond 1 Mi weights; [N,K] eight waves, narrow outputs split four ways
+    D, F = capi.FG_KERNEL_KN_DOT2, capi.FG_KERNEL_KN_MFMA
+    for (M, N, K, kern, mb, S, W, fused) in ((1, 1024, 1024, D, 1, 8, 4, 2), (8, 1024, 1024, D, 2, 8, 4, 2),
+                                             (16, 1024, 1024, D, 2, 8, 4, 2), (8, 1024, 2048, D, 2, 16, 4, 2),
+                                             (16, 2048, 512, D, 2, 4, 4, 2), (4, 2048, 2048, D, 2, 16, 4, 2),
+                                             (16, 2048, 1024, F, 16, 8, 4, 3), (16, 1024, 2048, F, 16, 8, 8, 3),
+                                             (16, 2048, 2048, F, 16, 8, 8, 3), (8, 4096, 1024, F, 16, 8, 4, 3),
+                                             (16, 1024, 4096, F, 16, 16, 8, 3)):
+        p = kn(M, N, K)
+        assert (p.kernel, p.m_block, p.splitk, p.waves, p.fused) == (kern, mb, S, W, fused), (M, N, K, p.as_dict())
+    for (M, N, K, S, band, fused) in ((8, 1024, 1024, 4, 128, 2), (16, 1024, 2048, 4, 128, 2), (4, 1024, 4096, 4, 256, 2),
+                                      (16, 512, 2048, 4, 128, 2), (8, 2048, 1024, 1, 128, 0), (16, 4096, 1024, 1, 128, 0)):
+        p = nk(M, N, K)
+        assert (p.kernel, p.waves, p.splitk, p.band, p.fused) == (R, 8, S, band, fused), (M, N, K, p.as_dict())
+    assert nk(8, 2048, 2048).splitk == 1 and nk(8, 2048, 2048).band == 256
 
 
 def test_plan_rejects_bad_arguments():
