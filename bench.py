@@ -378,7 +378,7 @@ def run_plan_grid(torch, capi, dev, steps, warmup):
             if M <= 8:
                 fams.append((capi.FG_KERNEL_KN_DOT2, M, 0, 0))
             for (kern, mb, tn, band), S, w, U in itertools.product(fams, (2, 4, 8, 16), (4, 8), (1, 2)):
-                for fused in (1, 2):
+                for fused in ((1, 2, 3) if kern == capi.FG_KERNEL_KN_MFMA else (1, 2)):
                     out.append(dict(kernel=kern, m_block=mb, tile_n=tn, band=band, splitk=S, waves=w, unroll=U,
                                     fused=fused))
         else:

@@ -151,7 +151,7 @@ int fg_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* out) {
   if (st != FG_OK) return st;
   st = fg::plan_make(M, N, K, w_layout, splitk, out);
   if (st != FG_OK) return st;
-  // FASTGATE_SPLITK_COMPLETION = two-pass | counter | atomic (read once) overrides how the
+  // FASTGATE_SPLITK_COMPLETION = two-pass | counter | atomic | xcd-local (read once) overrides how the
   // library's plans complete a split: a way back to the second kernel, whose only communication
   // is the kernel boundary, without rebuilding.
   static const int forced = [] {

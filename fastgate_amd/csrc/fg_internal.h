@@ -37,9 +37,6 @@ struct KnGeo {
   int log2_tiles, log2_tq, log2_xccs, log2_cus;  // log2 of those that are powers of two, else -1
   int spin_limit;  // polls of the mailbox owner before it recomputes what has not been delivered
   unsigned int nonce;  // host-side enqueue number of the launch (mailbox tags), 0 when unused
-#ifdef FG_PROBE
-  int probe;   // stage after which the kernel returns (timing probes; never in the product build)
-#endif
 };
 
 // Tile sets that exist as instantiations (the planner and the validators share these).

@@ -14,9 +14,6 @@
 #include "fg_device.h"
 #include "fg_internal.h"
 #include <atomic>
-#ifdef FG_PROBE
-#include <cstdlib>
-#endif
 
 namespace fg {
 
@@ -201,9 +198,6 @@ __global__ __launch_bounds__(64 * NW, (NW == 8 && U == 1) ? 4 : 1) void kn_mfma_
         for (int i = 0; i < 8; ++i)
           rws[u][i] = ok ? load16<true>(Wp + (size_t)(unit * 32 + i) * ldw) : zero;
         a[u] = (ok && arow) ? load16<false>(Ap + (size_t)unit * 32) : zero;
-#ifdef FG_PROBE
-        if (geo.probe == 101) a[u] = u32x4{0x3c003c00u, 0x3c003c00u, 0x3c003c00u, 0x3c003c00u};
-#endif
       }
 #pragma unroll
       for (int u = 0; u < U; ++u) {
@@ -215,10 +209,6 @@ __global__ __launch_bounds__(64 * NW, (NW == 8 && U == 1) ? 4 : 1) void kn_mfma_
                                                           0, 0);
       }
     }
-#ifdef FG_PROBE
-    if (geo.probe >= 100 && threadIdx.x == 0 && zz == it.z) { asm volatile("s_nop 0" :: "v"(acc[0]), "v"(acc[7])); reinterpret_cast<long long*>(reinterpret_cast<unsigned char*>(counters) + kWsHeaderBytes + (80u << 20))[(size_t)blockIdx.x * 8 + 1] = wall_clock64(); }
-    if (geo.probe == 1) { part[0] = acc[0] + acc[1] + acc[2] + acc[3] + acc[4] + acc[5] + acc[6] + acc[7]; if (part[0][0] == 12345.678f) C[0] = (half_t)1.f; return; }
-#endif
     float* mine = &red[wave][j][32 * g];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
@@ -265,19 +255,7 @@ __global__ __launch_bounds__(64 * NW, (NW == 8 && U == 1) ? 4 : 1) void kn_mfma_
     }
   };
 
-#ifdef FG_PROBE
-  long long* tdbg = reinterpret_cast<long long*>(reinterpret_cast<unsigned char*>(counters) + kWsHeaderBytes + (80u << 20)) + (size_t)blockIdx.x * 8;
-  const bool tstamp = geo.probe >= 100 && threadIdx.x == 0;
-  if (tstamp) { tdbg[0] = wall_clock64(); tdbg[7] = ((long long)xcc_id() << 32) | __builtin_amdgcn_s_getreg((31 << 11) | (0 << 6) | 4); }
-#define FG_TSTAMP(i) do { if (tstamp) tdbg[i] = wall_clock64(); } while (0)
-#else
-#define FG_TSTAMP(i) do { } while (0)
-#endif
   compute_partial(it.z);
-  FG_TSTAMP(2);
-#ifdef FG_PROBE
-  if (geo.probe == 2) { if (part[0][0] == 12345.678f) C[0] = (half_t)1.f; return; }
-#endif
   if (S == 1) {
     write_out(part);
     return;
@@ -316,25 +294,10 @@ __global__ __launch_bounds__(64 * NW, (NW == 8 && U == 1) ? 4 : 1) void kn_mfma_
     for (int q = 0; q < NQ; ++q) {
       const int e = q * NT + (int)threadIdx.x;
       const int m = e >> 5, c0 = (e & 31) * 4;
-#ifdef FG_PROBE
-      if (geo.probe == 201 || geo.probe == 202 || geo.probe == 203) {
-        const int byte = (int)((((size_t)it.z * M + m0 + m) * N + n0 + c0) * 4);
-        if (m < rows) {
-          if (geo.probe == 201) __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, part[q]), partials_rsrc(ws), byte, 0, 16);      // sc1
-          else if (geo.probe == 202) __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, part[q]), partials_rsrc(ws), byte, 0, 2);  // nt
-          else __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, part[q]), partials_rsrc(ws), byte, 0, 1);                        // sc0
-        }
-        continue;
-      }
-#endif
       if (m < rows) store_partial4(ws, ((size_t)it.z * M + m0 + m) * N + n0 + c0, part[q], coherent);
     }
   }
   if (counters == nullptr) return;  // a second kernel sums the partials
-#ifdef FG_PROBE
-  if (geo.probe == 3) return;
-#endif
-  FG_TSTAMP(3);
 
   float4_t tot[NQ];
   int off[NQ];                      // byte offset of the thread's groups within one partial
@@ -347,18 +310,9 @@ __global__ __launch_bounds__(64 * NW, (NW == 8 && U == 1) ? 4 : 1) void kn_mfma_
   }
   if (!mailbox) {
     const int arrived = splitk_arrive(counters + it.y * geo.tiles + it.tile, S, &s_arrival);
-    FG_TSTAMP(4);
     if (arrived == 0) return;
-#ifdef FG_PROBE
-    if (geo.probe == 4) return;
-#endif
     sum_partials_z<NQ, true>(ws, S, z_bytes, off, tot);
-    FG_TSTAMP(5);
     write_out(tot);
-#ifdef FG_PROBE
-    __builtin_amdgcn_s_waitcnt(0x0F70);
-#endif
-    FG_TSTAMP(6);
     return;
   }
 
@@ -369,7 +323,6 @@ __global__ __launch_bounds__(64 * NW, (NW == 8 && U == 1) ? 4 : 1) void kn_mfma_
   if (!owner) {
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's share of the partial is in the L2
     if (lane == 0) __hip_atomic_store(mb_flags + it.z * NW + wave, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-    FG_TSTAMP(4);
     return;
   }
   // Owner, up to eight partners (one flag per lane, one pass): every wave polls for itself and
@@ -435,7 +388,6 @@ __global__ __launch_bounds__(64 * NW, (NW == 8 && U == 1) ? 4 : 1) void kn_mfma_
       give_up = __builtin_amdgcn_readfirstlane(seen) == 2;
     }
     if (!give_up) {
-      FG_TSTAMP(4);
 #pragma unroll
       for (int q = 0; q < NQ; ++q) {
         float4_t sum = {0.f, 0.f, 0.f, 0.f};
@@ -443,12 +395,7 @@ __global__ __launch_bounds__(64 * NW, (NW == 8 && U == 1) ? 4 : 1) void kn_mfma_
         for (int z = 0; z < PF; ++z) sum += v[z][q];  // partners past S - 1 stayed +0
         tot[q] = sum + part[q];
       }
-      FG_TSTAMP(5);
       write_out(tot);
-#ifdef FG_PROBE
-      __builtin_amdgcn_s_waitcnt(0x0F70);
-#endif
-      FG_TSTAMP(6);
       return;
     }
     // every wave arrives here: recompute all partials (what was loaded is not used)
@@ -490,7 +437,6 @@ __global__ __launch_bounds__(64 * NW, (NW == 8 && U == 1) ? 4 : 1) void kn_mfma_
   }
   __syncthreads();
   const unsigned int ready = (unsigned int)s_arrival;
-  FG_TSTAMP(4);
   if (ready == all) {
     sum_partials_z<NQ, false>(ws, S - 1, z_bytes, off, tot);
 #pragma unroll
@@ -518,12 +464,7 @@ __global__ __launch_bounds__(64 * NW, (NW == 8 && U == 1) ? 4 : 1) void kn_mfma_
 #pragma unroll
     for (int q = 0; q < NQ; ++q) tot[q] += own[q];
   }
-  FG_TSTAMP(5);
   write_out(tot);
-#ifdef FG_PROBE
-  __builtin_amdgcn_s_waitcnt(0x0F70);
-#endif
-  FG_TSTAMP(6);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -696,9 +637,6 @@ static void kn_mfma_go(const fg_plan_t& p, const GemmArgs& a, hipStream_t s) {
   // a new number for every enqueue of a launch that uses the flags (1 .. 2^24 - 1, wrapping)
   static std::atomic<unsigned int> enqueues{0};
   geo.nonce = (a.accumulate & kFlagXcdLocal) ? enqueues.fetch_add(1, std::memory_order_relaxed) % 0xFFFFFu + 1u : 0u;
-#ifdef FG_PROBE
-  { const char* e = getenv("FG_PROBE"); geo.probe = e ? atoi(e) : 0; }
-#endif
   // one-dimensional grid: row blocks x splits x column tiles; in XCD-local order every XCD gets the
   // same number of column tiles (the last ones may be empty)
   const int tiles_padded = (a.accumulate & kFlagXcdLocal) ? (p.grid_x + a.xccs - 1) / a.xccs * a.xccs : p.grid_x;
