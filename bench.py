@@ -255,7 +255,7 @@ def run_sweep(torch, sg, capi, dev, steps, warmup, models=False):
     us_f16 = next(r["us_per_call"] for r in rows if r["config"] == "C5 sweep" and r["M"] == 1 and r["K"] == 8192
                   and r["w_layout"] == "[N,K]")
     rows.append(with_same_size({"config": "C4 int8 fastgemv", "op": "fastgemv_int8", "M": 1, "K": Kk, "N": Nn, "w_layout": "[N,K] int8",
-                 "seed": 1004, "kernel": "w8a16", "splitk": 1, "bytes": by, "us_per_call": round(us_i8, 2),
+                 "seed": 1004, "kernel": "wq_m1<int8>", "splitk": 1, "bytes": by, "us_per_call": round(us_i8, 2),
                  "GBps": round(by / us_i8 / 1e3, 1), "frac_hbm_peak": round(by / us_i8 / 1e3 / HBM_PEAK_GBPS, 4),
                  "frac_read_ceiling": round(by / us_i8 / 1e3 / ceiling, 4),
                  "weights_per_ns": round(Kk * Nn / us_i8 / 1e3, 3),
@@ -283,7 +283,7 @@ def run_sweep(torch, sg, capi, dev, steps, warmup, models=False):
     us_i4 = time_us(lambda i: sg.fastgemv_int4(wq4[i % 20], x, y, scale=scale, zero_point=8.0))
     by = Kk * Nn // 2 + 2 * Kk + 2 * Nn + 2 * Nn
     rows.append(with_same_size({"config": "extra: int4 fastgemv", "op": "fastgemv_int4", "M": 1, "K": Kk, "N": Nn,
-                 "w_layout": "[N,K/2] uint4x2", "seed": 1004, "kernel": "w4a16", "splitk": 1, "bytes": by,
+                 "w_layout": "[N,K/2] uint4x2", "seed": 1004, "kernel": "wq_m1<int4>", "splitk": 1, "bytes": by,
                  "us_per_call": round(us_i4, 2), "GBps": round(by / us_i4 / 1e3, 1),
                  "frac_hbm_peak": round(by / us_i4 / 1e3 / HBM_PEAK_GBPS, 4),
                  "frac_read_ceiling": round(by / us_i4 / 1e3 / ceiling, 4),
