@@ -325,7 +325,7 @@ __global__ __launch_bounds__(64 * NW, (NW == 8 && U == 1) ? 4 : 1) void kn_mfma_
     if (lane == 0) __hip_atomic_store(mb_flags + it.z * NW + wave, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     return;
   }
-  // Owner, up to eight partners (one flag per lane, one pass): every wave polls for itself and
+  // Owner, eight partners at a time (one flag per lane, one pass): every wave polls for itself and
   // loads a partner's partial the moment that partner's flags are up.  Partials of partners that
   // finished microseconds ago have left the L2 by now; loading them while waiting for the last
   // partner takes that memory latency off the end of the kernel.  The values wait in registers and
@@ -335,49 +335,61 @@ __global__ __launch_bounds__(64 * NW, (NW == 8 && U == 1) ? 4 : 1) void kn_mfma_
   // this launch from another XCD (everybody recomputes).
   constexpr int PF = 8;
   const unsigned int all = (1u << (S - 1)) - 1u;  // S <= 32
-  if (it.home && S - 1 <= PF && (S - 1) * NW <= 64) {
-    const int nflags = (S - 1) * NW;
+  if (it.home) {
+    // (more than eight partners: eight at a time, in ascending z; the sum runs on in that order)
     const __amdgpu_buffer_rsrc_t rsrc = partials_rsrc(ws);
-    float4_t v[PF][NQ];
+    float4_t run[NQ];
 #pragma unroll
-    for (int z = 0; z < PF; ++z)
-#pragma unroll
-      for (int q = 0; q < NQ; ++q) v[z][q] = float4_t{0.f, 0.f, 0.f, 0.f};
-    unsigned int loaded = 0;
+    for (int q = 0; q < NQ; ++q) run[q] = float4_t{0.f, 0.f, 0.f, 0.f};
     bool give_up = false;
-    for (int spins = 0;; ++spins) {
-      const unsigned long long f =
-          lane < nflags ? __hip_atomic_load(mb_flags + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : tag;
-      const unsigned long long b = __builtin_amdgcn_ballot_w64(f == tag);
-      const bool misplaced = __builtin_amdgcn_ballot_w64(tag_is_foreign(f, tag)) != 0;  // a partner on another XCD
+    int spins = 0;
+    for (int c0 = 0; c0 < S - 1 && !give_up; c0 += PF) {
+      const int np = S - 1 - c0 < PF ? S - 1 - c0 : PF;
+      const int nflags = np * NW;  // <= 64: one flag per lane
+      const unsigned int all_c = (1u << np) - 1u;
+      float4_t v[PF][NQ];
+      unsigned int loaded = 0;
+      for (;; ++spins) {
+        const unsigned long long f =
+            lane < nflags ? __hip_atomic_load(mb_flags + c0 * NW + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : tag;
+        const unsigned long long b = __builtin_amdgcn_ballot_w64(f == tag);
+        const bool misplaced = __builtin_amdgcn_ballot_w64(tag_is_foreign(f, tag)) != 0;  // a partner on another XCD
 #pragma unroll
-      for (int z = 0; z < PF; ++z) {
-        const unsigned long long lanes = ((1ull << NW) - 1) << (z * NW);
-        if (z < S - 1 && !((loaded >> z) & 1u) && (b & lanes) == lanes) {
+        for (int z = 0; z < PF; ++z) {
+          const unsigned long long lanes = ((1ull << NW) - 1) << (z * NW);
+          if (z < np && !((loaded >> z) & 1u) && (b & lanes) == lanes) {
 #pragma unroll
-          for (int q = 0; q < NQ; ++q)
-            v[z][q] = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc, off[q], z * z_bytes, 1));
-          loaded |= 1u << z;
+            for (int q = 0; q < NQ; ++q)
+              v[z][q] = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc, off[q], (c0 + z) * z_bytes, 1));
+            loaded |= 1u << z;
+          }
         }
-      }
-      if (loaded == all) break;
-      if (__hip_atomic_load(&s_state, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) == 2) {
-        give_up = true;
-        break;
-      }
-      if (misplaced || (wave == 0 && spins >= geo.spin_limit)) {
-        int seen = 0;
-        if (lane == 0) {
-          __hip_atomic_compare_exchange_strong(&s_state, &seen, 2, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
-                                               __HIP_MEMORY_SCOPE_WORKGROUP);
-        }
-        seen = __builtin_amdgcn_readfirstlane(seen);
-        if (seen != 1) {  // nobody has everything: give up (a wave that has, keeps the others going)
+        if (loaded == all_c) break;
+        if (__hip_atomic_load(&s_state, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) == 2) {
           give_up = true;
           break;
         }
+        if (misplaced || (wave == 0 && spins >= geo.spin_limit)) {
+          int seen = 0;
+          if (lane == 0) {
+            __hip_atomic_compare_exchange_strong(&s_state, &seen, 2, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                                 __HIP_MEMORY_SCOPE_WORKGROUP);
+          }
+          seen = __builtin_amdgcn_readfirstlane(seen);
+          if (seen != 1) {  // nobody has everything: give up (a wave that has, keeps the others going)
+            give_up = true;
+            break;
+          }
+        }
+        __builtin_amdgcn_s_sleep(1);
       }
-      __builtin_amdgcn_s_sleep(1);
+      if (give_up) break;
+#pragma unroll
+      for (int z = 0; z < PF; ++z)
+        if (z < np) {
+#pragma unroll
+          for (int q = 0; q < NQ; ++q) run[q] += v[z][q];
+        }
     }
     if (!give_up) {
       int seen = 0;
@@ -389,12 +401,7 @@ __global__ __launch_bounds__(64 * NW, (NW == 8 && U == 1) ? 4 : 1) void kn_mfma_
     }
     if (!give_up) {
 #pragma unroll
-      for (int q = 0; q < NQ; ++q) {
-        float4_t sum = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int z = 0; z < PF; ++z) sum += v[z][q];  // partners past S - 1 stayed +0
-        tot[q] = sum + part[q];
-      }
+      for (int q = 0; q < NQ; ++q) tot[q] = run[q] + part[q];
       write_out(tot);
       return;
     }
