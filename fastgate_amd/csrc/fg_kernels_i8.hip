@@ -35,6 +35,32 @@ __device__ __forceinline__ float scale_value(uint32_t raw) {
   return f16_bits_to_f32((uint16_t)raw);
 }
 
+// The zero point (and the 128 that the subnormal form of int8 carries) leaves a dot product as one
+// term, constant x Σx.  An activation row that holds an infinity or a NaN makes Σx non-finite, and
+// that term would then turn every output of the row into NaN, where element-by-element arithmetic
+// -- sum += x (float(w) - zp), backend/cuda/hk/fastgemv.cuh:344-363 -- gives ±inf when infinities
+// of one sign meet weights on one side of the zero point.  Σx is non-finite for such rows only
+// (finite halves cannot overflow an fp32 sum), so the thread that writes an output looks at it
+// and, for such a row, computes its one output again the reference's way: K steps in one thread,
+// paid only by input that is already broken.  BITS = 4: two nibbles a byte, the even k low.
+__device__ __forceinline__ bool not_finite(float v) { return !(__builtin_fabsf(v) <= 3.4028234664e38f); }
+template <int BITS>
+__device__ float elementwise_dot(const uint8_t* __restrict__ wrow, const half_t* __restrict__ xrow, int K,
+                                 float zero_point) {
+  float s = 0.f;
+  for (int k = 0; k < K; ++k) {
+    int w;
+    if (BITS == 8) {
+      w = static_cast<int8_t>(wrow[k]);
+    } else {
+      const uint32_t b = wrow[k >> 1];
+      w = (k & 1) ? b >> 4 : b & 15u;
+    }
+    s += static_cast<float>(xrow[k]) * (static_cast<float>(w) - zero_point);
+  }
+  return s;
+}
+
 template <int MB, int RN, int U>
 __global__ __launch_bounds__(512) void w8a16_kernel(const int8_t* __restrict__ Wq,
                                                     const half_t* __restrict__ X,
@@ -133,9 +159,12 @@ __global__ __launch_bounds__(512) void w8a16_kernel(const int8_t* __restrict__ W
     const float sum = lds_sum<32>(&red[0][r * MB + m], RN * MB, nw * 4);
     const float xs = lds_sum<32>(&redx[0][m], MB, nw * 4);
     const int n = n0 + r;
-    if (m < M)
-      Y[(size_t)m * N + n] =
-          static_cast<half_t>((sum - zero_point * xs) * (scalar_scale * scale_value(scale_raw)));
+    if (m < M) {
+      float v = sum - zero_point * xs;
+      if (not_finite(xs))
+        v = elementwise_dot<8>(reinterpret_cast<const uint8_t*>(Wq) + (size_t)n * K, X + (size_t)m * K, K, zero_point);
+      Y[(size_t)m * N + n] = static_cast<half_t>(v * (scalar_scale * scale_value(scale_raw)));
+    }
   }
 }
 
@@ -264,7 +293,9 @@ __global__ __launch_bounds__(64 * NWV) void wq_m1_kernel(const uint8_t* __restri
   if (threadIdx.x < RN) {
     const float sum = lds_sum<NWV * 4>(&red[0][threadIdx.x], RN + 1, NWV * 4);
     const float xs = lds_sum<NWV * 4>(&red[0][RN], RN + 1, NWV * 4);
-    Y[n0 + threadIdx.x] = static_cast<half_t>((sum - zp * xs) * (scalar_scale * scale_value(scale_raw)));
+    float v = sum - zp * xs;
+    if (not_finite(xs)) v = elementwise_dot<BITS>(Wt + (size_t)threadIdx.x * rowb, X, K, zero_point);
+    Y[n0 + threadIdx.x] = static_cast<half_t>(v * (scalar_scale * scale_value(scale_raw)));
   }
 }
 
@@ -479,8 +510,10 @@ __global__ __launch_bounds__(64 * NW) void w8a16_r_kernel(const int8_t* __restri
     if (m < M) {
       const float sum = lds_sum<NW>(&red[0][0][e], 2 * 16 * TN, nw);
       const float xs = lds_sum<NW>(&red[0][1][m * 16 + (e & 15)], 2 * 16 * TN, nw);
-      Y[(size_t)m * N + n] = static_cast<half_t>((sum * 16777216.f - (zero_point + 128.f) * xs) *
-                                                 (scalar_scale * scale_value(scale_raw)));
+      float v = sum * 16777216.f - (zero_point + 128.f) * xs;
+      if (not_finite(xs))
+        v = elementwise_dot<8>(reinterpret_cast<const uint8_t*>(Wq) + (size_t)n * K, X + (size_t)m * K, K, zero_point);
+      Y[(size_t)m * N + n] = static_cast<half_t>(v * (scalar_scale * scale_value(scale_raw)));
     }
   }
 }
@@ -602,8 +635,9 @@ __global__ __launch_bounds__(512) void w4a16_r_kernel(const uint8_t* __restrict_
     if (m < M) {
       const float sum = lds_sum<NW>(&red[0][0][e], 512, nw);
       const float xs = lds_sum<NW>(&red[0][1][e], 512, nw);
-      Y[(size_t)m * N + n] =
-          static_cast<half_t>((sum - zero_point * xs) * (scalar_scale * scale_value(scale_raw)));
+      float v = sum - zero_point * xs;
+      if (not_finite(xs)) v = elementwise_dot<4>(Wq + (size_t)n * rowb, X + (size_t)m * K, K, zero_point);
+      Y[(size_t)m * N + n] = static_cast<half_t>(v * (scalar_scale * scale_value(scale_raw)));
     }
   }
 }

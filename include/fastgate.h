@@ -220,7 +220,10 @@ int fg_workspace_init(void* ws, size_t ws_bytes, void* stream);
  * W8A16 GEMV: y[m,n] = s_n · ( Σ_k x[m,k]·float(Wq[n,k]) − zero_point·Σ_k x[m,k] ),
  * s_n = scalar_scale · (scale ? float(scale[n]) : 1).  Wq int8 [N,K] row-major, x fp16
  * [M,K], scale fp16 [N] or NULL, y fp16 [M,N].  fp32 accumulation, int8→fp16 conversion
- * is exact.  1 <= M <= 16.
+ * is exact.  1 <= M <= 16.  An activation row that holds an infinity or a NaN gets the class the
+ * reference's element-by-element sum of x·(float(Wq) − zero_point) has (±inf, or NaN where the
+ * weight under the infinity equals the zero point or infinities of both signs meet), not the
+ * NaN that inf − inf of the two-term form above would give; the same holds for fg_gemv_w4a16.
  * Services fastgemv_int8 (backend/cuda/hk/fastgemv.cu:35-61; kernel formula
  * hk/fastgemv.cuh:316-389, whose host passes scale = 1, zero_point = 0); the per-channel
  * scale vector is an extension the reference does not have.

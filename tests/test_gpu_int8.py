@@ -381,3 +381,52 @@ def test_one_row_kernels_small_integers_and_zero_point_are_exact(device, bits):
             got = _w4a16(W, x, None, 1.0, 8.0, device)
         # every fp32 sum on the way is an integer below 2^24: the one rounding to fp16 decides
         assert (got.view(np.uint16) == ref.view(np.uint16)).all(), (N, K)
+
+
+@pytest.mark.parametrize("bits,M,N", [(8, 1, 1024), (8, 2, 1024), (8, 4, 1024), (8, 4, 4096), (8, 8, 4096),
+                                      (8, 16, 2048), (8, 16, 16384), (4, 1, 1024), (4, 2, 512), (4, 4, 512)])
+@pytest.mark.parametrize("zp", [0.0, 3.0])
+def test_infinite_and_nan_activations_keep_the_class_of_element_by_element_sums(device, bits, M, N, zp):
+    # hk/fastgemv.cuh:344-363 adds x (float(w) - zp) element by element: +inf against weights above the
+    # zero point gives +inf, below it -inf, on it NaN; infinities of both signs or a NaN give NaN.
+    # The kernels take the zero point (and int8's + 128) out as one term with Σx, which alone would
+    # make every such output NaN; rows with finite activations must not notice their neighbours.
+    K = 1152
+    g = gen(6300 + bits + M + N)
+    x = normal((M, K), g)
+    k0, k1 = 5, 700
+    x[0, k0] = float("inf")
+    if M > 1:
+        x[1, k1] = float("nan")
+    if M > 2:
+        x[2, k0], x[2, k1] = float("inf"), float("-inf")
+    if M > 3:
+        x[3, k1] = float("-inf")
+    third = N // 3
+    if bits == 8:
+        W = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8)
+        W[:third, k0] = int(zp)        # on the zero point: NaN
+        W[third:2 * third, k0] = 100   # above: the sign of the infinity
+        W[2 * third:, k0] = -100       # below: the other sign
+        W[::2, k1] = 50
+        W[1::2, k1] = -50
+        ref, _ = oracle.gemv_w8a16(W.numpy(), x.numpy(), None, 1.0, zp)
+        got = _w8a16(W, x, None, 1.0, zp, device)
+    else:
+        W = torch.randint(0, 256, (N, K // 2), generator=g, dtype=torch.uint8)
+        lo = lambda col, v: (col & 0xF0) | v      # k0 is odd: the high nibble; k1 even: the low one
+        W[:third, k0 // 2] = (W[:third, k0 // 2] & 0x0F) | (int(zp) << 4)
+        W[third:2 * third, k0 // 2] = (W[third:2 * third, k0 // 2] & 0x0F) | (12 << 4)
+        W[2 * third:, k0 // 2] = (W[2 * third:, k0 // 2] & 0x0F) | (1 << 4)
+        W[::2, k1 // 2] = lo(W[::2, k1 // 2], 9)
+        W[1::2, k1 // 2] = lo(W[1::2, k1 // 2], 2)
+        ref, _ = oracle.gemv_w4a16(W.numpy(), x.numpy(), None, 1.0, zp)
+        got = _w4a16(W, x, None, 1.0, zp, device)
+    assert np.isnan(ref[0, :third]).all() and np.isinf(ref[0, third:]).all()  # the case is what it claims
+    assert (np.isnan(got) == np.isnan(ref)).all()
+    inf = np.isinf(ref)
+    assert (np.isinf(got) == inf).all() and (got[inf] == ref[inf]).all()
+    broken = min(M, 4)
+    assert np.isfinite(ref[broken:]).all()
+    if M > broken:
+        assert_close_f16(got[broken:], ref[broken:], "rows with finite activations")
