@@ -4,7 +4,9 @@
 //    integer pipe's cheap ops: flip the sign bit (w+128 as unsigned), splice each byte under
 //    the exponent 0x64 (fp16 value 1024 + byte), subtract 1152 with v_pk_add_f16 -> the exact
 //    integer as fp16, then v_dot2_f32_f16 against the activations (fp32 accumulation).  The
-//    per-output-channel scale and the zero point are applied once per output.
+//    per-output-channel scale and the zero point are applied once per output.  The one-row
+//    kernel and the row-load kernel take a shorter way (the bytes as fp16 subnormals, see
+//    wq_m1_kernel); this form remains in w8a16_kernel, for 2..4 rows against narrow outputs.
 //  * i8i8: int8 activations, v_dot4_i32_i8, exact int32 result.
 //
 // Replaces the device side of gemv_quantized_int8 (backend/cuda/hk/fastgemv.cuh:316-389,
