@@ -327,10 +327,13 @@ __device__ __forceinline__ int splitk_arrive(int* counter, int S, int* s_word) {
   return *s_word;
 }
 
-// 16 bytes of a partial that a workgroup of the same XCD stored with an ordinary store: a load that
-// is not served from this CU's L1 but by the XCD's L2, where that store landed.
+// 16 bytes of a partial that a workgroup of the same XCD stored with an ordinary store, served by
+// the XCD's L2, where that store landed.  A workgroup-scope load (sc0) may be answered by this CU's
+// L1 when the line is there, so the caller must be the first on its CU to touch the line since the
+// kernel began (a kernel starts with the L1 invalidated): read a partial once, after its flag, and
+// never poll with this load -- the second poll would see the first one's line for ever.
 __device__ __forceinline__ float4_t load_partial4_l2(const float* base, size_t idx) {
-  constexpr int kCachePolicyWorkgroup = 1;  // sc0: not served from this CU's L1
+  constexpr int kCachePolicyWorkgroup = 1;  // sc0
   return __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(
                                           partials_rsrc(base), (int)(idx * 4), 0, kCachePolicyWorkgroup));
 }
@@ -341,7 +344,7 @@ __device__ __forceinline__ float4_t load_partial4_l2(const float* base, size_t i
 template <int NQ, int BATCH, bool MEM>
 __device__ __forceinline__ void sum_partials_z_batched(const float* part, int S, int z_bytes, const int (&off)[NQ],
                                                        float4_t (&sum)[NQ]) {
-  constexpr int kPolicy = MEM ? kCachePolicyAgent : 1;  // sc1: past the L2s; sc0: past this CU's L1 only
+  constexpr int kPolicy = MEM ? kCachePolicyAgent : 1;  // sc1: past the L2s; sc0: this XCD's L2 (see load_partial4_l2)
   const __amdgpu_buffer_rsrc_t rsrc = partials_rsrc(part);
 #pragma unroll
   for (int q = 0; q < NQ; ++q) sum[q] = float4_t{0.f, 0.f, 0.f, 0.f};
