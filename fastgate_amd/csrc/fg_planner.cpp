@@ -598,7 +598,11 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
   // N=8192 K=16384 M=16 43.8 / 46.3; N=12288 K=8192 M=8 34.4 / 36.3, K=12288 M=16 50.0 / 52.7;
   // N=16384 K=3072 M=8 18.6 / 19.8; N=11008 K=4096 M=16 18.6 / 19.3; N=4096 K=4096 M=16 10.1 / 10.6;
   // N=3072 K=4096 M=16 8.8 / 9.9; N=2048 K=12288 M=16 13.0 / 14.1.  Not taken where it measured level
-  // or behind: 14 336 columns, N = 16384 with few rows and long K, short K.
+  // or behind: 14 336 columns, N = 16384 with few rows and long K, short K.  A later pass over
+  // N in {4096, 8192} x 10 K x M in {4, 8, 16} widened the 64-tile rows (N = 8192: M=4 K=5504 17.9 /
+  // 19.0, K=11008 31.2 / 32.5; M=8 K=4096 14.4 / 14.8, K=6144 19.2 / 20.1; M=16 K=5504 18.7 / 19.4,
+  // K=6144 19.3 / 20.4 with two units a step) and added long K at 32 tiles (N=4096 K=11008 M=8 18.3 /
+  // 18.8, K=14336 21.9 / 22.4; level for M=4 and for K = 12288).
   if (splitk == 0 && p->kernel == FG_KERNEL_KN_MFMA && M >= 3 && M <= 16 && p->grid_y == 1 && kXccs > 1 &&
       p->splitk > 1) {
     const int tiles = N / 128, units = K / 32;
@@ -609,13 +613,14 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
       if (tiles == 16) S = 16;
       else if (tiles == 24 && K <= 8192 && M > 12) S = 8;
       else if (tiles == 32) S = 8;
-      else if (tiles == 64 && K >= 8192) S = 8, U = 2;
+      else if (tiles == 64 && K >= 4096) S = 8, U = K >= 6144 ? 2 : 1;
       else if (tiles == 86) S = 5;
       else if (tiles == 96) S = 8;
       else if (tiles == 128 && K <= 4096) S = 4, w = 8;
       else if (tiles == 128) S = p->splitk, w = p->waves, U = p->unroll;
     } else {
-      if (tiles == 64 && K >= 8192 && M >= 7) S = 8;
+      if (tiles == 64 && K >= 3072) S = 8;
+      else if (tiles == 32 && K >= 11008 && M >= 7) S = 8;
       else if (tiles == 86 && K >= 3072 && K <= 4096 && M == 8) S = 5;
       else if (tiles == 96 && K >= 4096) S = 8;
       else if (tiles == 128 && K < 4096) S = 4, w = 8;
