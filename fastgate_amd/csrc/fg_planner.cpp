@@ -602,7 +602,13 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
   // N in {4096, 8192} x 10 K x M in {4, 8, 16} widened the 64-tile rows (N = 8192: M=4 K=5504 17.9 /
   // 19.0, K=11008 31.2 / 32.5; M=8 K=4096 14.4 / 14.8, K=6144 19.2 / 20.1; M=16 K=5504 18.7 / 19.4,
   // K=6144 19.3 / 20.4 with two units a step) and added long K at 32 tiles (N=4096 K=11008 M=8 18.3 /
-  // 18.8, K=14336 21.9 / 22.4; level for M=4 and for K = 12288).
+  // 18.8, K=14336 21.9 / 22.4; level for M=4 and for K = 12288).  A third pass put widths between
+  // the fitted ones beside them (N in {5120, 6144, 10240, 12288} x 9 K x M in {4, 8, 16}, the library's
+  // plan beside every flag plan that fills 224..1024 wave slots): 48 tiles x 9 splits (N=6144 K=4096
+  // M=8 12.1 / 12.4, K=8192 M=16 20.4 / 21.1, K=11008 24.6 / 25.3; K=3072 behind), 80 tiles x 6
+  // (N=10240 K=4096 M=16 17.2 / 18.3, K=11008 37.9 / 39.6, K=16384 53.5 / 55.9), 40 tiles x 6 from
+  // K = 8192 on for seven rows and more (N=5120 K=8192 M=16 18.0 / 18.5, level at K = 12288), and 96
+  // tiles from K = 2048 on for eight rows and fewer (N=12288 K=3072 M=8 15.7 / 16.4).
   if (splitk == 0 && p->kernel == FG_KERNEL_KN_MFMA && M >= 3 && M <= 16 && p->grid_y == 1 && kXccs > 1 &&
       p->splitk > 1) {
     const int tiles = N / 128, units = K / 32;
@@ -614,6 +620,9 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
       else if (tiles == 24 && K <= 8192 && M > 12) S = 8;
       else if (tiles == 32) S = 8;
       else if (tiles == 64 && K >= 4096) S = 8, U = K >= 6144 ? 2 : 1;
+      else if (tiles == 40 && K >= 8192) S = 6;
+      else if (tiles == 48 && K >= 4096) S = 9;
+      else if (tiles == 80 && K >= 3072) S = 6;
       else if (tiles == 86) S = 5;
       else if (tiles == 96) S = 8;
       else if (tiles == 128 && K <= 4096) S = 4, w = 8;
@@ -622,7 +631,10 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
       if (tiles == 64 && K >= 3072) S = 8;
       else if (tiles == 32 && K >= 11008 && M >= 7) S = 8;
       else if (tiles == 86 && K >= 3072 && K <= 4096 && M == 8) S = 5;
-      else if (tiles == 96 && K >= 4096) S = 8;
+      else if (tiles == 40 && K >= 8192 && M >= 7) S = 6;
+      else if (tiles == 48 && K >= 4096) S = 9;
+      else if (tiles == 80 && K >= 3072) S = 6;
+      else if (tiles == 96 && K >= 2048) S = 8;
       else if (tiles == 128 && K < 4096) S = 4, w = 8;
       else if (tiles == 128 && K == 4096) S = p->splitk, w = p->waves, U = p->unroll;
     }

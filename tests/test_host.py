@@ -203,7 +203,7 @@ def test_plan_choices_that_were_measured():
         assert (p.kernel, p.splitk, p.waves) == (capi.FG_KERNEL_KN_DOT2, S, 4), (M, N, K, p.as_dict())
     # completion of the split: atomics for v_dot2, for [N,K] and for few elements; the counter otherwise
     assert kn(1, 8192, 8192).fused == 2 and kn(8, 4096, 4096).fused == 2 and nk(16, 2048, 8192).fused == 2
-    assert kn(16, 5120, 8192).fused == 1 and kn(8, 14336, 8192).fused == 1
+    assert kn(16, 5120, 4096).fused == 1 and kn(8, 14336, 8192).fused == 1
     # the [K,N] MFMA kernel: atomics only for deep splits or few elements (four waves: from 8 splits on)
     assert kn(8, 4096, 8192).fused == 2 and kn(8, 11008, 2048).fused == 2
     # ... and flags in one XCD's L2 where the partials are large, with two or three 4-wave workgroups a
@@ -216,14 +216,19 @@ def test_plan_choices_that_were_measured():
                                # 64 tiles from K = 3072 (nine rows and more: 4096) on, 32 tiles with long K
                                (4, 8192, 8192, 8, 4, 1), (4, 8192, 5504, 8, 4, 1), (8, 8192, 4096, 8, 4, 1),
                                (6, 8192, 3072, 8, 4, 1), (16, 8192, 4096, 8, 4, 1), (16, 8192, 6144, 8, 4, 2),
-                               (8, 4096, 11008, 8, 4, 1)):
+                               (8, 4096, 11008, 8, 4, 1),
+                               # widths between the fitted ones: 48 tiles x 9, 80 x 6, 40 x 6, 96 x 8 for short K
+                               (16, 6144, 8192, 9, 4, 1), (8, 6144, 4096, 9, 4, 1), (4, 10240, 8192, 6, 4, 1),
+                               (16, 10240, 3072, 6, 4, 1), (16, 5120, 8192, 6, 4, 1), (8, 5120, 11008, 6, 4, 1),
+                               (8, 12288, 3072, 8, 4, 1)):
         p = kn(M, N, K)
         assert (p.splitk, p.waves, p.unroll, p.fused) == (S, W, U, 3), (M, N, K, p.as_dict())
     # not where the sweep did not go (48 tiles x 6 splits would fill the CUs unevenly) or measured level
-    assert kn(16, 6144, 8192).fused != 3 and kn(16, 14336, 8192).fused != 3 and kn(8, 16384, 8192).fused != 3
+    assert kn(16, 6144, 3072).fused != 3 and kn(16, 14336, 8192).fused != 3 and kn(8, 16384, 8192).fused != 3
+    assert kn(4, 5120, 8192).fused != 3 and kn(16, 5120, 6144).fused != 3 and kn(8, 10240, 2048).fused != 3
     assert kn(4, 8192, 2048).fused != 3 and kn(16, 8192, 3072).fused != 3 and kn(4, 4096, 11008).fused != 3
     assert kn(24, 2048, 4096).fused == 0           # more than 16 rows: second kernel
-    p = kn(16, 5120, 8192)
+    p = kn(16, 5120, 6144)
     assert (p.splitk, p.waves) == (6, 8)
     p = kn(12, 4096, 2048)
     assert (p.splitk, p.waves, p.fused) == (8, 4, 3)    # 7.65 us against 8.34 for four splits of 8 waves and the counter
