@@ -608,7 +608,12 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
   // M=8 12.1 / 12.4, K=8192 M=16 20.4 / 21.1, K=11008 24.6 / 25.3; K=3072 behind), 80 tiles x 6
   // (N=10240 K=4096 M=16 17.2 / 18.3, K=11008 37.9 / 39.6, K=16384 53.5 / 55.9), 40 tiles x 6 from
   // K = 8192 on for seven rows and more (N=5120 K=8192 M=16 18.0 / 18.5, level at K = 12288), and 96
-  // tiles from K = 2048 on for eight rows and fewer (N=12288 K=3072 M=8 15.7 / 16.4).
+  // tiles from K = 2048 on for eight rows and fewer (N=12288 K=3072 M=8 15.7 / 16.4).  The same for
+  // N in {2560, 3584, 9216, 18432, 20480, 24576}: 72 tiles x 7 (N=9216 K=4096 M=8 15.7 / 17.3, K=8192
+  // 26.3 / 28.4, K=16384 48.0 / 51.4), 144 x 5 (N=18432 K=4096 M=16 27.1 / 30.9, K=16384 95.8 / 105.1),
+  // 160 x 6 with two units a step up to eight rows (N=20480 K=8192 M=4 53.4 / 55.5), 192 x 4 (N=24576
+  // K=8192 M=16 65.9 / 69.3), and nine rows and more on 20 and 28 tiles with short K (N=2560 K=4096
+  // 8.8 / 9.5, N=3584 K=3072 8.8 / 9.3); 36, 56, 108 and 112 tiles measured level or behind.
   if (splitk == 0 && p->kernel == FG_KERNEL_KN_MFMA && M >= 3 && M <= 16 && p->grid_y == 1 && kXccs > 1 &&
       p->splitk > 1) {
     const int tiles = N / 128, units = K / 32;
@@ -620,9 +625,14 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
       else if (tiles == 24 && K <= 8192 && M > 12) S = 8;
       else if (tiles == 32) S = 8;
       else if (tiles == 64 && K >= 4096) S = 8, U = K >= 6144 ? 2 : 1;
+      else if (tiles == 20 && K >= 4096 && K <= 6144) S = 8, w = 8;
+      else if (tiles == 28 && K <= 4096) S = 8, w = K == 4096 ? 8 : 4;
       else if (tiles == 40 && K >= 8192) S = 6;
       else if (tiles == 48 && K >= 4096) S = 9;
+      else if (tiles == 72) S = 7;
       else if (tiles == 80 && K >= 3072) S = 6;
+      else if (tiles == 144) S = 5;
+      else if (tiles == 192 && K >= 4096) S = 4;
       else if (tiles == 86) S = 5;
       else if (tiles == 96) S = 8;
       else if (tiles == 128 && K <= 4096) S = 4, w = 8;
@@ -633,7 +643,11 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
       else if (tiles == 86 && K >= 3072 && K <= 4096 && M == 8) S = 5;
       else if (tiles == 40 && K >= 8192 && M >= 7) S = 6;
       else if (tiles == 48 && K >= 4096) S = 9;
+      else if (tiles == 72) S = 7;
       else if (tiles == 80 && K >= 3072) S = 6;
+      else if (tiles == 144) S = 5;
+      else if (tiles == 160 && K >= 4096) S = 6, U = 2;
+      else if (tiles == 192 && K >= 5120) S = 4;
       else if (tiles == 96 && K >= 2048) S = 8;
       else if (tiles == 128 && K < 4096) S = 4, w = 8;
       else if (tiles == 128 && K == 4096) S = p->splitk, w = p->waves, U = p->unroll;
