@@ -613,9 +613,11 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
   // 26.3 / 28.4, K=16384 48.0 / 51.4), 144 x 5 (N=18432 K=4096 M=16 27.1 / 30.9, K=16384 95.8 / 105.1),
   // 160 x 6 with two units a step up to eight rows (N=20480 K=8192 M=4 53.4 / 55.5), 192 x 4 (N=24576
   // K=8192 M=16 65.9 / 69.3), and nine rows and more on 20 and 28 tiles with short K (N=2560 K=4096
-  // 8.8 / 9.5, N=3584 K=3072 8.8 / 9.3); 36, 56, 108 and 112 tiles measured level or behind.
-  if (splitk == 0 && p->kernel == FG_KERNEL_KN_MFMA && M >= 3 && M <= 16 && p->grid_y == 1 && kXccs > 1 &&
-      p->splitk > 1) {
+  // 8.8 / 9.5, N=3584 K=3072 8.8 / 9.3); 100 tiles x 7 (N=12800 K=6144 M=16 28.9 / 31.7, K=16384 M=8
+  // 67.6 / 72.0; x 4 below K = 4096) and 172 x 4 (N=22016 K=4096 M=8 32.0 / 34.1, K=8192 M=16 60.8 /
+  // 67.6, K=16384 119 / 133; x 3 = 516 workgroups is 3..9 % behind the unsplit plan).  12, 36, 56, 108,
+  // 112, 120, 216, 224 and 256 tiles measured level or behind.
+  if (splitk == 0 && p->kernel == FG_KERNEL_KN_MFMA && M >= 3 && M <= 16 && p->grid_y == 1 && kXccs > 1) {
     const int tiles = N / 128, units = K / 32;
     int S = 0, w = 4, U = 1;
     // (only the column counts the sweep covered: a split that fills the CUs unevenly costs far more
@@ -631,7 +633,9 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
       else if (tiles == 48 && K >= 4096) S = 9;
       else if (tiles == 72) S = 7;
       else if (tiles == 80 && K >= 3072) S = 6;
+      else if (tiles == 100) S = K >= 4096 ? 7 : 4;
       else if (tiles == 144) S = 5;
+      else if (tiles == 172) S = 4;
       else if (tiles == 192 && K >= 4096) S = 4;
       else if (tiles == 86) S = 5;
       else if (tiles == 96) S = 8;
@@ -645,8 +649,10 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
       else if (tiles == 48 && K >= 4096) S = 9;
       else if (tiles == 72) S = 7;
       else if (tiles == 80 && K >= 3072) S = 6;
+      else if (tiles == 100) S = K >= 4096 ? 7 : 4;
       else if (tiles == 144) S = 5;
       else if (tiles == 160 && K >= 4096) S = 6, U = 2;
+      else if (tiles == 172) S = 4;
       else if (tiles == 192 && K >= 5120) S = 4;
       else if (tiles == 96 && K >= 2048) S = 8;
       else if (tiles == 128 && K < 4096) S = 4, w = 8;

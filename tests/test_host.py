@@ -220,7 +220,10 @@ def test_plan_choices_that_were_measured():
                                # widths between the fitted ones: 48 tiles x 9, 80 x 6, 40 x 6, 96 x 8 for short K
                                (16, 6144, 8192, 9, 4, 1), (8, 6144, 4096, 9, 4, 1), (4, 10240, 8192, 6, 4, 1),
                                (16, 10240, 3072, 6, 4, 1), (16, 5120, 8192, 6, 4, 1), (8, 5120, 11008, 6, 4, 1),
-                               (8, 12288, 3072, 8, 4, 1)):
+                               (8, 12288, 3072, 8, 4, 1), (8, 9216, 4096, 7, 4, 1), (16, 18432, 4096, 5, 4, 1),
+                               (8, 22016, 4096, 4, 4, 1), (16, 12800, 8192, 7, 4, 1), (4, 12800, 2048, 4, 4, 1),
+                               (4, 20480, 8192, 6, 4, 2), (16, 24576, 8192, 4, 4, 1), (16, 2560, 4096, 8, 8, 1),
+                               (16, 3584, 3072, 8, 4, 1)):
         p = kn(M, N, K)
         assert (p.splitk, p.waves, p.unroll, p.fused) == (S, W, U, 3), (M, N, K, p.as_dict())
     # not where the sweep did not go (48 tiles x 6 splits would fill the CUs unevenly) or measured level
