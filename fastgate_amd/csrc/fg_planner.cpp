@@ -201,6 +201,9 @@ WideTile pick_wide_tile(int M, int N, int K, int splitk) {
     if (N % 64 == 0) {
       const int t64 = N / 64;
       offer(64, 8, 1, t64, M >= 5 && K >= 2048 && t64 < kCUs && 16 * t64 >= 13 * kCUs);
+      // ... already on 25/32 of them from K = 4096 on (N=12800 M=8: K=4096 20.1 -> 18.3 us, K=8192
+      // 38.1 -> 33.7; N=13056 M=16: K=4096 22.8 -> 19.9, K=12288 64.4 -> 53.6)
+      offer(64, 8, 1, t64, M >= 5 && K >= 4096 && t64 < kCUs && 32 * t64 >= 25 * kCUs);
       // ... and one 64-column workgroup on every CU for 12 rows and more (N=16384 M=16: K=5120
       // 30.1 -> 28.0 us, K=14336 73.4 -> 70.5)
       offer(64, 8, 1, t64, M >= 12 && K >= 5120 && t64 == kCUs);
@@ -230,6 +233,9 @@ WideTile pick_wide_tile(int M, int N, int K, int splitk) {
       const bool long_k = t32 <= 64 ? K / S >= 2048 : K / S >= 3072 && (S > 2 || K > 8192);
       offer(32, 8, S, wgs, long_k && M >= 9 && wgs <= kCUs && 4 * wgs >= 3 * kCUs);
     }
+    // (80 tiles split three ways already from 1365 k a split: N=2560 M=16 K=4096 8.0 -> 7.4 us, K=8192
+    // 12.7 -> 10.6; eight rows from K = 6144 on, 9.4 -> 8.3 and 10.8 -> 9.9)
+    offer(32, 8, 3, 3 * t32, t32 == 80 && ((M >= 9 && K >= 4096) || (M == 8 && K >= 6144)));
     if (N % 48 == 0) {
       // (N=3072 K=12288 M=16: 48 columns split 4 ways 16.4 us, 32 columns split 2 ways 17.9)
       const int t48 = N / 48;
@@ -265,7 +271,11 @@ WideTile pick_wide_tile(int M, int N, int K, int splitk) {
   }
   if (K >= 1024 && N % (2 * kCUs) == 0) {
     const int tw = N / (2 * kCUs);
-    offer(tw, 8, 1, 2 * kCUs, tw >= 20 && tw < 48 && tw % 16 != 0 && M >= 9, 0.15);
+    // (not over 64-column tiles on 25/32 of the CUs or more: N=12800 M=16 K=8192 25 columns 35.5 us,
+    // 64 columns 34.3; N=13824 K=4096 27 columns 21.3 / 20.4, K=8192 37.4 / 36.3; at K = 5120 the two
+    // are within 4 % either way: N=12800 M=9 23.4 / 24.4, N=13824 M=16 26.2 / 25.8.  Rows off 2 KB
+    // boundaries were not measured and keep the ragged form.)
+    offer(tw, 8, 1, 2 * kCUs, tw >= 20 && tw < 48 && tw % 16 != 0 && M >= 9 && (best.tile_n != 64 || odd_pitch), 0.15);
   }
   return best;
 }

@@ -165,6 +165,12 @@ def test_plan_choices_that_were_measured():
     assert nk(8, 12288, 10240).tile_n == 48
     assert nk(4, 9216, 4096).tile_n == 48 and nk(3, 9216, 8192).tile_n == 48
     assert nk(8, 14336, 4096).tile_n == 64 and nk(16, 16384, 8192).tile_n == 64
+    # 64 columns from 25/32 of the CUs on, also instead of ragged tiles two a CU (rows on 2 KB boundaries)
+    assert nk(8, 12800, 8192).tile_n == 64 and nk(16, 13056, 8192).tile_n == 64 and nk(16, 12800, 8192).tile_n == 64
+    assert nk(16, 13824, 4096).tile_n == 64 and nk(16, 13824, 5120).tile_n == 64 and nk(16, 13824, 11008).tile_n == 27
+    # 80 tiles of 32 columns split three ways
+    p = nk(16, 2560, 8192)
+    assert (p.tile_n, p.splitk, p.band) == (32, 3, 128) and nk(8, 2560, 6144).splitk == 3 and nk(8, 2560, 4096).splitk == 1
     assert nk(8, 14336, 2048).tile_n == 32 and nk(8, 14336, 2048).waves == 8
     assert nk(3, 5120, 8192).tile_n == 20
     p = nk(6, 12288, 4096)
