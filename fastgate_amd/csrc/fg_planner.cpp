@@ -362,13 +362,14 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
     }
   } else {
     const size_t weights = (size_t)N * K;
-    if (M <= 2 && (weights < ((size_t)1 << 27) || (weights < ((size_t)1 << 28) && (M == 1 || N <= 12288)))) {
+    if (M <= 2 && (weights < ((size_t)1 << 27) || (weights < ((size_t)1 << 28) && (M == 1 || N <= 12288 || (K <= 8192 && (N == 18432 || N == 22016)))))) {
       // One or two rows take the v_dot2 kernel up to 2^28 weights: its deep splits cost little now
       // that they complete through one atomic per element (M = 1, v_dot2 / MFMA kernel, us:
       // K=16384 N=8192 42.5 / 45.4, K=11008 N=12288 42.8 / 45.6, K=16384 N=12288 62.0 / 66.2,
       // K=8192 N=16384 42.2 / 44.0; at K = N = 16384 the two are level and the MFMA kernel stays;
       // two rows from 2^27 weights on only up to N = 12288: K=16384 N=12288 63.2 / 66.1, but
-      // K=16384 N=14336 76.0 / 74.0).
+      // K=16384 N=14336 76.0 / 74.0; two widths measured later with K = 8192 again: N=18432 49.3 / 52.0,
+      // N=22016 60.9 / 70.7).
       p->kernel = FG_KERNEL_KN_DOT2;
       p->m_block = M;
     } else {
@@ -674,6 +675,31 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
       fg_plan_t q = *p;
       q.splitk = S, q.waves = w, q.unroll = U, q.fused = 3;
       if (finish_plan(M, N, K, &q) == FG_OK && q.fused == 3) *p = q;
+    }
+  }
+  // One or two rows, [K,N] v_dot2 kernel, widths between the fitted ones with K = 4096 .. 8192: three or
+  // four 4-wave workgroups a CU, completed by atomics.  From a pass over 14 widths x K in {4096, 8192},
+  // the plan above beside every v_dot2 plan that fills 200..1100 wave slots (us, M = 1, this rule / the
+  // plan it replaces): N=6144 K=4096 10.8 / 11.4, K=8192 18.5 / 19.1; N=9216 K=8192 25.5 / 26.3; N=10240
+  // K=8192 28.1 / 28.8; N=11008 K=4096 16.8 / 17.4; N=12288 K=4096 18.4 / 19.1, K=8192 33.2 / 34.0;
+  // N=12800 K=4096 19.4 / 20.0, K=8192 35.0 / 36.3; N=18432 K=4096 25.7 / 27.3, K=8192 48.0 / 49.8;
+  // N=22016 K=4096 31.5 / 37.4, K=8192 59.3 / 61.0.  20, 28, 40, 56, 108 and 112 tiles measured within
+  // 2 % of their plans.
+  if (splitk == 0 && p->kernel == FG_KERNEL_KN_DOT2 && M <= 2 && K >= 4096 && K <= 8192) {
+    const int tiles = N / 128;
+    int S = 0, U = 1;
+    if (tiles == 48) S = 16, U = K <= 4096 ? 2 : 1;
+    else if (tiles == 72 && K >= 8192) S = 14;
+    else if (tiles == 80 && K >= 8192) S = 12, U = 2;
+    else if (tiles == 86 && K <= 4096) S = 5;
+    else if (tiles == 96) S = 10;
+    else if (tiles == 100) S = 10, U = K >= 8192 ? 2 : 1;
+    else if (tiles == 144) S = 7;
+    else if (tiles == 172) S = 4, U = 2;
+    if (S && (K / 32) / (4 * S * U) >= 1) {
+      fg_plan_t q = *p;
+      q.splitk = S, q.waves = 4, q.unroll = U, q.fused = 2;
+      if (finish_plan(M, N, K, &q) == FG_OK && q.fused == 2) *p = q;
     }
   }
   // Small problems (4 Mi weights or fewer, up to 16 rows).  Their kernels last 3 .. 7 us, a handful

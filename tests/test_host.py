@@ -202,6 +202,13 @@ def test_plan_choices_that_were_measured():
     assert kn(2, 16384, 8192).kernel == capi.FG_KERNEL_KN_MFMA
     assert kn(2, 14336, 16384).kernel == capi.FG_KERNEL_KN_MFMA
     assert kn(1, 16384, 16384).kernel == capi.FG_KERNEL_KN_MFMA
+    # widths between the fitted ones with K = 4096 .. 8192: three or four 4-wave workgroups a CU
+    for (M, N, K, S, U) in ((1, 6144, 4096, 16, 2), (2, 6144, 8192, 16, 1), (1, 9216, 8192, 14, 1), (1, 10240, 8192, 12, 2),
+                            (1, 11008, 4096, 5, 1), (2, 12288, 4096, 10, 1), (1, 12800, 8192, 10, 2), (1, 18432, 4096, 7, 1),
+                            (2, 18432, 8192, 7, 1), (1, 22016, 4096, 4, 2), (2, 22016, 8192, 4, 2)):
+        p = kn(M, N, K)
+        assert (p.kernel, p.splitk, p.waves, p.unroll, p.fused) == (capi.FG_KERNEL_KN_DOT2, S, 4, U, 2), (M, N, K, p.as_dict())
+    assert kn(1, 9216, 4096).splitk == 7 and kn(1, 14336, 4096).splitk == 4 and kn(1, 9216, 11008).splitk != 14
     assert kn(1, 28672, 8192).kernel == capi.FG_KERNEL_KN_DOT2
     assert kn(1, 8192, 8192).kernel == capi.FG_KERNEL_KN_DOT2
     for (M, N, K, S) in ((1, 16384, 8192, 8), (1, 8192, 16384, 16), (2, 12288, 16384, 10)):
@@ -249,7 +256,7 @@ def test_plan_choices_that_were_measured():
     p = kn(1, 4096, 4096)
     assert (p.splitk, p.waves) == (8, 8)           # two units a wave only: stays one 8-wave workgroup a CU
     p = kn(2, 12288, 4096)
-    assert (p.splitk, p.waves) == (2, 8)           # 384 workgroups would fill the CUs unevenly
+    assert (p.splitk, p.waves) == (10, 4)          # 19.1 us; two splits of 8 waves 19.7 (four would fill the CUs unevenly)
     # small problems (4 Mi weights or fewer), fitted to per-launch times inside a replayed graph:
     # [K,N] v_dot2 on two rows a workgroup with one unit a wave, the MFMA kernel with flags for nine
     # rows and more beyond 1 Mi weights; [N,K] eight waves, narrow outputs split four ways
