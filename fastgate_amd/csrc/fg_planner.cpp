@@ -543,11 +543,14 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
       // 8-wave workgroup, where that lands on 448..512 workgroups and leaves every wave four units
       // (M=1, twice the split with 4 waves / 8 waves: K=14336 N=8192 37.3 / 40.6 us, K=11008 N=8192
       // 30.4 / 32.4, K=5120 N=16384 28.2 / 29.8; M=2: K=11008 N=4096 17.6 / 18.5, K=4096 N=8192
-      // 14.1 / 14.7)
+      // 14.1 / 14.7); two units a wave are enough (five alternating runs each, minimum: K = N = 4096
+      // M=1 8.03 / 8.29, M=2 8.31 / 8.62; K=5120 N=4096 9.11 / 9.89; K=6144 N=4096 10.35 / 10.82;
+      // K=3072 N=8192 10.53 / 11.09; K=5120 N=3072 7.98 / 8.18; one and a half are not: K=3072
+      // N=4096 7.96 / 7.88)
       {
         const int twice = 2 * tiles * p->splitk;
         if (splitk == 0 && M <= 2 && p->kernel == FG_KERNEL_KN_DOT2 && p->waves == 8 &&
-            p->splitk <= 8 && twice >= 448 && twice <= 2 * kCUs && items / (4 * 2 * p->splitk) >= 4) {
+            p->splitk <= 12 && twice >= 448 && twice <= 2 * kCUs && items / (4 * 2 * p->splitk) >= 2) {
           p->splitk *= 2;
           p->waves = 4;
         }

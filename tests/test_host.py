@@ -254,7 +254,9 @@ def test_plan_choices_that_were_measured():
         p = kn(1, N, K)
         assert (p.splitk, p.waves) == (S, 4), (N, K, p.as_dict())
     p = kn(1, 4096, 4096)
-    assert (p.splitk, p.waves) == (8, 8)           # two units a wave only: stays one 8-wave workgroup a CU
+    assert (p.splitk, p.waves) == (16, 4)          # two units a wave are enough: 8.03 us against 8.29
+    p = kn(1, 4096, 3072)
+    assert (p.splitk, p.waves) == (8, 8)           # one and a half are not
     p = kn(2, 12288, 4096)
     assert (p.splitk, p.waves) == (10, 4)          # 19.1 us; two splits of 8 waves 19.7 (four would fill the CUs unevenly)
     # small problems (4 Mi weights or fewer), fitted to per-launch times inside a replayed graph:
