@@ -171,7 +171,7 @@ __global__ __launch_bounds__(512) void w8a16_kernel(const int8_t* __restrict__ W
 }
 
 // ---------------------------------------------------------------------------------------
-// One activation row (the GEMV proper), int8 and int4 weights.
+// One activation row (the GEMV proper), int8 and int4 weights; MR = 2 rows for int4.
 //  * Lanes own 8 activations each, not 16 weight bytes: a chunk is UD 16-byte units of x a lane
 //    (unit 64 d + lane, d < UD), so every x load is one contiguous KB per wave, and the weights
 //    under a unit are 8 bytes (int8) or 4 bytes (int4) per row: UD 8- or 4-byte loads a row,
@@ -194,7 +194,7 @@ __global__ __launch_bounds__(512) void w8a16_kernel(const int8_t* __restrict__ W
 // Replaces the device side of gemv_quantized_int8 (backend/cuda/hk/fastgemv.cuh:316-389) and of
 // gemv_quantized_int4 (:394-495, defined there but never launched) for one row.
 // ---------------------------------------------------------------------------------------
-template <int BITS, int RN, int NWV, int UD>
+template <int BITS, int RN, int NWV, int UD, int MR>
 __global__ __launch_bounds__(64 * NWV) void wq_m1_kernel(const uint8_t* __restrict__ Wq,
                                                          const half_t* __restrict__ X,
                                                          const half_t* __restrict__ scale,
@@ -202,13 +202,14 @@ __global__ __launch_bounds__(64 * NWV) void wq_m1_kernel(const uint8_t* __restri
                                                          half_t* __restrict__ Y, int N, int K) {
   constexpr int WB = BITS == 4 ? 4 : 8;  // weight bytes under one 16-byte unit of x
   typedef uint32_t wreg_t __attribute__((ext_vector_type(WB / 4)));
-  __shared__ float red[NWV * 4][RN + 1];
+  constexpr int RC = RN + 1;             // columns of the reduction table per activation row: RN sums and Σx
+  __shared__ float red[NWV * 4][MR * RC];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: addresses stay scalar
   const int n0 = blockIdx.x * RN;
   const size_t rowb = BITS == 4 ? (size_t)K >> 1 : (size_t)K;
-  static_assert(RN <= 64, "one output per thread of the first wave");
-  const uint32_t scale_raw = scale_fetch(scale, n0 + (int)threadIdx.x, threadIdx.x < RN);
+  static_assert(MR * RN <= 64, "one output per thread of the first wave");
+  const uint32_t scale_raw = scale_fetch(scale, n0 + (int)threadIdx.x % RN, threadIdx.x < MR * RN);
   // the constant that comes out with Σx: the zero point, and int8's + 128
   const float zp = BITS == 4 ? zero_point : zero_point + 128.f;
   const bool use_xsum = zp != 0.f;
@@ -216,16 +217,20 @@ __global__ __launch_bounds__(64 * NWV) void wq_m1_kernel(const uint8_t* __restri
   const uint32_t lane_w = lane * WB, lane_x = lane * 16;
   const half2_t ones = {static_cast<half_t>(1.f), static_cast<half_t>(1.f)};
   const u32x4 zero = {0u, 0u, 0u, 0u};
-  float acc0[RN], acc1[RN];
-  float xsum = 0.f;
+  float acc0[MR][RN], acc1[MR][RN];
+  float xsum[MR];
 #pragma unroll
-  for (int r = 0; r < RN; ++r) acc0[r] = acc1[r] = 0.f;
+  for (int m = 0; m < MR; ++m) {
+    xsum[m] = 0.f;
+#pragma unroll
+    for (int r = 0; r < RN; ++r) acc0[m][r] = acc1[m][r] = 0.f;
+  }
 
   const int nunits = K >> 3;
   const int nchunks = (nunits + 64 * UD - 1) / (64 * UD);
   for (int ch = wave; ch < nchunks; ch += NWV) {
     wreg_t wr[RN][UD];
-    u32x4 xv[UD];
+    u32x4 xv[MR][UD];
     bool ok[UD];
 #pragma unroll
     for (int d = 0; d < UD; ++d) ok[d] = ch * (64 * UD) + 64 * d + lane < nunits;
@@ -239,23 +244,31 @@ __global__ __launch_bounds__(64 * NWV) void wq_m1_kernel(const uint8_t* __restri
                          : none;
       }
 #pragma unroll
-    for (int d = 0; d < UD; ++d)
-      xv[d] = ok[d] ? load16<false>(reinterpret_cast<const uint8_t*>(X) + (size_t)(ch * (64 * UD) + 64 * d) * 16 + lane_x) : zero;
-    if (use_xsum) {
+    for (int m = 0; m < MR; ++m)
 #pragma unroll
       for (int d = 0; d < UD; ++d)
+        xv[m][d] = ok[d] ? load16<false>(reinterpret_cast<const uint8_t*>(X + (size_t)m * K) +
+                                         (size_t)(ch * (64 * UD) + 64 * d) * 16 + lane_x)
+                         : zero;
+    if (use_xsum) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) xsum = __builtin_amdgcn_fdot2(as_half2(xv[d][i]), ones, xsum, false);
+      for (int m = 0; m < MR; ++m)
+#pragma unroll
+        for (int d = 0; d < UD; ++d)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) xsum[m] = __builtin_amdgcn_fdot2(as_half2(xv[m][d][i]), ones, xsum[m], false);
     }
     if (BITS == 4) {  // (x_j, x_{j+4}): the halves that meet nibbles j and j + 4 of a register
 #pragma unroll
-      for (int d = 0; d < UD; ++d) {
-        const u32x4 t = xv[d];
-        xv[d].x = __builtin_amdgcn_perm(t.z, t.x, 0x05040100u);
-        xv[d].y = __builtin_amdgcn_perm(t.z, t.x, 0x07060302u);
-        xv[d].z = __builtin_amdgcn_perm(t.w, t.y, 0x05040100u);
-        xv[d].w = __builtin_amdgcn_perm(t.w, t.y, 0x07060302u);
-      }
+      for (int m = 0; m < MR; ++m)
+#pragma unroll
+        for (int d = 0; d < UD; ++d) {
+          const u32x4 t = xv[m][d];
+          xv[m][d].x = __builtin_amdgcn_perm(t.z, t.x, 0x05040100u);
+          xv[m][d].y = __builtin_amdgcn_perm(t.z, t.x, 0x07060302u);
+          xv[m][d].z = __builtin_amdgcn_perm(t.w, t.y, 0x05040100u);
+          xv[m][d].w = __builtin_amdgcn_perm(t.w, t.y, 0x07060302u);
+        }
     }
 #pragma unroll
     for (int r = 0; r < RN; ++r)
@@ -263,41 +276,51 @@ __global__ __launch_bounds__(64 * NWV) void wq_m1_kernel(const uint8_t* __restri
       for (int d = 0; d < UD; ++d) {
         if constexpr (BITS == 4) {
           const uint32_t w = wr[r][d][0], w8 = w >> 8;  // nibbles 0,4 | 1,5 | 2,6 | 3,7
-          acc0[r] = __builtin_amdgcn_fdot2(as_half2(w & 0x000F000Fu), as_half2(xv[d].x), acc0[r], false);
-          acc1[r] = __builtin_amdgcn_fdot2(as_half2(w & 0x00F000F0u), as_half2(xv[d].y), acc1[r], false);
-          acc0[r] = __builtin_amdgcn_fdot2(as_half2(w8 & 0x000F000Fu), as_half2(xv[d].z), acc0[r], false);
-          acc1[r] = __builtin_amdgcn_fdot2(as_half2(w8 & 0x00F000F0u), as_half2(xv[d].w), acc1[r], false);
+          const uint32_t n04 = w & 0x000F000Fu, n15 = w & 0x00F000F0u, n26 = w8 & 0x000F000Fu, n37 = w8 & 0x00F000F0u;
+#pragma unroll
+          for (int m = 0; m < MR; ++m) {
+            acc0[m][r] = __builtin_amdgcn_fdot2(as_half2(n04), as_half2(xv[m][d].x), acc0[m][r], false);
+            acc1[m][r] = __builtin_amdgcn_fdot2(as_half2(n15), as_half2(xv[m][d].y), acc1[m][r], false);
+            acc0[m][r] = __builtin_amdgcn_fdot2(as_half2(n26), as_half2(xv[m][d].z), acc0[m][r], false);
+            acc1[m][r] = __builtin_amdgcn_fdot2(as_half2(n37), as_half2(xv[m][d].w), acc1[m][r], false);
+          }
         } else {
 #pragma unroll
           for (int h = 0; h < 2; ++h) {
             const uint32_t t = wr[r][d][h] ^ 0x80808080u;  // w + 128 as unsigned bytes
             const uint32_t b01 = __builtin_amdgcn_perm(0u, t, 0x04010400u);  // halves (b0, b1)
             const uint32_t b23 = __builtin_amdgcn_perm(0u, t, 0x04030402u);  // halves (b2, b3)
-            acc0[r] = __builtin_amdgcn_fdot2(as_half2(b01), as_half2(xv[d][2 * h]), acc0[r], false);
-            acc1[r] = __builtin_amdgcn_fdot2(as_half2(b23), as_half2(xv[d][2 * h + 1]), acc1[r], false);
+#pragma unroll
+            for (int m = 0; m < MR; ++m) {
+              acc0[m][r] = __builtin_amdgcn_fdot2(as_half2(b01), as_half2(xv[m][d][2 * h]), acc0[m][r], false);
+              acc1[m][r] = __builtin_amdgcn_fdot2(as_half2(b23), as_half2(xv[m][d][2 * h + 1]), acc1[m][r], false);
+            }
           }
         }
       }
   }
 
 #pragma unroll
-  for (int r = 0; r < RN; ++r) {
-    // int4: acc1 holds the nibbles that sat 4 bits up
-    const float a = BITS == 4 ? acc0[r] * 16777216.f + acc1[r] * 1048576.f : (acc0[r] + acc1[r]) * 16777216.f;
-    const float v = row16_allreduce(a);
-    if ((lane & 15) == 0) red[wave * 4 + (lane >> 4)][r] = v;
-  }
-  {
-    const float xs = row16_allreduce(xsum);
-    if ((lane & 15) == 0) red[wave * 4 + (lane >> 4)][RN] = xs;
+  for (int m = 0; m < MR; ++m) {
+#pragma unroll
+    for (int r = 0; r < RN; ++r) {
+      // int4: acc1 holds the nibbles that sat 4 bits up
+      const float a = BITS == 4 ? acc0[m][r] * 16777216.f + acc1[m][r] * 1048576.f
+                                : (acc0[m][r] + acc1[m][r]) * 16777216.f;
+      const float v = row16_allreduce(a);
+      if ((lane & 15) == 0) red[wave * 4 + (lane >> 4)][m * RC + r] = v;
+    }
+    const float xs = row16_allreduce(xsum[m]);
+    if ((lane & 15) == 0) red[wave * 4 + (lane >> 4)][m * RC + RN] = xs;
   }
   __syncthreads();
-  if (threadIdx.x < RN) {
-    const float sum = lds_sum<NWV * 4>(&red[0][threadIdx.x], RN + 1, NWV * 4);
-    const float xs = lds_sum<NWV * 4>(&red[0][RN], RN + 1, NWV * 4);
+  if (threadIdx.x < MR * RN) {
+    const int m = threadIdx.x / RN, r = threadIdx.x % RN;
+    const float sum = lds_sum<NWV * 4>(&red[0][m * RC + r], MR * RC, NWV * 4);
+    const float xs = lds_sum<NWV * 4>(&red[0][m * RC + RN], MR * RC, NWV * 4);
     float v = sum - zp * xs;
-    if (not_finite(xs)) v = elementwise_dot<BITS>(Wt + (size_t)threadIdx.x * rowb, X, K, zero_point);
-    Y[n0 + threadIdx.x] = static_cast<half_t>(v * (scalar_scale * scale_value(scale_raw)));
+    if (not_finite(xs)) v = elementwise_dot<BITS>(Wt + (size_t)r * rowb, X + (size_t)m * K, K, zero_point);
+    Y[(size_t)m * N + n0 + r] = static_cast<half_t>(v * (scalar_scale * scale_value(scale_raw)));
   }
 }
 
@@ -661,7 +684,11 @@ static int i8_waves(int K) {
 // 4096 x 14336 10.1 -> 8.1, 16384 x 16384 27.9 -> 24.5; int8 8192 x 8192 13.3 -> 12.1,
 // 4096 x 4096 5.7 -> 5.25, 28672 x 4096 20.8 -> 18.8, 4096 x 14336 12.6 -> 11.4, 16384 x 16384
 // 41.9 -> 40.6.  int8 with four units a lane (2 KB of a row per wave): 8192 x 8192 13.0.
-template <int BITS>
+// Two activation rows of int4 (MR = 2) against the row-load MFMA kernel: 8192 x 8192 11.4 -> 10.6,
+// 4096 x 4096 5.7 -> 5.0, 4096 x 14336 11.6 -> 10.7, 28672 x 4096 level; the second row costs 2 us at
+// 8192 x 8192 because its x traffic (64 MiB from L2) is twice the weights'; eight weight rows a
+// workgroup to halve it lose more in occupancy (11.9).  int8 keeps its row-load kernel for two rows.
+template <int BITS, int MR>
 static void launch_wq_m1(const W8A16Args& a, hipStream_t s) {
   auto* Wq = static_cast<const uint8_t*>(a.Wq);
   auto* X = static_cast<const half_t*>(a.x);
@@ -670,8 +697,8 @@ static void launch_wq_m1(const W8A16Args& a, hipStream_t s) {
   constexpr int UD = BITS == 4 ? 4 : 2;
   const int chunks = (a.K + 512 * UD - 1) / (512 * UD);
   const bool small = (size_t)a.N * a.K * BITS / 8 <= (8u << 20);
-#define FG_WQ_M1(RN, NWV)                                                                     \
-  hipLaunchKernelGGL((wq_m1_kernel<BITS, RN, NWV, UD>), dim3(a.N / RN), dim3(64 * NWV), 0, s, Wq, \
+#define FG_WQ_M1(RN, NWV)                                                                         \
+  hipLaunchKernelGGL((wq_m1_kernel<BITS, RN, NWV, UD, MR>), dim3(a.N / RN), dim3(64 * NWV), 0, s, Wq, \
                      X, sc, a.scalar_scale, a.zero_point, Y, a.N, a.K)
 #define FG_WQ_M1_ROWS(NWV) \
   if (small) FG_WQ_M1(2, NWV); else FG_WQ_M1(4, NWV)
@@ -717,7 +744,7 @@ bool launch_w8a16(const W8A16Args& a, hipStream_t s) {
   hipLaunchKernelGGL((w8a16_r_kernel<XR, 8, BW, CB>), dim3(a.N / (16 * CB)), dim3(512), 0, s, Wq, \
                      X, sc, a.scalar_scale, a.zero_point, Y, a.M, a.N, a.K)
   if (a.M == 1) {
-    launch_wq_m1<8>(a, s);
+    launch_wq_m1<8, 1>(a, s);
   } else if (a.M <= 4 && (a.N <= 2048 || (a.M == 2 && a.N <= 6144))) {
     // narrow outputs leave the 16-column tiles of the row-load kernel on half the CUs or fewer: lanes
     // along K, four weight rows a workgroup (N=2048 K=8192: M=2 8.8 -> 6.0 us, M=4 9.0 -> 7.3;
@@ -755,10 +782,9 @@ bool launch_w4a16(const W8A16Args& a, hipStream_t s) {
   auto* Y = static_cast<half_t*>(a.y);
   if (a.M < 1 || a.M > 4) return false;
   if (a.M == 1) {
-    launch_wq_m1<4>(a, s);
+    launch_wq_m1<4, 1>(a, s);
   } else if (a.M == 2) {
-    hipLaunchKernelGGL((w4a16_r_kernel<2>), dim3(a.N / 16), dim3(512), 0, s, Wq, X, sc, a.scalar_scale,
-                       a.zero_point, Y, a.M, a.N, a.K);
+    launch_wq_m1<4, 2>(a, s);
   } else {
     hipLaunchKernelGGL((w4a16_r_kernel<4>), dim3(a.N / 16), dim3(512), 0, s, Wq, X, sc, a.scalar_scale,
                        a.zero_point, Y, a.M, a.N, a.K);
