@@ -1,12 +1,9 @@
-// int8-weight GEMV kernels, weights [N,K] row-major (16 weights per 16-byte load).
+// int8- and int4-weight GEMV kernels, weights [N,K] row-major.
 //
-//  * w8a16: fp16 activations.  Four int8 of a register become two half2 without leaving the
-//    integer pipe's cheap ops: flip the sign bit (w+128 as unsigned), splice each byte under
-//    the exponent 0x64 (fp16 value 1024 + byte), subtract 1152 with v_pk_add_f16 -> the exact
-//    integer as fp16, then v_dot2_f32_f16 against the activations (fp32 accumulation).  The
-//    per-output-channel scale and the zero point are applied once per output.  The one-row
-//    kernel and the row-load kernel take a shorter way (the bytes as fp16 subnormals, see
-//    wq_m1_kernel); this form remains in w8a16_kernel, for 2..4 rows against narrow outputs.
+//  * w8a16 / w4a16: fp16 activations.  The integers reach v_dot2_f32_f16 or the MFMA as fp16
+//    subnormals (a byte or nibble in the low mantissa bits under a zero exponent is that number
+//    times 2^-24, exactly; see wq_m1_kernel), products and sums are fp32, and the per-output-channel
+//    scale and the zero point are applied once per output.
 //  * i8i8: int8 activations, v_dot4_i32_i8, exact int32 result.
 //
 // Replaces the device side of gemv_quantized_int8 (backend/cuda/hk/fastgemv.cuh:316-389,
@@ -15,13 +12,6 @@
 #include "fg_internal.h"
 
 namespace fg {
-
-__device__ __forceinline__ void i8x4_to_half2x2(uint32_t w, half2_t& lo, half2_t& hi) {
-  const uint32_t t = w ^ 0x80808080u;
-  const half2_t bias = {static_cast<half_t>(1152.f), static_cast<half_t>(1152.f)};
-  lo = as_half2(__builtin_amdgcn_perm(0x64646464u, t, 0x04010400u)) - bias;
-  hi = as_half2(__builtin_amdgcn_perm(0x64646464u, t, 0x04030402u)) - bias;
-}
 
 // Per-channel scale of the output a thread writes at the end, fetched ahead of the weight stream
 // as raw bits.  Converting it at the point of the load would make the wave wait for this cold
@@ -63,115 +53,9 @@ __device__ float elementwise_dot(const uint8_t* __restrict__ wrow, const half_t*
   return s;
 }
 
-template <int MB, int RN, int U>
-__global__ __launch_bounds__(512) void w8a16_kernel(const int8_t* __restrict__ Wq,
-                                                    const half_t* __restrict__ X,
-                                                    const half_t* __restrict__ scale,
-                                                    float scalar_scale, float zero_point,
-                                                    half_t* __restrict__ Y, int M, int N, int K) {
-  __shared__ float red[32][RN * MB];
-  __shared__ float redx[32][MB];
-  const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
-  const int nw = blockDim.x >> 6;
-  const int n0 = blockIdx.x * RN;
-  const int nq = K >> 4;  // 16-weight chunks per row
-  const bool use_zp = zero_point != 0.f;
-  // scale of the output this thread writes at the end, fetched ahead of the weight stream (a load
-  // issued after the last barrier would add its whole latency to the workgroup's life)
-  static_assert(RN * MB <= 64, "one output per thread of the first wave");
-  const uint32_t scale_raw = scale_fetch(scale, n0 + (int)threadIdx.x % RN, threadIdx.x < RN * MB);
-
-  float acc[RN][MB];
-  float xsum[MB];
-#pragma unroll
-  for (int m = 0; m < MB; ++m) {
-    xsum[m] = 0.f;
-#pragma unroll
-    for (int r = 0; r < RN; ++r) acc[r][m] = 0.f;
-  }
-  const int8_t* Wt = Wq + (size_t)n0 * K;
-  const u32x4 zero = {0u, 0u, 0u, 0u};
-  const half2_t ones = {static_cast<half_t>(1.f), static_cast<half_t>(1.f)};
-
-  const int nsteps = (nq + nw * (64 * U) - 1) / (nw * (64 * U));
-  int step = stagger_start(nsteps, 0);
-  for (int it = 0; it < nsteps; ++it) {
-    const int q0 = (step * nw + wave) * (64 * U);
-    step = step + 1 == nsteps ? 0 : step + 1;
-    u32x4 wr[U][RN];
-    u32x4 xr[U][MB][2];
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int q = q0 + u * 64 + lane;
-      const bool ok = q < nq;
-#pragma unroll
-      for (int r = 0; r < RN; ++r)
-        wr[u][r] = ok ? load16<true>(Wt + (size_t)r * K + (size_t)q * 16) : zero;
-#pragma unroll
-      for (int m = 0; m < MB; ++m) {
-        const bool okm = ok && m < M;
-        const half_t* xp = X + (size_t)m * K + (size_t)q * 16;
-        xr[u][m][0] = okm ? load16<false>(xp) : zero;
-        xr[u][m][1] = okm ? load16<false>(xp + 8) : zero;
-      }
-    }
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-#pragma unroll
-      for (int r = 0; r < RN; ++r) {
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-          half2_t lo, hi;
-          i8x4_to_half2x2(wr[u][r][c], lo, hi);
-#pragma unroll
-          for (int m = 0; m < MB; ++m) {
-            const u32x4 xv = xr[u][m][c >> 1];
-            const uint32_t x0 = (c & 1) ? xv.z : xv.x, x1 = (c & 1) ? xv.w : xv.y;
-            acc[r][m] = __builtin_amdgcn_fdot2(lo, as_half2(x0), acc[r][m], false);
-            acc[r][m] = __builtin_amdgcn_fdot2(hi, as_half2(x1), acc[r][m], false);
-          }
-        }
-      }
-      if (use_zp) {
-#pragma unroll
-        for (int m = 0; m < MB; ++m)
-#pragma unroll
-          for (int h = 0; h < 2; ++h)
-#pragma unroll
-            for (int c = 0; c < 4; ++c)
-              xsum[m] = __builtin_amdgcn_fdot2(as_half2(xr[u][m][h][c]), ones, xsum[m], false);
-      }
-    }
-  }
-
-#pragma unroll
-  for (int m = 0; m < MB; ++m) {
-#pragma unroll
-    for (int r = 0; r < RN; ++r) {
-      const float v = row16_allreduce(acc[r][m]);
-      if ((lane & 15) == 0) red[wave * 4 + (lane >> 4)][r * MB + m] = v;
-    }
-    const float xs = row16_allreduce(xsum[m]);
-    if ((lane & 15) == 0) redx[wave * 4 + (lane >> 4)][m] = xs;
-  }
-  __syncthreads();
-  for (int t = threadIdx.x; t < RN * MB; t += blockDim.x) {
-    const int m = t / RN, r = t % RN;
-    const float sum = lds_sum<32>(&red[0][r * MB + m], RN * MB, nw * 4);
-    const float xs = lds_sum<32>(&redx[0][m], MB, nw * 4);
-    const int n = n0 + r;
-    if (m < M) {
-      float v = sum - zero_point * xs;
-      if (not_finite(xs))
-        v = elementwise_dot<8>(reinterpret_cast<const uint8_t*>(Wq) + (size_t)n * K, X + (size_t)m * K, K, zero_point);
-      Y[(size_t)m * N + n] = static_cast<half_t>(v * (scalar_scale * scale_value(scale_raw)));
-    }
-  }
-}
-
 // ---------------------------------------------------------------------------------------
-// One activation row (the GEMV proper), int8 and int4 weights; MR = 2 rows for int4.
+// MR activation rows: one (the GEMV proper), and up to four where the launchers say so; int8 and int4
+// weights.
 //  * Lanes own 8 activations each, not 16 weight bytes: a chunk is UD 16-byte units of x a lane
 //    (unit 64 d + lane, d < UD), so every x load is one contiguous KB per wave, and the weights
 //    under a unit are 8 bytes (int8) or 4 bytes (int4) per row: UD 8- or 4-byte loads a row,
@@ -668,8 +552,8 @@ __global__ __launch_bounds__(512) void w4a16_r_kernel(const uint8_t* __restrict_
 }
 
 // ---------------------------------------------------------------------------------------
-// Host launchers.  Rows per workgroup: 8 when that still yields >= 512 workgroups, else 4.
-// Waves per workgroup: as many (<= 4) as the row has 1 KB pieces.
+// Host launchers.  The integer-dot kernel: rows per workgroup 8 when that still yields >= 512
+// workgroups, else 4; waves per workgroup as many (<= 4) as the row has 1 KB pieces.
 // ---------------------------------------------------------------------------------------
 static int i8_waves(int K) {
   const int pieces = (K / 16 + 63) / 64;
@@ -710,9 +594,8 @@ static void launch_wq_m1(const W8A16Args& a, hipStream_t s) {
 #undef FG_WQ_M1
 }
 
-// Measured (us per call; lanes-along-K kernel / row-load kernel on 256-byte bands):
-//   K = N = 8192   M=1 12.6 / 14.3   M=2 15.1 / 14.2   M=4 21.1 / 14.9   M=8 32.9 / 17.2
-//   K = N = 16384  M=1 41.2 / 44.8   M=8  -   / 49.7
+// An earlier kernel with lanes along K (16 weight bytes a lane) against the row-load kernel on 256-byte
+// bands, us per call: K = N = 8192 M=1 12.6 / 14.3, M=2 15.1 / 14.2, M=4 21.1 / 14.9, M=8 32.9 / 17.2.
 // The row-load kernel exists with 8 waves only.
 bool launch_w8a16(const W8A16Args& a, hipStream_t s) {
   auto* Wq = static_cast<const int8_t*>(a.Wq);
@@ -743,19 +626,23 @@ bool launch_w8a16(const W8A16Args& a, hipStream_t s) {
 #define FG_W8A16_R(XR, BW, CB)                                                                    \
   hipLaunchKernelGGL((w8a16_r_kernel<XR, 8, BW, CB>), dim3(a.N / (16 * CB)), dim3(512), 0, s, Wq, \
                      X, sc, a.scalar_scale, a.zero_point, Y, a.M, a.N, a.K)
+  // Two rows run the lanes-over-x kernel on two rows -- except where the 16-column tiles of the row-load
+  // kernel fill the CUs evenly (us, two-row kernel / row-load kernel: N=4096 K=4096 6.0 / 7.1, K=14336
+  // 13.2 / 14.7; N=11008 K=4096 10.8 / 12.5; N=12288 K=3072 9.2 / 10.9, K=8192 20.0 / 20.8; N=28672 K=4096
+  // 22.0 / 24.0; N=2048 K=8192 6.1 / 6.8; N=1024 K=4096 3.7 / 4.5; but N=8192 K=8192 14.6 / 13.5, K=11008
+  // 19.0 / 16.9, K=4096 8.9 / 8.6; N=16384 K=8192 25.5 / 23.3; N=13824 K=5120 16.1 / 15.5; N=14336 K=4096
+  // 12.9 / 12.7).  Three and four rows only against narrow outputs, which leave the row-load kernel on
+  // half the CUs or fewer (M=4: N=1024 K=4096 4.5 / 5.3, N=2048 K=2048 4.3 / 5.6, K=8192 7.8 / 8.1;
+  // N=4096 K=4096 7.6 / 6.6 and N=8192 K=8192 23.2 / 13.7 the other way).
+  const bool even_tiles = a.N % 8192 == 0 || (a.N >= 13312 && a.N <= 14336);
   if (a.M == 1) {
     launch_wq_m1<8, 1>(a, s);
-  } else if (a.M <= 4 && (a.N <= 2048 || (a.M == 2 && a.N <= 6144))) {
-    // narrow outputs leave the 16-column tiles of the row-load kernel on half the CUs or fewer: lanes
-    // along K, four weight rows a workgroup (N=2048 K=8192: M=2 8.8 -> 6.0 us, M=4 9.0 -> 7.3;
-    // N=1024 K=4096 M=4 5.8 -> 4.4; N=4096 K=8192 M=4 9.6 -> 11.6 the other way; two rows up to
-    // N = 6144: N=4096 K=8192 9.5 -> 9.1, N=8192 K=4096 8.6 -> 9.0)
-    if (a.M <= 2)
-      hipLaunchKernelGGL((w8a16_kernel<2, 4, 1>), dim3(a.N / 4), dim3(64 * i8_waves(a.K)), 0, s, Wq, X,
-                         sc, a.scalar_scale, a.zero_point, Y, a.M, a.N, a.K);
-    else
-      hipLaunchKernelGGL((w8a16_kernel<4, 4, 1>), dim3(a.N / 4), dim3(64 * i8_waves(a.K)), 0, s, Wq, X,
-                         sc, a.scalar_scale, a.zero_point, Y, a.M, a.N, a.K);
+  } else if (a.M == 2 && !even_tiles) {
+    launch_wq_m1<8, 2>(a, s);
+  } else if (a.M == 3 && a.N <= 2048) {
+    launch_wq_m1<8, 3>(a, s);
+  } else if (a.M == 4 && a.N <= 2048) {
+    launch_wq_m1<8, 4>(a, s);
   } else if (a.M <= 4) {  // 2 rows take the 4-row strip too: K=14336 N=4096 M=2 13.1 us
     if (wide) FG_W8A16_R(4, 128, 2);
     else if (bw256) FG_W8A16_R(4, 256, 1);
