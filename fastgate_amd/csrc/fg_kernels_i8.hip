@@ -672,6 +672,12 @@ bool launch_w4a16(const W8A16Args& a, hipStream_t s) {
     launch_wq_m1<4, 1>(a, s);
   } else if (a.M == 2) {
     launch_wq_m1<4, 2>(a, s);
+  } else if (a.N <= 2048) {
+    // narrow outputs leave the 16-column tiles of the row-load kernel on half the CUs or fewer (M=4, us,
+    // lanes-over-x / row-load: N=1024 K=4096 4.6 / 5.3, K=8192 5.3 / 7.4; N=2048 K=2048 4.3 / 5.0, K=8192
+    // 7.5 / 7.7; N=3072 K=3072 5.7 / 5.3 and N=4096 K=4096 6.6 / 5.7 the other way)
+    if (a.M == 3) launch_wq_m1<4, 3>(a, s);
+    else launch_wq_m1<4, 4>(a, s);
   } else {
     hipLaunchKernelGGL((w4a16_r_kernel<4>), dim3(a.N / 16), dim3(512), 0, s, Wq, X, sc, a.scalar_scale,
                        a.zero_point, Y, a.M, a.N, a.K);
