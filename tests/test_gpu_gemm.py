@@ -430,3 +430,33 @@ def test_planner_splits_narrow_kn_outputs(device, M):
         ref, _ = oracle.gemm_f16(A.numpy(), W.numpy(), KN)
         got, _ = _run(A, W, KN, device)
         assert_close_f16(got, ref, "auto plan M=%d N=%d K=%d" % (M, N, K))
+
+
+@pytest.mark.parametrize("M,N,K,layout,want", [
+    # [K,N], flags in one L2: (split, waves, units a step)
+    (8, 9216, 4096, KN, (7, 4, 1)), (16, 18432, 2048, KN, (5, 4, 1)), (5, 22016, 4096, KN, (4, 4, 1)),
+    (16, 12800, 4096, KN, (7, 4, 1)), (4, 20480, 4096, KN, (6, 4, 2)), (16, 24576, 4096, KN, (4, 4, 1)),
+    (16, 2560, 4096, KN, (8, 8, 1)), (16, 3584, 3072, KN, (8, 4, 1)), (8, 6144, 4096, KN, (9, 4, 1)),
+    (16, 10240, 3072, KN, (6, 4, 1)), (16, 5120, 8192, KN, (6, 4, 1)), (8, 12288, 2048, KN, (8, 4, 1)),
+    (3, 8192, 3072, KN, (8, 4, 1)),
+    # [K,N], one or two rows, atomics
+    (1, 6144, 4096, KN, (16, 4, 2)), (2, 18432, 4096, KN, (7, 4, 1)), (1, 22016, 4096, KN, (4, 4, 2)),
+    (2, 4096, 4096, KN, (16, 4, 1)),
+    # [N,K]: (tile, split, band)
+    (16, 2560, 8192, NK, (32, 3, 128)), (8, 12800, 4096, NK, (64, 1, 128)), (16, 13056, 4096, NK, (64, 1, 128)),
+])
+def test_plans_for_widths_between_the_fitted_ones(device, M, N, K, layout, want):
+    # the planner's rules by tile count: each plan runs at its real width and three windows of 128
+    # output columns are held to the oracle
+    A, W = _case(M, N, K, layout, 7000 + M + N // 128 + K // 128)
+    got, p = _run(A, W, layout, device)
+    if layout == KN:
+        assert (p.splitk, p.waves, p.unroll) == want, p.as_dict()
+        assert p.fused == (3 if M >= 3 else 2)
+    else:
+        assert (p.tile_n, p.splitk, p.band) == want, p.as_dict()
+    assert not np.isnan(got.astype(np.float32)).any()
+    for lo in (0, (N // 2) // 128 * 128, N - 128):
+        Wwin = W[:, lo:lo + 128] if layout == KN else W[lo:lo + 128]
+        ref, _ = oracle.gemm_f16(A.numpy(), Wwin.contiguous().numpy(), layout)
+        assert_close_f16(got[:, lo:lo + 128], ref, "columns %d.." % lo)
