@@ -100,7 +100,6 @@ __global__ __launch_bounds__(64 * NWV) void wq_m1_kernel(const uint8_t* __restri
   const uint8_t* Wt = Wq + (size_t)n0 * rowb;  // uniform; the lane's part is a 32-bit offset
   const uint32_t lane_w = lane * WB, lane_x = lane * 16;
   const half2_t ones = {static_cast<half_t>(1.f), static_cast<half_t>(1.f)};
-  const u32x4 zero = {0u, 0u, 0u, 0u};
   float acc0[MR][RN], acc1[MR][RN];
   float xsum[MR];
 #pragma unroll
@@ -110,30 +109,35 @@ __global__ __launch_bounds__(64 * NWV) void wq_m1_kernel(const uint8_t* __restri
     for (int r = 0; r < RN; ++r) acc0[m][r] = acc1[m][r] = 0.f;
   }
 
+  constexpr int kNonTemporal = 2;  // the nt bit of a buffer load's cache policy
+  const __amdgpu_buffer_rsrc_t wrs =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(Wt), 0, (int)(RN * rowb), 0x00020000);
+  __amdgpu_buffer_rsrc_t xrs[MR];
+#pragma unroll
+  for (int m = 0; m < MR; ++m)
+    xrs[m] = __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(X + (size_t)m * K), 0, K * 2, 0x00020000);
   const int nunits = K >> 3;
   const int nchunks = (nunits + 64 * UD - 1) / (64 * UD);
   for (int ch = wave; ch < nchunks; ch += NWV) {
     wreg_t wr[RN][UD];
     u32x4 xv[MR][UD];
-    bool ok[UD];
-#pragma unroll
-    for (int d = 0; d < UD; ++d) ok[d] = ch * (64 * UD) + 64 * d + lane < nunits;
+    // Buffer loads: a lane past the end of K gets zeros for x (the descriptor ends with the row), so
+    // whatever its weight load returns -- the start of the next row, or zeros past the workgroup's
+    // last row -- multiplies to zero: no predicate, no branch around any of the loads.
 #pragma unroll
     for (int r = 0; r < RN; ++r)
 #pragma unroll
       for (int d = 0; d < UD; ++d) {
-        const wreg_t none = {};
-        wr[r][d] = ok[d] ? __builtin_nontemporal_load(reinterpret_cast<const wreg_t*>(
-                               Wt + (size_t)r * rowb + (size_t)(ch * (64 * UD) + 64 * d) * WB + lane_w))
-                         : none;
+        const int off = r * (int)rowb + (ch * (64 * UD) + 64 * d) * WB + (int)lane_w;
+        if constexpr (WB == 4) wr[r][d][0] = __builtin_amdgcn_raw_buffer_load_b32(wrs, off, 0, kNonTemporal);
+        else wr[r][d] = __builtin_bit_cast(wreg_t, __builtin_amdgcn_raw_buffer_load_b64(wrs, off, 0, kNonTemporal));
       }
 #pragma unroll
     for (int m = 0; m < MR; ++m)
 #pragma unroll
       for (int d = 0; d < UD; ++d)
-        xv[m][d] = ok[d] ? load16<false>(reinterpret_cast<const uint8_t*>(X + (size_t)m * K) +
-                                         (size_t)(ch * (64 * UD) + 64 * d) * 16 + lane_x)
-                         : zero;
+        xv[m][d] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(
+                                                 xrs[m], (ch * (64 * UD) + 64 * d) * 16 + (int)lane_x, 0, 0));
     if (use_xsum) {
 #pragma unroll
       for (int m = 0; m < MR; ++m)
@@ -568,6 +572,9 @@ static int i8_waves(int K) {
 // 4096 x 14336 10.1 -> 8.1, 16384 x 16384 27.9 -> 24.5; int8 8192 x 8192 13.3 -> 12.1,
 // 4096 x 4096 5.7 -> 5.25, 28672 x 4096 20.8 -> 18.8, 4096 x 14336 12.6 -> 11.4, 16384 x 16384
 // 41.9 -> 40.6.  int8 with four units a lane (2 KB of a row per wave): 8192 x 8192 13.0.
+// Loads through buffer descriptors that end with the row (no predicate, so no branch around each of
+// the 10 .. 20 small loads of a chunk), six alternating runs each: int4 8192 x 8192 8.57 -> 8.15, 4096
+// x 4096 4.08 -> 3.98; int8 12.25 -> 12.17, 5.30 -> 5.21.
 // Two activation rows of int4 (MR = 2) against the row-load MFMA kernel: 8192 x 8192 11.4 -> 10.6,
 // 4096 x 4096 5.7 -> 5.0, 4096 x 14336 11.6 -> 10.7, 28672 x 4096 level; the second row costs 2 us at
 // 8192 x 8192 because its x traffic (64 MiB from L2) is twice the weights'; eight weight rows a
