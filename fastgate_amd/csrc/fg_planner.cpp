@@ -308,6 +308,9 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
       // workgroup id / 8 at 8192 (22.0 -> 21.8) and from 16384 on (N=4096 23.2 -> 21.6, N=8192
       // 42.5 -> 40.2, N=14336 71.5 -> 68.8)
       p->unroll = (K > 8192 || M > 2) ? 2 : 1;
+      // K = 5120 is two and a half steps of four waves: four load groups in flight make it one (inside a
+      // replayed graph, M=1: N=4096 8.96 -> 8.37 us, N=5120 10.25 -> 9.81, N=8192 14.61 -> 14.22)
+      if (K == 5120 && M <= 2) p->unroll = 4;
       items = ceil_div(K / 8, 64 * p->unroll);
       p->stagger = M <= 2 ? (K < 8192 || (K > 8192 && K < 16384)) : items <= 16;
     } else if (M <= 8 && huge) {
@@ -385,6 +388,7 @@ int make_plan(int M, int N, int K, int w_layout, int splitk, fg_plan_t* p) {
   }
   {
     p->waves = (row_tiles && !wide_tiles && p->unroll == 1 && items >= 16) ? 8 : pick_waves(items);
+    if (p->kernel == FG_KERNEL_NK_DOT2 && K == 5120 && M <= 2) p->waves = 4;  // (measured with four)
     if (wide_band_waves) {
       p->waves = wide_band_waves;
       while (p->waves > 1 && p->waves > K / 64) p->waves >>= 1;  // one 128-byte band per wave at least

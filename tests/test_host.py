@@ -191,6 +191,8 @@ def test_plan_choices_that_were_measured():
     p = nk(2, 8192, 16384)
     assert (p.unroll, p.stagger) == (2, 0)
     assert nk(1, 16384, 16384).kernel == capi.FG_KERNEL_NK_MFMA4
+    p = nk(1, 5120, 5120)
+    assert (p.kernel, p.unroll, p.waves) == (capi.FG_KERNEL_NK_DOT2, 4, 4)   # two and a half steps of four waves made one
     # [K,N]
     # sixteen column tiles or fewer: deep splits (they complete through atomics), four waves for one
     # or two rows from nine tiles on
