@@ -637,11 +637,11 @@ bool launch_w8a16(const W8A16Args& a, hipStream_t s) {
   // kernel fill the CUs evenly (us, two-row kernel / row-load kernel: N=4096 K=4096 6.0 / 7.1, K=14336
   // 13.2 / 14.7; N=11008 K=4096 10.8 / 12.5; N=12288 K=3072 9.2 / 10.9, K=8192 20.0 / 20.8; N=28672 K=4096
   // 22.0 / 24.0; N=2048 K=8192 6.1 / 6.8; N=1024 K=4096 3.7 / 4.5; but N=8192 K=8192 14.6 / 13.5, K=11008
-  // 19.0 / 16.9, K=4096 8.9 / 8.6; N=16384 K=8192 25.5 / 23.3; N=13824 K=5120 16.1 / 15.5; N=14336 K=4096
-  // 12.9 / 12.7).  Three and four rows only against narrow outputs, which leave the row-load kernel on
+  // 18.4 / 17.0, K=4096 8.6 / 8.4, but K=2048 5.6 / 6.2; N=16384 K=8192 25.5 / 23.5; level at N=13824
+  // K=5120 and N=14336 K=4096).  Three and four rows only against narrow outputs, which leave the row-load kernel on
   // half the CUs or fewer (M=4: N=1024 K=4096 4.5 / 5.3, N=2048 K=2048 4.3 / 5.6, K=8192 7.8 / 8.1;
   // N=4096 K=4096 7.6 / 6.6 and N=8192 K=8192 23.2 / 13.7 the other way).
-  const bool even_tiles = a.N % 8192 == 0 || (a.N >= 13312 && a.N <= 14336);
+  const bool even_tiles = a.N % 8192 == 0 && a.K >= 4096;
   if (a.M == 1) {
     launch_wq_m1<8, 1>(a, s);
   } else if (a.M == 2 && !even_tiles) {
