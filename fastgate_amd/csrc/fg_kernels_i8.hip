@@ -298,7 +298,7 @@ __global__ __launch_bounds__(256) void dequant_i32_f16_kernel(const int32_t* __r
 // on the matrix pipe, and the VALU only converts.  16-column tiles, 8 waves interleaving over K.
 // XROWS = activation rows staged: 4, 8 or 16.
 // ---------------------------------------------------------------------------------------
-template <int XROWS, int NW, int BW, int CB>
+template <int XROWS, int NW, int BW, int CB, int DEPTH = 2>
 __global__ __launch_bounds__(64 * NW) void w8a16_r_kernel(const int8_t* __restrict__ Wq,
                                                           const half_t* __restrict__ X,
                                                           const half_t* __restrict__ scale,
@@ -389,7 +389,9 @@ __global__ __launch_bounds__(64 * NW) void w8a16_r_kernel(const int8_t* __restri
     wave_lds_sync();
   };
 
-  u32x4 w0[WI], w1[WI], x0[XI], x1[XI];
+  // DEPTH bands of a wave in flight or in use: the loads of band t + DEPTH - 1 go out before band t is
+  // multiplied
+  u32x4 wbuf[DEPTH][WI], xbuf[DEPTH][XI];
   const int nsteps = (nbands + nw - 1) / nw;
   int step = stagger_start(nsteps, 0);
   auto next_band = [&]() {
@@ -397,13 +399,17 @@ __global__ __launch_bounds__(64 * NW) void w8a16_r_kernel(const int8_t* __restri
     step = step + 1 == nsteps ? 0 : step + 1;
     return band;
   };
-  load_band(next_band(), w0, x0);
-  for (int it = 0; it < nsteps; it += 2) {
-    if (it + 1 < nsteps) load_band(next_band(), w1, x1);
-    multiply(w0, x0);
-    if (it + 1 >= nsteps) break;
-    if (it + 2 < nsteps) load_band(next_band(), w0, x0);
-    multiply(w1, x1);
+#pragma unroll
+  for (int d = 0; d < DEPTH - 1; ++d)
+    if (d < nsteps) load_band(next_band(), wbuf[d], xbuf[d]);
+  for (int it = 0; it < nsteps; it += DEPTH) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+      if (it + d >= nsteps) break;
+      if (it + d + DEPTH - 1 < nsteps)
+        load_band(next_band(), wbuf[(d + DEPTH - 1) % DEPTH], xbuf[(d + DEPTH - 1) % DEPTH]);
+      multiply(wbuf[d], xbuf[d]);
+    }
   }
 
   // acc[b][r] = D[m = 4g + r][column 16b + j] (xacc: sum of x of row m in every column); the waves
@@ -615,7 +621,7 @@ bool launch_w8a16(const W8A16Args& a, hipStream_t s) {
   //  * two workgroups (16 waves) on every CU, 448..512 tiles or a multiple of 512: K = N = 16384 M=8
   //    44.8 / 49.3, K=4096 N=16384 14.9 / 17.3, K=4096 N=14336 M=8 13.7 / 14.5 -- but not with rows
   //    8 KB apart: K=8192 N=16384 M=8 27.6 / 25.2;
-  //  * one workgroup on every CU (N = 8192): long rows or 15..16 activation rows only, K=16384 M=8
+  //  * one workgroup on every CU (N = 8192): long rows or 12..16 activation rows only (15..16 before three bands were in flight), K=16384 M=8
   //    25.4 / 27.3, K=28672 M=14 47.8 / 55.4, K=4096 M=16 10.5 / 11.1, against K=8192 M=8 16.9 /
   //    14.9, K=28672 M=4 40.0 / 38.7, K=2048 M=16 7.7 / 7.1;
   //  * 13..16 rows from 160 tiles on: N=5120 K=11008 M=16 19.5 / 23.0, N=14336 K=14336 44.5 / 55.1.
@@ -623,7 +629,7 @@ bool launch_w8a16(const W8A16Args& a, hipStream_t s) {
   const bool two_per_cu = aligned && ((t32 >= 448 && t32 <= 512) || (t32 >= 512 && t32 % 512 == 0)) &&
                           (a.K != 8192 || a.M > 8);
   const bool one_per_cu = aligned && t32 == 256 &&
-                          ((a.M >= 15 && a.K >= 4096) || (a.K >= 16384 && (a.M >= 5 || a.K < 24576)));
+                          ((a.M >= 12 && a.K >= 4096) || (a.K >= 16384 && (a.M >= 5 || a.K < 24576)));
   const bool many_rows = aligned && a.M >= 13 && t32 >= 160 && t32 != 256;
   const bool wide = two_per_cu || one_per_cu || many_rows;
   // 16-column tiles take 128-byte bands (smaller strips, more steps in flight): M=8, 128- / 256-byte
@@ -659,8 +665,16 @@ bool launch_w8a16(const W8A16Args& a, hipStream_t s) {
     else if (bw256) FG_W8A16_R(8, 256, 1);
     else FG_W8A16_R(8, 128, 1);
   } else if (a.M <= 16) {
-    // 16-row activation strip on 128-byte bands only (the 256-byte form would need 100 KB of LDS)
-    if (wide) FG_W8A16_R(16, 128, 2);
+    // 16-row activation strip on 128-byte bands only (the 256-byte form would need 100 KB of LDS).
+    // 32-column tiles with three bands of a wave in flight instead of two (us): N = K = 8192 M=16 17.3 /
+    // 18.2, K=16384 25.9 / 27.5; N=16384 K=8192 31.3 / 32.7; N=14336 K=4096 17.2 / 18.1 -- with eight rows
+    // level or behind (N = K = 8192 15.3 / 14.7 against 16-column tiles, N=14336 K=4096 15.2 / 13.6), and
+    // 16-column tiles lose with any deeper pipeline (M=16 19.9 with three, 21.4 with four).  With three in
+    // flight the one-a-CU form at N = 8192 pays from 12 rows on (K=4096 M=12 9.8 / 10.6, K=8192 M=13 17.0 /
+    // 17.5; M=9 level).
+    if (wide)
+      hipLaunchKernelGGL((w8a16_r_kernel<16, 8, 128, 2, 3>), dim3(a.N / 32), dim3(512), 0, s, Wq, X, sc,
+                         a.scalar_scale, a.zero_point, Y, a.M, a.N, a.K);
     else FG_W8A16_R(16, 128, 1);
   } else {
     return false;
